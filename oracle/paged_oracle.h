@@ -1,0 +1,187 @@
+/*
+ * CPU oracle for the paged-KV attention path.  TEST INFRASTRUCTURE ONLY:
+ * nothing in the shipped library links or loads this file; it is the checker
+ * the GPU kernels are compared with, and the CPU baseline that is timed
+ * beside them.
+ *
+ * Every function restates, in plain C, one piece of the reference
+ * (G-Krishna-chandra/MLcompiler); the citation next to each prototype names
+ * the reference file and lines it follows.
+ *
+ * Pinning status (what each function has been checked against):
+ *   oracle_fp16_to_float, oracle_float_to_fp16_ref
+ *       - all 65536 halves / a float sweep against the reference's own inline
+ *         functions compiled from compiler/runtime/float_convert.hpp
+ *         (oracle/_ref), and against numpy's IEEE binary16.
+ *   oracle_paged_attention_executor
+ *       - bit-for-bit against the reference's RunAttentionCPU compiled from
+ *         its own sources (oracle/_ref), on gathered-contiguous copies of the
+ *         same paged cache; known answers tests/test_runtime.cpp:1692-1705,
+ *         compiler/main.cpp:4026-4031; closed forms (S=1, equal keys,
+ *         constant V, page-permutation invariance) and a float64 brute force.
+ *   oracle_paged_attention_flashref
+ *       - same known answers and closed forms; agreement with the executor
+ *         ordering to float rounding; float64 brute force.
+ *   oracle_scatter_*, oracle_gather_*
+ *       - closed-form index pattern of tests/test_paged_kv.cpp:219-267 and
+ *         scatter->gather identity; untouched-bytes invariant.
+ *   oracle_pool_*, oracle_req_*
+ *       - the allocator sequences asserted in tests/test_paged_kv.cpp:34-207.
+ *   oracle_paged_attention_prefill
+ *       - PARITY UNPINNED against the reference: the reference has no
+ *         multi-query paged attention.  It is defined row-wise through
+ *         oracle_paged_attention_executor (a query at absolute position p
+ *         sees kv positions <= p, metal_runtime.mm:2286) and checked against
+ *         a float64 brute force only.
+ */
+#ifndef PAGED_ORACLE_H
+#define PAGED_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* compiler/runtime/float_convert.hpp:14-48 -- IEEE binary16 -> binary32. */
+float oracle_fp16_to_float(uint16_t h);
+
+/* compiler/runtime/float_convert.hpp:57-76 -- the reference's own
+ * binary32 -> binary16: round-half-up on the magnitude, NaN becomes Inf,
+ * |x| < 2^-25 flushes to signed zero.  NOT round-to-nearest-even. */
+uint16_t oracle_float_to_fp16_ref(float value);
+
+/* IEEE round-to-nearest-even binary32 -> binary16 (what the GPU's convert
+ * instruction and numpy do); used to build inputs shared by both sides. */
+uint16_t oracle_float_to_fp16_rne(float value);
+
+/* Bulk forms of the three conversions above (float_convert.hpp:80-104 are the
+ * reference's bulk loops: element-wise calls of the scalar functions). */
+void oracle_fp16_to_float_n(const uint16_t* src, float* dst, size_t n);
+void oracle_float_to_fp16_ref_n(const float* src, uint16_t* dst, size_t n);
+void oracle_float_to_fp16_rne_n(const float* src, uint16_t* dst, size_t n);
+
+/* compiler/runtime/metal_runtime.mm:405-424 (kernel) and :7231-7294 (host
+ * argument checks).  src is [batch][n_kv_heads][head_dim] halves; row r goes
+ * to page page_ids[r], slot slots_in_page[r].  Returns 1 on success, 0 on the
+ * argument errors the reference rejects. */
+int oracle_scatter_kv_paged_batched_f16(uint16_t* page_storage,
+                                        const uint32_t* page_ids,
+                                        const uint32_t* slots_in_page,
+                                        size_t page_size_tokens,
+                                        size_t n_kv_heads,
+                                        size_t head_dim,
+                                        size_t batch,
+                                        const uint16_t* src);
+
+/* compiler/runtime/metal_runtime.mm:468-512 (kernels), :7828-7906 (host).
+ * src is [n_kv_heads][tokens][head_dim]; token t lands at absolute slot
+ * start_slot + t of the request's page table.  dtype_bytes is 2 or 4. */
+int oracle_scatter_kv_paged(void* page_storage,
+                            const uint32_t* page_table, size_t n_page_table,
+                            size_t page_size_tokens, size_t n_kv_heads,
+                            size_t head_dim, size_t tokens, size_t start_slot,
+                            const void* src, size_t dtype_bytes);
+
+/* compiler/runtime/metal_runtime.mm:328-370 (kernels), :7647-7721 (host).
+ * dst is [n_kv_heads][num_tokens][head_dim]. */
+int oracle_gather_kv_pages(const void* page_storage,
+                           const uint32_t* page_table, size_t n_page_table,
+                           size_t page_size_tokens, size_t n_kv_heads,
+                           size_t head_dim, size_t num_tokens,
+                           void* dst, size_t dtype_bytes);
+
+/* The executor-CPU attention, compiler/runtime/attention_cpu.cpp:437-470
+ * (per head: left-to-right dot over every cached row :99-105, softmax that
+ * subtracts the max, exponentiates and divides each weight by the sum :21-33,
+ * then V axpy :166-170), reading rows through the page layout of
+ * compiler/runtime/metal_runtime.mm:2266-2276 and applying that kernel's
+ * causal rule :2286 and empty-sequence rule :2254-2257,2333.  GQA map
+ * kv = head*kv_heads/heads (attention_cpu.cpp:443).  fp32 throughout.
+ * n_threads > 1 spreads (request, head) pairs over OpenMP threads; the
+ * arithmetic of each pair is unchanged.  Returns 1, or 0 on the argument
+ * errors of metal_runtime.mm:7742-7750. */
+int oracle_paged_attention_executor(const float* q,
+                                    const uint16_t* k_pages,
+                                    const uint16_t* v_pages,
+                                    float* out,
+                                    const uint32_t* page_tables_flat, size_t n_page_tables_flat,
+                                    const uint32_t* page_table_offsets,
+                                    const uint32_t* seq_lens,
+                                    const uint32_t* q_positions,
+                                    size_t batch, size_t num_heads, size_t kv_heads,
+                                    size_t head_dim, size_t page_size_tokens,
+                                    int apply_causal, int n_threads);
+
+/* The kernel's in-test CPU twin, tests/test_paged_flash.cpp:17-91: same
+ * semantics, but weights stay un-normalised and the accumulated output is
+ * multiplied by 1/sum at the end. */
+int oracle_paged_attention_flashref(const float* q,
+                                    const uint16_t* k_pages,
+                                    const uint16_t* v_pages,
+                                    float* out,
+                                    const uint32_t* page_tables_flat, size_t n_page_tables_flat,
+                                    const uint32_t* page_table_offsets,
+                                    const uint32_t* seq_lens,
+                                    const uint32_t* q_positions,
+                                    size_t batch, size_t num_heads, size_t kv_heads,
+                                    size_t head_dim, size_t page_size_tokens,
+                                    int apply_causal);
+
+/* Chunked prefill over paged KV.  q is fp16 [batch][chunk][num_heads][head_dim];
+ * request r's chunk row i sits at absolute position q_start[r] + i and sees
+ * kv positions <= that (metal_runtime.mm:2286 applied per row; the reference
+ * reaches the same result by looping its decode path once per token,
+ * compiler/runtime/batched_executor.cpp:454-466).  out is fp32, same shape. */
+int oracle_paged_attention_prefill(const uint16_t* q_f16,
+                                   const uint16_t* k_pages,
+                                   const uint16_t* v_pages,
+                                   float* out,
+                                   const uint32_t* page_tables_flat, size_t n_page_tables_flat,
+                                   const uint32_t* page_table_offsets,
+                                   const uint32_t* seq_lens,
+                                   const uint32_t* q_start,
+                                   size_t batch, size_t chunk, size_t num_heads,
+                                   size_t kv_heads, size_t head_dim,
+                                   size_t page_size_tokens, int n_threads);
+
+/* compiler/runtime/parity_harness.cpp:214-255 -- max|a-b|, mean|a-b|, rms and
+ * cosine, all accumulated in double.  cosine is NaN when either norm is 0. */
+void oracle_metrics(const float* a, const float* b, size_t n,
+                    double* max_abs, double* mean_abs, double* rms, double* cosine);
+
+/* tests/test_paged_flash.cpp:93-102 -- cosine that returns 0 for a zero norm. */
+double oracle_cosine(const float* a, const float* b, size_t n);
+
+/* compiler/runtime/paged_kv.cpp:10-42 -- LIFO free list of page ids; a fresh
+ * pool hands out 0,1,2,...  The caller owns `pool` (oracle_pool_free). */
+typedef struct oracle_page_pool oracle_page_pool;
+oracle_page_pool* oracle_pool_new(uint32_t capacity);
+void oracle_pool_free(oracle_page_pool* pool);
+int oracle_pool_allocate(oracle_page_pool* pool, uint32_t* id_out);          /* 0 = exhausted */
+int oracle_pool_allocate_n(oracle_page_pool* pool, size_t n, uint32_t* out); /* all or nothing */
+void oracle_pool_release(oracle_page_pool* pool, uint32_t page_id);
+size_t oracle_pool_in_use(const oracle_page_pool* pool);
+size_t oracle_pool_free_count(const oracle_page_pool* pool);
+
+/* compiler/runtime/paged_kv.hpp:65-97, paged_kv.cpp:44-81 -- one request's
+ * page chain.  page_table is caller storage of page_table_cap entries. */
+typedef struct {
+    uint32_t page_size_tokens;
+    uint32_t* page_table;
+    size_t page_table_cap;
+    size_t n_pages;
+    uint32_t tokens_in_last_page;
+} oracle_request_kv;
+size_t oracle_req_total_tokens(const oracle_request_kv* st);
+int oracle_req_reserve(oracle_request_kv* st, oracle_page_pool* pool, size_t target_tokens);
+int oracle_req_extend_one_token(oracle_request_kv* st, oracle_page_pool* pool,
+                                uint32_t* page_id, uint32_t* slot);
+int oracle_req_locate(const oracle_request_kv* st, size_t pos, uint32_t* page_id, uint32_t* slot);
+void oracle_req_release_all(oracle_request_kv* st, oracle_page_pool* pool);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
