@@ -1,0 +1,169 @@
+/*
+ * mlc_hip.h -- C ABI of the MI355X (gfx950) implementation of MLcompiler's
+ * paged-KV attention hot path.
+ *
+ * Every entry point is what a HIP-backed mlc::runtime::MetalExecutor method
+ * forwards to; the comment above each one names the reference method (or
+ * kernel) it replaces.  All pointers named *_buf / page_storage / q / o are
+ * DEVICE pointers obtained from mlc_hip_alloc / mlc_hip_cached (or any other
+ * hipMalloc'ed memory of the current device); pointers to uint32_t metadata
+ * are HOST pointers, borrowed for the duration of the call only (they are
+ * copied before the call returns), exactly like the std::vector arguments of
+ * the reference.
+ *
+ * Return convention mirrors the reference's `bool`: 1 = success, 0 = failure
+ * (GPU unavailable, bad arguments, no open pass for an encode variant, or a
+ * HIP error).  mlc_hip_last_error() describes the most recent failure of the
+ * calling thread.  Nothing here throws.
+ *
+ * Threading: single-threaded by contract, like the reference
+ * (compiler/runtime/paged_kv.hpp:25-27).  All work is ordered on one HIP
+ * stream; "encode" variants enqueue and return, "run"/sync variants also wait.
+ */
+#ifndef MLC_HIP_H
+#define MLC_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* MetalExecutor::isAvailable  (compiler/runtime/metal_runtime.hpp:27).
+ * 1 when a gfx950 device is usable; initialises the library on first call. */
+int mlc_hip_available(void);
+
+/* Text of the last failure on this thread ("" if none). Never NULL. */
+const char* mlc_hip_last_error(void);
+
+/* ---- device buffers -------------------------------------------------------
+ * MetalExecutor::allocateScratchBuffer / releaseScratchBuffer
+ * (metal_runtime.hpp:693-694, metal_runtime.mm:8248-8271).  Caller owns. */
+void* mlc_hip_alloc(size_t bytes);
+void  mlc_hip_free(void* buffer);
+
+/* MetalExecutor::getOrAllocCachedBuffer (metal_runtime.hpp:703,
+ * metal_runtime.mm:8218-8246): name-keyed, library-owned, grow-only; a larger
+ * request reallocates and invalidates the pointer handed out before. */
+void* mlc_hip_cached(const char* name, size_t bytes);
+
+/* MetalExecutor::uploadToBuffer / downloadFromBuffer (metal_runtime.hpp:695-696,
+ * metal_runtime.mm:8273-8297).  Ordered after all work already enqueued on the
+ * library's stream; both return when the copy is complete. */
+int mlc_hip_upload(void* buffer, const void* src, size_t bytes, size_t dst_offset);
+int mlc_hip_download(const void* buffer, void* dst, size_t bytes, size_t src_offset);
+
+/* Fill `bytes` bytes with zero on the stream (PagedKVStorage::initialize
+ * zero-fills its pools through uploadToBuffer, paged_kv.cpp:113-117; this is
+ * the same result without the host staging copy). */
+int mlc_hip_zero(void* buffer, size_t bytes);
+
+/* ---- forward pass ("command buffer") --------------------------------------
+ * MetalExecutor::beginForwardPassCB / flushForwardPassCB / hasForwardPassCB
+ * (metal_runtime.hpp:181-183, metal_runtime.mm:6000-6064).  begin is
+ * idempotent; flush waits for everything enqueued since begin and closes the
+ * pass (returns 0 if a kernel failed). */
+int mlc_hip_begin(void);
+int mlc_hip_flush(void);
+int mlc_hip_has_open_pass(void);
+
+/* ---- the hot path ----------------------------------------------------------
+ * Batched paged flash-attention decode: one query token per request.
+ *   sync = 0: MetalExecutor::encodePagedFlashAttention
+ *             (metal_runtime.hpp:510-523, metal_runtime.mm:7074-7166) --
+ *             requires an open pass, enqueues, no argument validation beyond
+ *             what keeps the kernel in bounds of the metadata.
+ *   sync = 1: MetalExecutor::runPagedFlashAttention
+ *             (metal_runtime.hpp:645-658, metal_runtime.mm:7727-7826) --
+ *             validates like :7742-7750, runs, waits.
+ * Kernel semantics: MSL paged_flash_attention, metal_runtime.mm:2216-2335.
+ *   q  fp32 [batch][num_heads][head_dim]           o  fp32, same shape
+ *   k_pages, v_pages  fp16 [pool pages][page_size_tokens][kv_heads][head_dim]
+ *   page_tables_flat  all requests' page ids, concatenated (n_page_tables_flat)
+ *   page_table_offsets [batch+1]; seq_lens [batch]; q_positions [batch]
+ * Softmax scale is 1/sqrt(head_dim), derived inside as the reference does
+ * (metal_runtime.mm:7133).  Query head h reads KV head h*kv_heads/num_heads. */
+int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_pages, void* o,
+                              const uint32_t* page_tables_flat, size_t n_page_tables_flat,
+                              const uint32_t* page_table_offsets,
+                              const uint32_t* seq_lens,
+                              const uint32_t* q_positions,
+                              size_t batch, size_t num_heads, size_t kv_heads,
+                              size_t head_dim, size_t page_size_tokens,
+                              int apply_causal, int sync);
+
+/* Batched paged KV write: one new fp16 K (or V) row per request.
+ *   sync = 0: MetalExecutor::encodeScatterKVPagedBatched
+ *             (metal_runtime.hpp:526-533, metal_runtime.mm:7168-7225)
+ *   sync = 1: MetalExecutor::scatterKVPagedBatched
+ *             (metal_runtime.hpp:680-687, metal_runtime.mm:7231-7294)
+ * Kernel: MSL scatter_kv_paged_batched_f16, metal_runtime.mm:405-424.
+ *   src  fp16 [batch][n_kv_heads][head_dim]; row r -> page page_ids[r],
+ *   slot slots_in_page[r] of page_storage. */
+int mlc_hip_scatter_kv_paged_batched_f16(void* page_storage,
+                                         const uint32_t* page_ids,
+                                         const uint32_t* slots_in_page,
+                                         size_t page_size_tokens, size_t n_kv_heads,
+                                         size_t head_dim, size_t batch,
+                                         const void* src, int sync);
+
+/* ---- the callers' data formats either side of the path --------------------
+ * MetalExecutor::scatterKVPaged (metal_runtime.hpp:666-674,
+ * metal_runtime.mm:7828-7906; kernels :468-512): multi-token write for one
+ * request, src [n_kv_heads][tokens][head_dim], dtype_bytes 2 or 4.  Waits. */
+int mlc_hip_scatter_kv_paged(void* page_storage,
+                             const uint32_t* page_table, size_t n_page_table,
+                             size_t page_size_tokens, size_t n_kv_heads, size_t head_dim,
+                             size_t tokens, size_t start_slot,
+                             const void* src, size_t dtype_bytes);
+
+/* MetalExecutor::gatherKVPages (metal_runtime.hpp:619-626,
+ * metal_runtime.mm:7647-7721; kernels :328-370): pages -> contiguous
+ * [n_kv_heads][num_tokens][head_dim].  Waits. */
+int mlc_hip_gather_kv_pages(const void* page_storage,
+                            const uint32_t* page_table, size_t n_page_table,
+                            size_t page_size_tokens, size_t n_kv_heads, size_t head_dim,
+                            size_t num_tokens, void* dst, size_t dtype_bytes);
+
+/* Chunked prefill over paged KV (MFMA path).  No counterpart in the reference,
+ * which prefills by looping the decode path once per prompt token
+ * (compiler/runtime/batched_executor.cpp:454-466); semantics are the decode
+ * kernel's causal rule (metal_runtime.mm:2286) applied per query row:
+ *   q  fp16 [batch][chunk][num_heads][head_dim]; row i of request r sits at
+ *      absolute position q_start[r] + i and attends kv positions <= that and
+ *      < seq_lens[r].   o  fp32, same shape as q.
+ * sync as above (0 needs an open pass). */
+int mlc_hip_paged_attn_prefill(const void* q_f16, const void* k_pages, const void* v_pages,
+                               void* o,
+                               const uint32_t* page_tables_flat, size_t n_page_tables_flat,
+                               const uint32_t* page_table_offsets,
+                               const uint32_t* seq_lens,
+                               const uint32_t* q_start,
+                               size_t batch, size_t chunk, size_t num_heads, size_t kv_heads,
+                               size_t head_dim, size_t page_size_tokens, int sync);
+
+/* ---- measurement helpers (no reference counterpart) ------------------------
+ * The library's stream as a hipStream_t, for callers that need to order their
+ * own work or events with it. */
+void* mlc_hip_stream(void);
+
+/* hipEvent pair on the library's stream: start records, stop records, waits
+ * and returns the elapsed milliseconds (negative on error). */
+int   mlc_hip_timer_start(void);
+float mlc_hip_timer_stop(void);
+
+/* Number of kernels the last mlc_hip_paged_attn_decode call launched and the
+ * number of split-K work items it planned (for benchmarks and tests). */
+int mlc_hip_last_decode_launches(void);
+int mlc_hip_last_decode_work_items(void);
+
+/* Tunables: "decode_target_items" (split-K work items aimed for per launch),
+ * "decode_force_generic" (1 = always use the shape-agnostic kernel).
+ * Returns 0 for an unknown name. */
+int mlc_hip_set_option(const char* name, long value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MLC_HIP_H */

@@ -1,0 +1,144 @@
+// HipExecutor: vector-taking C++ methods forwarded to the C ABI.  The length
+// checks the reference makes on its std::vector arguments
+// (compiler/runtime/metal_runtime.mm:7241-7243, 7747-7749) live here, because
+// the C ABI only sees pointers.
+#include "hip_executor.hpp"
+
+#include "../../include/mlc_hip.h"
+
+namespace mlc_amd {
+
+namespace {
+const uint32_t kNoIds[1] = {0};
+const uint32_t* data_or_dummy(const std::vector<uint32_t>& v) {
+    return v.empty() ? kNoIds : v.data();
+}
+}  // namespace
+
+HipExecutor& HipExecutor::Instance() {
+    static HipExecutor inst;
+    return inst;
+}
+
+bool HipExecutor::isAvailable() const { return mlc_hip_available() != 0; }
+const char* HipExecutor::lastError() const { return mlc_hip_last_error(); }
+
+bool HipExecutor::beginForwardPassCB() const { return mlc_hip_begin() != 0; }
+bool HipExecutor::flushForwardPassCB() const { return mlc_hip_flush() != 0; }
+bool HipExecutor::hasForwardPassCB() const { return mlc_hip_has_open_pass() != 0; }
+
+bool HipExecutor::encodePagedFlashAttention(void* q_buf, void* k_pages_buf, void* v_pages_buf,
+                                            void* o_buf,
+                                            const std::vector<uint32_t>& page_tables_flat,
+                                            const std::vector<uint32_t>& page_table_offsets,
+                                            const std::vector<uint32_t>& seq_lens,
+                                            const std::vector<uint32_t>& q_positions,
+                                            size_t batch, size_t num_heads, size_t kv_heads,
+                                            size_t head_dim, size_t page_size_tokens,
+                                            bool apply_causal) const {
+    // The reference's encode variant trusts its caller; vectors that are too short
+    // would be read out of bounds here, so they are refused instead.
+    if (page_table_offsets.size() < batch + 1 || seq_lens.size() < batch ||
+        q_positions.size() < batch)
+        return false;
+    return mlc_hip_paged_attn_decode(q_buf, k_pages_buf, v_pages_buf, o_buf,
+                                     data_or_dummy(page_tables_flat), page_tables_flat.size(),
+                                     page_table_offsets.data(), seq_lens.data(),
+                                     q_positions.data(), batch, num_heads, kv_heads, head_dim,
+                                     page_size_tokens, apply_causal ? 1 : 0, /*sync=*/0) != 0;
+}
+
+bool HipExecutor::runPagedFlashAttention(void* q_buffer, void* k_pages_buffer,
+                                         void* v_pages_buffer, void* o_buffer,
+                                         const std::vector<uint32_t>& page_tables_flat,
+                                         const std::vector<uint32_t>& page_table_offsets,
+                                         const std::vector<uint32_t>& seq_lens,
+                                         const std::vector<uint32_t>& q_positions,
+                                         size_t batch, size_t num_heads, size_t kv_heads,
+                                         size_t head_dim, size_t page_size_tokens,
+                                         bool apply_causal) const {
+    if (page_table_offsets.size() != batch + 1) return false;                 // :7747
+    if (seq_lens.size() != batch || q_positions.size() != batch) return false;  // :7748
+    return mlc_hip_paged_attn_decode(q_buffer, k_pages_buffer, v_pages_buffer, o_buffer,
+                                     data_or_dummy(page_tables_flat), page_tables_flat.size(),
+                                     page_table_offsets.data(), seq_lens.data(),
+                                     q_positions.data(), batch, num_heads, kv_heads, head_dim,
+                                     page_size_tokens, apply_causal ? 1 : 0, /*sync=*/1) != 0;
+}
+
+bool HipExecutor::encodeScatterKVPagedBatched(void* page_storage_buffer,
+                                              const std::vector<uint32_t>& page_ids,
+                                              const std::vector<uint32_t>& slots_in_page,
+                                              size_t page_size_tokens, size_t n_kv_heads,
+                                              size_t head_dim, size_t batch,
+                                              const void* src_buffer) const {
+    if (page_ids.size() < batch || slots_in_page.size() < batch) return false;
+    return mlc_hip_scatter_kv_paged_batched_f16(page_storage_buffer, page_ids.data(),
+                                                slots_in_page.data(), page_size_tokens,
+                                                n_kv_heads, head_dim, batch, src_buffer,
+                                                /*sync=*/0) != 0;
+}
+
+bool HipExecutor::scatterKVPagedBatched(void* page_storage_buffer,
+                                        const std::vector<uint32_t>& page_ids,
+                                        const std::vector<uint32_t>& slots_in_page,
+                                        size_t page_size_tokens, size_t n_kv_heads,
+                                        size_t head_dim, size_t batch,
+                                        const void* src_buffer) const {
+    if (page_ids.size() != batch || slots_in_page.size() != batch) return false;  // :7243
+    return mlc_hip_scatter_kv_paged_batched_f16(page_storage_buffer, page_ids.data(),
+                                                slots_in_page.data(), page_size_tokens,
+                                                n_kv_heads, head_dim, batch, src_buffer,
+                                                /*sync=*/1) != 0;
+}
+
+bool HipExecutor::scatterKVPaged(void* page_storage_buffer, const std::vector<uint32_t>& page_table,
+                                 size_t page_size_tokens, size_t n_kv_heads, size_t head_dim,
+                                 size_t tokens, size_t start_slot, const void* src_buffer,
+                                 size_t dtype_bytes) const {
+    return mlc_hip_scatter_kv_paged(page_storage_buffer, data_or_dummy(page_table),
+                                    page_table.size(), page_size_tokens, n_kv_heads, head_dim,
+                                    tokens, start_slot, src_buffer, dtype_bytes) != 0;
+}
+
+bool HipExecutor::gatherKVPages(void* page_storage_buffer, const std::vector<uint32_t>& page_table,
+                                size_t page_size_tokens, size_t n_kv_heads, size_t head_dim,
+                                size_t num_tokens, void* dst_buffer, size_t dtype_bytes) const {
+    return mlc_hip_gather_kv_pages(page_storage_buffer, data_or_dummy(page_table),
+                                   page_table.size(), page_size_tokens, n_kv_heads, head_dim,
+                                   num_tokens, dst_buffer, dtype_bytes) != 0;
+}
+
+bool HipExecutor::runPagedPrefillAttention(void* q_f16_buffer, void* k_pages_buffer,
+                                           void* v_pages_buffer, void* o_buffer,
+                                           const std::vector<uint32_t>& page_tables_flat,
+                                           const std::vector<uint32_t>& page_table_offsets,
+                                           const std::vector<uint32_t>& seq_lens,
+                                           const std::vector<uint32_t>& q_start,
+                                           size_t batch, size_t chunk, size_t num_heads,
+                                           size_t kv_heads, size_t head_dim,
+                                           size_t page_size_tokens) const {
+    if (page_table_offsets.size() != batch + 1) return false;
+    if (seq_lens.size() != batch || q_start.size() != batch) return false;
+    return mlc_hip_paged_attn_prefill(q_f16_buffer, k_pages_buffer, v_pages_buffer, o_buffer,
+                                      data_or_dummy(page_tables_flat), page_tables_flat.size(),
+                                      page_table_offsets.data(), seq_lens.data(), q_start.data(),
+                                      batch, chunk, num_heads, kv_heads, head_dim,
+                                      page_size_tokens, /*sync=*/1) != 0;
+}
+
+void* HipExecutor::allocateScratchBuffer(size_t bytes) const { return mlc_hip_alloc(bytes); }
+void HipExecutor::releaseScratchBuffer(void* buffer) const { mlc_hip_free(buffer); }
+void HipExecutor::uploadToBuffer(void* buffer, const void* src, size_t bytes,
+                                 size_t dst_offset) const {
+    (void)mlc_hip_upload(buffer, src, bytes, dst_offset);
+}
+void HipExecutor::downloadFromBuffer(const void* buffer, void* dst, size_t bytes,
+                                     size_t src_offset) const {
+    (void)mlc_hip_download(buffer, dst, bytes, src_offset);
+}
+void* HipExecutor::getOrAllocCachedBuffer(const char* name, size_t bytes) const {
+    return mlc_hip_cached(name, bytes);
+}
+
+}  // namespace mlc_amd

@@ -1,0 +1,791 @@
+// C ABI (include/mlc_hip.h) of the MI355X paged-attention hot path: device
+// buffers, the single in-order stream that stands in for the reference's
+// command buffer, the host-side split-K planner, and the kernel launches.
+//
+// Host-side behaviour follows the reference's MetalExecutor entry points
+// (compiler/runtime/metal_runtime.mm): see the citation at each function.
+#include "../../include/mlc_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "paged_copy_kernels.h"
+#include "paged_decode_kernels.h"
+#include "paged_prefill_kernels.h"
+
+namespace {
+
+using namespace mlc_hip;
+
+thread_local std::string g_err;
+
+int fail(const std::string& msg) {
+    g_err = msg;
+    return 0;
+}
+
+#define HIP_OK(expr)                                                                  \
+    do {                                                                              \
+        hipError_t e_ = (expr);                                                       \
+        if (e_ != hipSuccess)                                                         \
+            return fail(std::string(#expr) + ": " + hipGetErrorString(e_));           \
+    } while (0)
+
+// A host-pinned + device pair used to hand small metadata to kernels with one
+// stream-ordered copy.  `done` is recorded after the kernel that reads the
+// device copy, so waiting on it makes both halves safe to overwrite or grow.
+struct MetaSlot {
+    void* host = nullptr;
+    void* dev = nullptr;
+    size_t cap = 0;
+    hipEvent_t done = nullptr;
+    bool pending = false;
+};
+
+struct DecodePlan {
+    bool valid = false;
+    // key
+    std::vector<uint32_t> pt_flat, pt_off, seq_lens, q_pos;
+    size_t B = 0, H = 0, Hkv = 0, D = 0, P = 0;
+    int causal = 0;
+    long target_items = 0, force_generic = 0;
+    // result
+    bool fast = false;
+    int hpw = 0;
+    uint32_t n_items = 0, n_merge = 0, n_part = 0;
+    size_t off_items = 0, off_merge = 0, off_ptoff = 0, off_limits = 0;  // byte offsets in blob
+    int slot = -1;
+};
+
+struct Ctx {
+    bool inited = false;
+    bool available = false;
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    bool pass_open = false;
+    std::unordered_map<std::string, std::pair<void*, size_t>> cached;
+    std::unordered_map<const void*, size_t> allocs;  // base pointer -> bytes (ours only)
+    MetaSlot ring[8];
+    int ring_next = 0;
+    MetaSlot plan_slots[4];
+    int plan_next = 0;
+    DecodePlan plan;
+    float* part_o = nullptr;
+    float2* part_ml = nullptr;
+    size_t part_o_cap = 0, part_ml_cap = 0;  // in elements
+    long opt_target_items = 0;               // 0 = automatic
+    long opt_force_generic = 0;
+    int last_launches = 0;
+    int last_items = 0;
+    int n_cu = 256;
+};
+
+Ctx g;
+
+bool init_once() {
+    if (g.inited) return g.available;
+    g.inited = true;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
+        g_err = "no HIP device";
+        return false;
+    }
+    if (hipGetDevice(&g.device) != hipSuccess) return false;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, g.device) != hipSuccess) return false;
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        g_err = std::string("device is ") + prop.gcnArchName + ", library is built for gfx950";
+        return false;
+    }
+    g.n_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    if (hipStreamCreateWithFlags(&g.stream, hipStreamNonBlocking) != hipSuccess) return false;
+    if (hipEventCreate(&g.ev0) != hipSuccess || hipEventCreate(&g.ev1) != hipSuccess) return false;
+    g.available = true;
+    return true;
+}
+
+int slot_reserve(MetaSlot& s, size_t bytes) {
+    if (s.pending) {
+        HIP_OK(hipEventSynchronize(s.done));
+        s.pending = false;
+    }
+    if (!s.done) HIP_OK(hipEventCreateWithFlags(&s.done, hipEventDisableTiming));
+    if (bytes > s.cap) {
+        size_t cap = std::max<size_t>(4096, bytes * 2);
+        if (s.host) HIP_OK(hipHostFree(s.host));
+        if (s.dev) HIP_OK(hipFree(s.dev));
+        s.host = s.dev = nullptr;
+        s.cap = 0;
+        HIP_OK(hipHostMalloc(&s.host, cap, hipHostMallocDefault));
+        HIP_OK(hipMalloc(&s.dev, cap));
+        s.cap = cap;
+    }
+    return 1;
+}
+
+int slot_upload(MetaSlot& s, size_t bytes) {
+    HIP_OK(hipMemcpyAsync(s.dev, s.host, bytes, hipMemcpyHostToDevice, g.stream));
+    return 1;
+}
+
+int slot_mark(MetaSlot& s) {
+    HIP_OK(hipEventRecord(s.done, g.stream));
+    s.pending = true;
+    return 1;
+}
+
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+size_t known_bytes(const void* p) {
+    auto it = g.allocs.find(p);
+    return it == g.allocs.end() ? 0 : it->second;
+}
+
+int finish(int sync) {
+    HIP_OK(hipGetLastError());
+    if (sync) HIP_OK(hipStreamSynchronize(g.stream));
+    return 1;
+}
+
+// ---------------------------------------------------------------- decode plan
+
+int gcd_pow2_cap8(size_t group) {
+    int h = 8;
+    while (h > 1 && (group % (size_t)h) != 0) h >>= 1;
+    return h;
+}
+
+bool plan_matches(const DecodePlan& p, const uint32_t* flat, size_t n_flat, const uint32_t* off,
+                  const uint32_t* seq, const uint32_t* qpos, size_t B, size_t H, size_t Hkv,
+                  size_t D, size_t P, int causal) {
+    if (!p.valid || p.B != B || p.H != H || p.Hkv != Hkv || p.D != D || p.P != P ||
+        p.causal != causal || p.target_items != g.opt_target_items ||
+        p.force_generic != g.opt_force_generic)
+        return false;
+    if (p.pt_flat.size() != n_flat) return false;
+    if (n_flat && std::memcmp(p.pt_flat.data(), flat, n_flat * 4) != 0) return false;
+    if (std::memcmp(p.pt_off.data(), off, (B + 1) * 4) != 0) return false;
+    if (std::memcmp(p.seq_lens.data(), seq, B * 4) != 0) return false;
+    if (std::memcmp(p.q_pos.data(), qpos, B * 4) != 0) return false;
+    return true;
+}
+
+// Builds (or reuses) the device-side metadata for one decode call: the page
+// tables and either the split-K work list of the fast kernel or the per-request
+// limits of the generic one.  The walker calls with byte-identical tables for
+// every layer of a step (compiler/runtime/batched_walker.cpp:316-325), so the
+// result is cached and re-uploaded only when the tables change.
+int build_plan(const uint32_t* flat, size_t n_flat, const uint32_t* off, const uint32_t* seq,
+               const uint32_t* qpos, size_t B, size_t H, size_t Hkv, size_t D, size_t P,
+               int causal, bool pointers_aligned) {
+    DecodePlan& p = g.plan;
+    if (plan_matches(p, flat, n_flat, off, seq, qpos, B, H, Hkv, D, P, causal)) return 1;
+    p.valid = false;
+    p.pt_flat.assign(flat, flat + n_flat);
+    p.pt_off.assign(off, off + B + 1);
+    p.seq_lens.assign(seq, seq + B);
+    p.q_pos.assign(qpos, qpos + B);
+    p.B = B; p.H = H; p.Hkv = Hkv; p.D = D; p.P = P; p.causal = causal;
+    p.target_items = g.opt_target_items;
+    p.force_generic = g.opt_force_generic;
+
+    std::vector<uint32_t> limits(B);
+    for (size_t r = 0; r < B; ++r) {
+        uint64_t lim = seq[r];
+        if (causal && (uint64_t)qpos[r] + 1 < lim) lim = (uint64_t)qpos[r] + 1;  // :2286
+        limits[r] = (uint32_t)lim;
+    }
+
+    const size_t tile = (D == 64) ? 64 : 32;
+    p.fast = !g.opt_force_generic && pointers_aligned && (D == 64 || D == 128) && (P % tile) == 0;
+    const size_t flat_bytes = align_up(n_flat * 4, 16);
+
+    std::vector<DecodeWorkItem> items;
+    std::vector<MergeEntry> merges;
+    p.n_part = 0;
+    if (p.fast) {
+        const size_t G = H / Hkv;
+        p.hpw = gcd_pow2_cap8(G);
+        const size_t NG = G / (size_t)p.hpw;
+        size_t total_tiles = 0;
+        for (size_t r = 0; r < B; ++r) total_tiles += (limits[r] + tile - 1) / tile;
+        total_tiles *= Hkv * NG;
+        // Aim for a few resident waves per SIMD on every CU; never split below one tile.
+        size_t target = g.opt_target_items > 0 ? (size_t)g.opt_target_items : (size_t)g.n_cu * 8;
+        size_t chunk = std::max<size_t>(1, (total_tiles + target - 1) / target);
+        for (size_t r = 0; r < B; ++r) {
+            const size_t tiles_r = (limits[r] + tile - 1) / tile;
+            const size_t ns = std::max<size_t>(1, (tiles_r + chunk - 1) / chunk);
+            const size_t per = (tiles_r + ns - 1) / ns;
+            const size_t ns_eff = tiles_r == 0 ? 1 : (tiles_r + per - 1) / per;
+            for (size_t kvh = 0; kvh < Hkv; ++kvh) {
+                for (size_t hg = 0; hg < NG; ++hg) {
+                    const uint32_t head0 = (uint32_t)(kvh * G + hg * p.hpw);
+                    uint32_t first_part = kNoPartial;
+                    if (ns_eff > 1) {
+                        first_part = p.n_part;
+                        merges.push_back({(uint32_t)r, head0, first_part, (uint32_t)ns_eff});
+                        p.n_part += (uint32_t)ns_eff;
+                    }
+                    for (size_t s = 0; s < ns_eff; ++s) {
+                        DecodeWorkItem it;
+                        it.req = (uint32_t)r;
+                        it.head0 = head0;
+                        it.kv_head = (uint32_t)kvh;
+                        it.pt_base = off[r];
+                        it.tok_begin = (uint32_t)std::min<size_t>(s * per * tile, limits[r]);
+                        it.tok_end = (uint32_t)std::min<size_t>((s + 1) * per * tile, limits[r]);
+                        it.part_idx = ns_eff > 1 ? first_part + (uint32_t)s : kNoPartial;
+                        it.pad = 0;
+                        items.push_back(it);
+                    }
+                }
+            }
+        }
+        // Longest first, so the tail of the launch is made of short items.
+        std::stable_sort(items.begin(), items.end(), [](const DecodeWorkItem& x,
+                                                        const DecodeWorkItem& y) {
+            return (x.tok_end - x.tok_begin) > (y.tok_end - y.tok_begin);
+        });
+        p.n_items = (uint32_t)items.size();
+        p.n_merge = (uint32_t)merges.size();
+        p.off_items = flat_bytes;
+        p.off_merge = p.off_items + items.size() * sizeof(DecodeWorkItem);
+        const size_t total = p.off_merge + merges.size() * sizeof(MergeEntry);
+        MetaSlot& s = g.plan_slots[g.plan_next];
+        if (!slot_reserve(s, std::max<size_t>(total, 16))) return 0;
+        char* h = static_cast<char*>(s.host);
+        if (n_flat) std::memcpy(h, flat, n_flat * 4);
+        if (!items.empty()) std::memcpy(h + p.off_items, items.data(), items.size() * sizeof(DecodeWorkItem));
+        if (!merges.empty()) std::memcpy(h + p.off_merge, merges.data(), merges.size() * sizeof(MergeEntry));
+        if (!slot_upload(s, std::max<size_t>(total, 16))) return 0;
+    } else {
+        p.hpw = 0;
+        p.n_items = (uint32_t)(B * H);
+        p.n_merge = 0;
+        p.off_ptoff = flat_bytes;
+        p.off_limits = p.off_ptoff + align_up(B * 4, 16);
+        const size_t total = p.off_limits + align_up(B * 4, 16);
+        MetaSlot& s = g.plan_slots[g.plan_next];
+        if (!slot_reserve(s, total)) return 0;
+        char* h = static_cast<char*>(s.host);
+        if (n_flat) std::memcpy(h, flat, n_flat * 4);
+        std::memcpy(h + p.off_ptoff, off, B * 4);
+        std::memcpy(h + p.off_limits, limits.data(), B * 4);
+        if (!slot_upload(s, total)) return 0;
+    }
+    p.slot = g.plan_next;
+    g.plan_next = (g.plan_next + 1) % 4;
+    p.valid = true;
+    return 1;
+}
+
+int ensure_partials(size_t n_part, int hpw, size_t D) {
+    const size_t need_o = n_part * (size_t)hpw * D;
+    const size_t need_ml = n_part * (size_t)hpw;
+    if (need_o > g.part_o_cap || need_ml > g.part_ml_cap) {
+        HIP_OK(hipStreamSynchronize(g.stream));
+        if (g.part_o) HIP_OK(hipFree(g.part_o));
+        if (g.part_ml) HIP_OK(hipFree(g.part_ml));
+        g.part_o = nullptr;
+        g.part_ml = nullptr;
+        g.part_o_cap = g.part_ml_cap = 0;
+        const size_t cap_o = std::max<size_t>(need_o * 2, 1 << 20);
+        const size_t cap_ml = std::max<size_t>(need_ml * 2, 1 << 14);
+        HIP_OK(hipMalloc(reinterpret_cast<void**>(&g.part_o), cap_o * sizeof(float)));
+        HIP_OK(hipMalloc(reinterpret_cast<void**>(&g.part_ml), cap_ml * sizeof(float2)));
+        g.part_o_cap = cap_o;
+        g.part_ml_cap = cap_ml;
+    }
+    return 1;
+}
+
+template <int D>
+void launch_fast(int hpw, const DecodeArgs& a) {
+    const dim3 grid(a.n_items), block(64);
+    switch (hpw) {
+        case 8: hipLaunchKernelGGL((paged_decode_fast_kernel<D, 8>), grid, block, 0, g.stream, a); break;
+        case 4: hipLaunchKernelGGL((paged_decode_fast_kernel<D, 4>), grid, block, 0, g.stream, a); break;
+        case 2: hipLaunchKernelGGL((paged_decode_fast_kernel<D, 2>), grid, block, 0, g.stream, a); break;
+        default: hipLaunchKernelGGL((paged_decode_fast_kernel<D, 1>), grid, block, 0, g.stream, a); break;
+    }
+}
+
+void launch_merge(int hpw, uint32_t n_merge, const MergeEntry* e, float* o, uint32_t H, uint32_t D) {
+    const dim3 grid(n_merge, (unsigned)hpw), block(D <= 64 ? 64 : 128);
+    switch (hpw) {
+        case 8: hipLaunchKernelGGL((paged_decode_merge_kernel<8>), grid, block, 0, g.stream, e, g.part_o, g.part_ml, o, H, D); break;
+        case 4: hipLaunchKernelGGL((paged_decode_merge_kernel<4>), grid, block, 0, g.stream, e, g.part_o, g.part_ml, o, H, D); break;
+        case 2: hipLaunchKernelGGL((paged_decode_merge_kernel<2>), grid, block, 0, g.stream, e, g.part_o, g.part_ml, o, H, D); break;
+        default: hipLaunchKernelGGL((paged_decode_merge_kernel<1>), grid, block, 0, g.stream, e, g.part_o, g.part_ml, o, H, D); break;
+    }
+}
+
+// Largest page id a request actually dereferences, for bounds checks against
+// pools this library allocated itself.
+int check_pool_bounds(const void* pool, const uint32_t* flat, const uint32_t* off,
+                      const uint32_t* seq, size_t B, size_t P, size_t row_bytes,
+                      const char* what) {
+    const size_t bytes = known_bytes(pool);
+    if (!bytes) return 1;
+    for (size_t r = 0; r < B; ++r) {
+        const size_t pages = (seq[r] + P - 1) / P;
+        for (size_t i = 0; i < pages; ++i) {
+            const size_t end = ((size_t)flat[off[r] + i] + 1) * P * row_bytes;
+            if (end > bytes) return fail(std::string(what) + ": page id beyond the pool");
+        }
+    }
+    return 1;
+}
+
+}  // namespace
+
+// ============================================================== C ABI
+
+extern "C" {
+
+int mlc_hip_available(void) { return init_once() ? 1 : 0; }
+
+const char* mlc_hip_last_error(void) { return g_err.c_str(); }
+
+void* mlc_hip_alloc(size_t bytes) {
+    if (!init_once()) return nullptr;
+    void* p = nullptr;
+    if (hipMalloc(&p, bytes ? bytes : 1) != hipSuccess) {
+        g_err = "hipMalloc failed";
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    g.allocs[p] = bytes;
+    return p;
+}
+
+void mlc_hip_free(void* buffer) {
+    if (!buffer || !init_once()) return;
+    (void)hipStreamSynchronize(g.stream);
+    g.allocs.erase(buffer);
+    (void)hipFree(buffer);
+}
+
+void* mlc_hip_cached(const char* name, size_t bytes) {
+    if (!init_once() || !name) return nullptr;
+    auto it = g.cached.find(name);
+    if (it != g.cached.end() && it->second.second >= bytes) return it->second.first;
+    if (it != g.cached.end()) {  // grow-only reallocation, metal_runtime.mm:8222-8241
+        (void)hipStreamSynchronize(g.stream);
+        g.allocs.erase(it->second.first);
+        (void)hipFree(it->second.first);
+        g.cached.erase(it);
+    }
+    void* p = nullptr;
+    if (hipMalloc(&p, bytes ? bytes : 1) != hipSuccess) {
+        g_err = "hipMalloc failed";
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    g.cached[name] = {p, bytes};
+    g.allocs[p] = bytes;
+    return p;
+}
+
+int mlc_hip_upload(void* buffer, const void* src, size_t bytes, size_t dst_offset) {
+    if (!init_once()) return fail("GPU unavailable");
+    if (!buffer || (!src && bytes)) return fail("upload: null pointer");
+    if (!bytes) return 1;
+    const size_t known = known_bytes(buffer);
+    if (known && dst_offset + bytes > known) return fail("upload: beyond the buffer");
+    HIP_OK(hipMemcpyAsync(static_cast<char*>(buffer) + dst_offset, src, bytes,
+                          hipMemcpyHostToDevice, g.stream));
+    HIP_OK(hipStreamSynchronize(g.stream));
+    return 1;
+}
+
+int mlc_hip_download(const void* buffer, void* dst, size_t bytes, size_t src_offset) {
+    if (!init_once()) return fail("GPU unavailable");
+    if (!buffer || (!dst && bytes)) return fail("download: null pointer");
+    if (!bytes) return 1;
+    const size_t known = known_bytes(buffer);
+    if (known && src_offset + bytes > known) return fail("download: beyond the buffer");
+    HIP_OK(hipMemcpyAsync(dst, static_cast<const char*>(buffer) + src_offset, bytes,
+                          hipMemcpyDeviceToHost, g.stream));
+    HIP_OK(hipStreamSynchronize(g.stream));
+    return 1;
+}
+
+int mlc_hip_zero(void* buffer, size_t bytes) {
+    if (!init_once()) return fail("GPU unavailable");
+    if (!buffer) return fail("zero: null pointer");
+    const size_t known = known_bytes(buffer);
+    if (known && bytes > known) return fail("zero: beyond the buffer");
+    if (bytes) HIP_OK(hipMemsetAsync(buffer, 0, bytes, g.stream));
+    return 1;
+}
+
+int mlc_hip_begin(void) {
+    if (!init_once()) return fail("GPU unavailable");
+    g.pass_open = true;  // idempotent, metal_runtime.mm:6003
+    return 1;
+}
+
+int mlc_hip_flush(void) {
+    if (!init_once()) return fail("GPU unavailable");
+    if (!g.pass_open) return 1;
+    g.pass_open = false;
+    HIP_OK(hipStreamSynchronize(g.stream));
+    return 1;
+}
+
+int mlc_hip_has_open_pass(void) { return (g.inited && g.pass_open) ? 1 : 0; }
+
+int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_pages, void* o,
+                              const uint32_t* page_tables_flat, size_t n_flat,
+                              const uint32_t* page_table_offsets, const uint32_t* seq_lens,
+                              const uint32_t* q_positions, size_t batch, size_t num_heads,
+                              size_t kv_heads, size_t head_dim, size_t page_size_tokens,
+                              int apply_causal, int sync) {
+    if (!init_once()) return fail("GPU unavailable");
+    if (!sync && !g.pass_open) return fail("encode: no open forward pass");  // :7090
+    // metal_runtime.mm:7742-7750
+    if (!q || !k_pages || !v_pages || !o) return fail("decode: null buffer");
+    if (batch == 0 || num_heads == 0 || head_dim == 0 || page_size_tokens == 0)
+        return fail("decode: zero dimension");
+    if (kv_heads == 0 || (num_heads % kv_heads) != 0) return fail("decode: heads % kv_heads != 0");
+    if (!page_table_offsets || !seq_lens || !q_positions) return fail("decode: null metadata");
+    if (n_flat && !page_tables_flat) return fail("decode: null page table");
+    if (n_flat < page_table_offsets[batch]) return fail("decode: page table shorter than offsets");
+    if (head_dim > 256) return fail("decode: head_dim > 256");
+    if (batch > 0x7FFFFFFFull / num_heads) return fail("decode: batch*heads too large");
+    // Beyond the reference: every request's table must cover its sequence, or the
+    // kernel would read page ids past the end of the metadata.
+    for (size_t r = 0; r < batch; ++r) {
+        const size_t pages = ((size_t)seq_lens[r] + page_size_tokens - 1) / page_size_tokens;
+        if ((size_t)page_table_offsets[r] + pages > n_flat)
+            return fail("decode: page table does not cover seq_len");
+    }
+    const size_t row_bytes = kv_heads * head_dim * 2;
+    if (!check_pool_bounds(k_pages, page_tables_flat, page_table_offsets, seq_lens, batch,
+                           page_size_tokens, row_bytes, "decode K") ||
+        !check_pool_bounds(v_pages, page_tables_flat, page_table_offsets, seq_lens, batch,
+                           page_size_tokens, row_bytes, "decode V"))
+        return 0;
+
+    const bool aligned = aligned16(q) && aligned16(k_pages) && aligned16(v_pages) && aligned16(o);
+    if (!build_plan(page_tables_flat, n_flat, page_table_offsets, seq_lens, q_positions, batch,
+                    num_heads, kv_heads, head_dim, page_size_tokens, apply_causal ? 1 : 0, aligned))
+        return 0;
+    const DecodePlan& p = g.plan;
+    MetaSlot& slot = g.plan_slots[p.slot];
+    const char* dev = static_cast<const char*>(slot.dev);
+    const float scale_log2e = (1.0f / std::sqrt(static_cast<float>(head_dim))) * 1.44269504088896340736f;
+
+    g.last_launches = 0;
+    g.last_items = (int)p.n_items;
+    if (p.fast) {
+        if (p.n_part && !ensure_partials(p.n_part, p.hpw, head_dim)) return 0;
+        DecodeArgs a;
+        a.q = static_cast<const float*>(q);
+        a.k_pages = static_cast<const uint4*>(k_pages);
+        a.v_pages = static_cast<const uint4*>(v_pages);
+        a.o = static_cast<float*>(o);
+        a.pt_flat = reinterpret_cast<const uint32_t*>(dev);
+        a.items = reinterpret_cast<const DecodeWorkItem*>(dev + p.off_items);
+        a.part_o = g.part_o;
+        a.part_ml = g.part_ml;
+        a.num_heads = (uint32_t)num_heads;
+        a.kv_heads = (uint32_t)kv_heads;
+        a.page_size = (uint32_t)page_size_tokens;
+        a.n_items = p.n_items;
+        a.scale_log2e = scale_log2e;
+        if (head_dim == 64) launch_fast<64>(p.hpw, a); else launch_fast<128>(p.hpw, a);
+        ++g.last_launches;
+        if (p.n_merge) {
+            launch_merge(p.hpw, p.n_merge, reinterpret_cast<const MergeEntry*>(dev + p.off_merge),
+                         a.o, a.num_heads, (uint32_t)head_dim);
+            ++g.last_launches;
+        }
+    } else {
+        GenericArgs a;
+        a.q = static_cast<const float*>(q);
+        a.k_pages = static_cast<const _Float16*>(k_pages);
+        a.v_pages = static_cast<const _Float16*>(v_pages);
+        a.o = static_cast<float*>(o);
+        a.pt_flat = reinterpret_cast<const uint32_t*>(dev);
+        a.pt_off = reinterpret_cast<const uint32_t*>(dev + p.off_ptoff);
+        a.limits = reinterpret_cast<const uint32_t*>(dev + p.off_limits);
+        a.num_heads = (uint32_t)num_heads;
+        a.kv_heads = (uint32_t)kv_heads;
+        a.head_dim = (uint32_t)head_dim;
+        a.page_size = (uint32_t)page_size_tokens;
+        a.scale_log2e = scale_log2e;
+        hipLaunchKernelGGL(paged_decode_generic_kernel, dim3((unsigned)(batch * num_heads)),
+                           dim3(64), 0, g.stream, a);
+        ++g.last_launches;
+    }
+    if (!slot_mark(slot)) return 0;
+    return finish(sync);
+}
+
+int mlc_hip_scatter_kv_paged_batched_f16(void* page_storage, const uint32_t* page_ids,
+                                         const uint32_t* slots_in_page, size_t page_size_tokens,
+                                         size_t n_kv_heads, size_t head_dim, size_t batch,
+                                         const void* src, int sync) {
+    if (!init_once()) return fail("GPU unavailable");
+    if (!sync && !g.pass_open) return fail("encode: no open forward pass");  // :7178
+    // metal_runtime.mm:7241-7243
+    if (!page_storage || !src) return fail("scatter: null buffer");
+    if (batch == 0 || n_kv_heads == 0 || head_dim == 0 || page_size_tokens == 0)
+        return fail("scatter: zero dimension");
+    if (!page_ids || !slots_in_page) return fail("scatter: null metadata");
+    const size_t row_bytes = n_kv_heads * head_dim * 2;
+    if (batch * row_bytes / 2 > 0x7FFFFFFFull) return fail("scatter: too many elements");
+    // Beyond the reference: a slot outside the page would land in the next page.
+    for (size_t r = 0; r < batch; ++r)
+        if (slots_in_page[r] >= page_size_tokens) return fail("scatter: slot >= page size");
+    const size_t known = known_bytes(page_storage);
+    if (known) {
+        for (size_t r = 0; r < batch; ++r)
+            if (((size_t)page_ids[r] + 1) * page_size_tokens * row_bytes > known)
+                return fail("scatter: page id beyond the pool");
+    }
+    const size_t known_src = known_bytes(src);
+    if (known_src && batch * row_bytes > known_src) return fail("scatter: src too small");
+
+    MetaSlot& s = g.ring[g.ring_next];
+    g.ring_next = (g.ring_next + 1) % 8;
+    const size_t ids_bytes = align_up(batch * 4, 16);
+    if (!slot_reserve(s, ids_bytes * 2)) return 0;
+    std::memcpy(s.host, page_ids, batch * 4);
+    std::memcpy(static_cast<char*>(s.host) + ids_bytes, slots_in_page, batch * 4);
+    if (!slot_upload(s, ids_bytes * 2)) return 0;
+    const uint32_t* d_ids = static_cast<const uint32_t*>(s.dev);
+    const uint32_t* d_slots = reinterpret_cast<const uint32_t*>(static_cast<char*>(s.dev) + ids_bytes);
+
+    const unsigned block = 256;
+    if ((row_bytes % 16) == 0 && aligned16(page_storage) && aligned16(src)) {
+        const uint32_t row_units = (uint32_t)(row_bytes / 16);
+        const unsigned total = (unsigned)(batch * row_units);
+        hipLaunchKernelGGL(scatter_kv_paged_batched_kernel<uint4>, dim3((total + block - 1) / block),
+                           dim3(block), 0, g.stream, static_cast<const uint4*>(src),
+                           static_cast<uint4*>(page_storage), d_ids, d_slots, (uint32_t)batch,
+                           row_units, (uint32_t)page_size_tokens);
+    } else {
+        const uint32_t row_units = (uint32_t)(row_bytes / 2);
+        const unsigned total = (unsigned)(batch * row_units);
+        hipLaunchKernelGGL(scatter_kv_paged_batched_kernel<uint16_t>,
+                           dim3((total + block - 1) / block), dim3(block), 0, g.stream,
+                           static_cast<const uint16_t*>(src), static_cast<uint16_t*>(page_storage),
+                           d_ids, d_slots, (uint32_t)batch, row_units, (uint32_t)page_size_tokens);
+    }
+    if (!slot_mark(s)) return 0;
+    return finish(sync);
+}
+
+int mlc_hip_scatter_kv_paged(void* page_storage, const uint32_t* page_table, size_t n_page_table,
+                             size_t page_size_tokens, size_t n_kv_heads, size_t head_dim,
+                             size_t tokens, size_t start_slot, const void* src,
+                             size_t dtype_bytes) {
+    if (!init_once()) return fail("GPU unavailable");
+    // metal_runtime.mm:7839-7845
+    if (!page_storage || !src) return fail("scatter_paged: null buffer");
+    if (page_size_tokens == 0 || n_kv_heads == 0 || head_dim == 0 || tokens == 0)
+        return fail("scatter_paged: zero dimension");
+    if (dtype_bytes != 2 && dtype_bytes != 4) return fail("scatter_paged: dtype_bytes");
+    if (start_slot >= page_size_tokens) return fail("scatter_paged: start_slot >= page size");
+    const size_t needed = (start_slot + tokens + page_size_tokens - 1) / page_size_tokens;
+    if (n_page_table < needed || !page_table) return fail("scatter_paged: page table too short");
+    const size_t row_bytes = n_kv_heads * head_dim * dtype_bytes;
+    const size_t known = known_bytes(page_storage);
+    if (known)
+        for (size_t i = 0; i < needed; ++i)
+            if (((size_t)page_table[i] + 1) * page_size_tokens * row_bytes > known)
+                return fail("scatter_paged: page id beyond the pool");
+    const size_t known_src = known_bytes(src);
+    if (known_src && tokens * row_bytes > known_src) return fail("scatter_paged: src too small");
+
+    MetaSlot& s = g.ring[g.ring_next];
+    g.ring_next = (g.ring_next + 1) % 8;
+    if (!slot_reserve(s, needed * 4)) return 0;
+    std::memcpy(s.host, page_table, needed * 4);
+    if (!slot_upload(s, needed * 4)) return 0;
+    const uint32_t* d_pt = static_cast<const uint32_t*>(s.dev);
+    const size_t head_bytes = head_dim * dtype_bytes;
+    const unsigned block = 256;
+    if ((head_bytes % 16) == 0 && aligned16(page_storage) && aligned16(src)) {
+        const uint32_t hu = (uint32_t)(head_bytes / 16);
+        const size_t total = n_kv_heads * tokens * hu;
+        hipLaunchKernelGGL(scatter_kv_paged_kernel<uint4>, dim3((unsigned)((total + block - 1) / block)),
+                           dim3(block), 0, g.stream, static_cast<const uint4*>(src),
+                           static_cast<uint4*>(page_storage), d_pt, (uint32_t)n_kv_heads,
+                           (uint32_t)tokens, hu, (uint32_t)page_size_tokens, (uint32_t)start_slot);
+    } else if (dtype_bytes == 4) {
+        const size_t total = n_kv_heads * tokens * head_dim;
+        hipLaunchKernelGGL(scatter_kv_paged_kernel<uint32_t>, dim3((unsigned)((total + block - 1) / block)),
+                           dim3(block), 0, g.stream, static_cast<const uint32_t*>(src),
+                           static_cast<uint32_t*>(page_storage), d_pt, (uint32_t)n_kv_heads,
+                           (uint32_t)tokens, (uint32_t)head_dim, (uint32_t)page_size_tokens,
+                           (uint32_t)start_slot);
+    } else {
+        const size_t total = n_kv_heads * tokens * head_dim;
+        hipLaunchKernelGGL(scatter_kv_paged_kernel<uint16_t>, dim3((unsigned)((total + block - 1) / block)),
+                           dim3(block), 0, g.stream, static_cast<const uint16_t*>(src),
+                           static_cast<uint16_t*>(page_storage), d_pt, (uint32_t)n_kv_heads,
+                           (uint32_t)tokens, (uint32_t)head_dim, (uint32_t)page_size_tokens,
+                           (uint32_t)start_slot);
+    }
+    if (!slot_mark(s)) return 0;
+    return finish(1);
+}
+
+int mlc_hip_gather_kv_pages(const void* page_storage, const uint32_t* page_table,
+                            size_t n_page_table, size_t page_size_tokens, size_t n_kv_heads,
+                            size_t head_dim, size_t num_tokens, void* dst, size_t dtype_bytes) {
+    if (!init_once()) return fail("GPU unavailable");
+    // metal_runtime.mm:7657-7662
+    if (!page_storage || !dst) return fail("gather: null buffer");
+    if (page_size_tokens == 0 || n_kv_heads == 0 || head_dim == 0 || num_tokens == 0)
+        return fail("gather: zero dimension");
+    if (dtype_bytes != 2 && dtype_bytes != 4) return fail("gather: dtype_bytes");
+    const size_t needed = (num_tokens + page_size_tokens - 1) / page_size_tokens;
+    if (n_page_table < needed || !page_table) return fail("gather: page table too short");
+    const size_t row_bytes = n_kv_heads * head_dim * dtype_bytes;
+    const size_t known = known_bytes(page_storage);
+    if (known)
+        for (size_t i = 0; i < needed; ++i)
+            if (((size_t)page_table[i] + 1) * page_size_tokens * row_bytes > known)
+                return fail("gather: page id beyond the pool");
+    const size_t known_dst = known_bytes(dst);
+    if (known_dst && num_tokens * row_bytes > known_dst) return fail("gather: dst too small");
+
+    MetaSlot& s = g.ring[g.ring_next];
+    g.ring_next = (g.ring_next + 1) % 8;
+    if (!slot_reserve(s, needed * 4)) return 0;
+    std::memcpy(s.host, page_table, needed * 4);
+    if (!slot_upload(s, needed * 4)) return 0;
+    const uint32_t* d_pt = static_cast<const uint32_t*>(s.dev);
+    const size_t head_bytes = head_dim * dtype_bytes;
+    const unsigned block = 256;
+    if ((head_bytes % 16) == 0 && aligned16(page_storage) && aligned16(dst)) {
+        const uint32_t hu = (uint32_t)(head_bytes / 16);
+        const size_t total = n_kv_heads * num_tokens * hu;
+        hipLaunchKernelGGL(gather_kv_pages_kernel<uint4>, dim3((unsigned)((total + block - 1) / block)),
+                           dim3(block), 0, g.stream, static_cast<const uint4*>(page_storage),
+                           static_cast<uint4*>(dst), d_pt, (uint32_t)n_kv_heads,
+                           (uint32_t)num_tokens, hu, (uint32_t)page_size_tokens);
+    } else if (dtype_bytes == 4) {
+        const size_t total = n_kv_heads * num_tokens * head_dim;
+        hipLaunchKernelGGL(gather_kv_pages_kernel<uint32_t>, dim3((unsigned)((total + block - 1) / block)),
+                           dim3(block), 0, g.stream, static_cast<const uint32_t*>(page_storage),
+                           static_cast<uint32_t*>(dst), d_pt, (uint32_t)n_kv_heads,
+                           (uint32_t)num_tokens, (uint32_t)head_dim, (uint32_t)page_size_tokens);
+    } else {
+        const size_t total = n_kv_heads * num_tokens * head_dim;
+        hipLaunchKernelGGL(gather_kv_pages_kernel<uint16_t>, dim3((unsigned)((total + block - 1) / block)),
+                           dim3(block), 0, g.stream, static_cast<const uint16_t*>(page_storage),
+                           static_cast<uint16_t*>(dst), d_pt, (uint32_t)n_kv_heads,
+                           (uint32_t)num_tokens, (uint32_t)head_dim, (uint32_t)page_size_tokens);
+    }
+    if (!slot_mark(s)) return 0;
+    return finish(1);
+}
+
+int mlc_hip_paged_attn_prefill(const void* q_f16, const void* k_pages, const void* v_pages,
+                               void* o, const uint32_t* page_tables_flat, size_t n_flat,
+                               const uint32_t* page_table_offsets, const uint32_t* seq_lens,
+                               const uint32_t* q_start, size_t batch, size_t chunk,
+                               size_t num_heads, size_t kv_heads, size_t head_dim,
+                               size_t page_size_tokens, int sync) {
+    if (!init_once()) return fail("GPU unavailable");
+    if (!sync && !g.pass_open) return fail("encode: no open forward pass");
+    if (!q_f16 || !k_pages || !v_pages || !o) return fail("prefill: null buffer");
+    if (batch == 0 || chunk == 0 || num_heads == 0 || head_dim == 0 || page_size_tokens == 0)
+        return fail("prefill: zero dimension");
+    if (kv_heads == 0 || (num_heads % kv_heads) != 0) return fail("prefill: heads % kv_heads != 0");
+    if (!page_table_offsets || !seq_lens || !q_start) return fail("prefill: null metadata");
+    if (n_flat && !page_tables_flat) return fail("prefill: null page table");
+    if (n_flat < page_table_offsets[batch]) return fail("prefill: page table shorter than offsets");
+    for (size_t r = 0; r < batch; ++r) {
+        const size_t pages = ((size_t)seq_lens[r] + page_size_tokens - 1) / page_size_tokens;
+        if ((size_t)page_table_offsets[r] + pages > n_flat)
+            return fail("prefill: page table does not cover seq_len");
+    }
+    const size_t row_bytes = kv_heads * head_dim * 2;
+    if (!check_pool_bounds(k_pages, page_tables_flat, page_table_offsets, seq_lens, batch,
+                           page_size_tokens, row_bytes, "prefill K") ||
+        !check_pool_bounds(v_pages, page_tables_flat, page_table_offsets, seq_lens, batch,
+                           page_size_tokens, row_bytes, "prefill V"))
+        return 0;
+    if (!prefill_shape_supported(head_dim, page_size_tokens) || !aligned16(q_f16) ||
+        !aligned16(k_pages) || !aligned16(v_pages) || !aligned16(o))
+        return fail("prefill: unsupported shape (head_dim must be 128 or 64, page size a multiple of 32, 16-byte aligned buffers)");
+
+    MetaSlot& s = g.ring[g.ring_next];
+    g.ring_next = (g.ring_next + 1) % 8;
+    const size_t flat_bytes = align_up(std::max<size_t>(n_flat, 1) * 4, 16);
+    const size_t vec_bytes = align_up(batch * 4, 16);
+    const size_t total = flat_bytes + 3 * vec_bytes;
+    if (!slot_reserve(s, total)) return 0;
+    char* h = static_cast<char*>(s.host);
+    if (n_flat) std::memcpy(h, page_tables_flat, n_flat * 4);
+    std::memcpy(h + flat_bytes, page_table_offsets, batch * 4);
+    std::memcpy(h + flat_bytes + vec_bytes, seq_lens, batch * 4);
+    std::memcpy(h + flat_bytes + 2 * vec_bytes, q_start, batch * 4);
+    if (!slot_upload(s, total)) return 0;
+    const char* dev = static_cast<const char*>(s.dev);
+    PrefillArgs a;
+    a.q = static_cast<const _Float16*>(q_f16);
+    a.k_pages = static_cast<const _Float16*>(k_pages);
+    a.v_pages = static_cast<const _Float16*>(v_pages);
+    a.o = static_cast<float*>(o);
+    a.pt_flat = reinterpret_cast<const uint32_t*>(dev);
+    a.pt_off = reinterpret_cast<const uint32_t*>(dev + flat_bytes);
+    a.seq_lens = reinterpret_cast<const uint32_t*>(dev + flat_bytes + vec_bytes);
+    a.q_start = reinterpret_cast<const uint32_t*>(dev + flat_bytes + 2 * vec_bytes);
+    a.batch = (uint32_t)batch;
+    a.chunk = (uint32_t)chunk;
+    a.num_heads = (uint32_t)num_heads;
+    a.kv_heads = (uint32_t)kv_heads;
+    a.page_size = (uint32_t)page_size_tokens;
+    a.scale_log2e = (1.0f / std::sqrt(static_cast<float>(head_dim))) * 1.44269504088896340736f;
+    launch_prefill(a, head_dim, g.stream);
+    if (!slot_mark(s)) return 0;
+    return finish(sync);
+}
+
+void* mlc_hip_stream(void) { return init_once() ? static_cast<void*>(g.stream) : nullptr; }
+
+int mlc_hip_timer_start(void) {
+    if (!init_once()) return fail("GPU unavailable");
+    HIP_OK(hipEventRecord(g.ev0, g.stream));
+    return 1;
+}
+
+float mlc_hip_timer_stop(void) {
+    if (!init_once()) return -1.f;
+    if (hipEventRecord(g.ev1, g.stream) != hipSuccess) return -1.f;
+    if (hipEventSynchronize(g.ev1) != hipSuccess) return -1.f;
+    float ms = -1.f;
+    if (hipEventElapsedTime(&ms, g.ev0, g.ev1) != hipSuccess) return -1.f;
+    return ms;
+}
+
+int mlc_hip_last_decode_launches(void) { return g.last_launches; }
+int mlc_hip_last_decode_work_items(void) { return g.last_items; }
+
+int mlc_hip_set_option(const char* name, long value) {
+    if (!name) return 0;
+    if (!std::strcmp(name, "decode_target_items")) { g.opt_target_items = value; return 1; }
+    if (!std::strcmp(name, "decode_force_generic")) { g.opt_force_generic = value; return 1; }
+    return 0;
+}
+
+}  // extern "C"

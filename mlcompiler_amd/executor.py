@@ -1,0 +1,194 @@
+"""HipExecutor: the Python face of the C ABI, with the method names, argument
+order and bool-return conventions of the reference's MetalExecutor paged path
+(compiler/runtime/metal_runtime.hpp:181-183, 510-533, 619-703), so that tests
+read like tests/test_paged_flash.cpp and tests/test_paged_kv.cpp.
+
+Buffers are opaque device pointers (ints), metadata are sequences of uint32.
+Nothing here computes: every method is one call into csrc/libmlc_hip.so.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from ._lib import NativeLibraryError, load
+
+_u32p = C.POINTER(C.c_uint32)
+
+
+def _u32(seq) -> np.ndarray:
+    return np.ascontiguousarray(seq, dtype=np.uint32)
+
+
+def _ptr(a: np.ndarray):
+    return a.ctypes.data_as(_u32p)
+
+
+class HipExecutor:
+    """Singleton, like MetalExecutor::Instance() (metal_runtime.mm:5774-5777)."""
+
+    _instance = None
+
+    @classmethod
+    def Instance(cls) -> "HipExecutor":
+        if cls._instance is None:
+            cls._instance = cls()
+        return cls._instance
+
+    def __init__(self):
+        self._lib = load()
+
+    # -- availability / errors
+    def isAvailable(self) -> bool:
+        return bool(self._lib.mlc_hip_available())
+
+    def requireAvailable(self) -> None:
+        if not self.isAvailable():
+            raise NativeLibraryError("no gfx950 device: " + self.lastError())
+
+    def lastError(self) -> str:
+        return self._lib.mlc_hip_last_error().decode()
+
+    # -- buffers (metal_runtime.hpp:693-703)
+    def allocateScratchBuffer(self, nbytes: int) -> int:
+        return self._lib.mlc_hip_alloc(nbytes) or 0
+
+    def releaseScratchBuffer(self, buffer: int) -> None:
+        self._lib.mlc_hip_free(buffer)
+
+    def getOrAllocCachedBuffer(self, name: str, nbytes: int) -> int:
+        return self._lib.mlc_hip_cached(name.encode(), nbytes) or 0
+
+    def uploadToBuffer(self, buffer: int, src: np.ndarray, nbytes: int | None = None,
+                       dst_offset: int = 0) -> bool:
+        src = np.ascontiguousarray(src)
+        n = src.nbytes if nbytes is None else nbytes
+        return bool(self._lib.mlc_hip_upload(buffer, src.ctypes.data, n, dst_offset))
+
+    def downloadFromBuffer(self, buffer: int, dst: np.ndarray, nbytes: int | None = None,
+                           src_offset: int = 0) -> bool:
+        assert dst.flags.c_contiguous and dst.flags.writeable
+        n = dst.nbytes if nbytes is None else nbytes
+        return bool(self._lib.mlc_hip_download(buffer, dst.ctypes.data, n, src_offset))
+
+    def zeroBuffer(self, buffer: int, nbytes: int) -> bool:
+        return bool(self._lib.mlc_hip_zero(buffer, nbytes))
+
+    # -- forward pass (metal_runtime.hpp:181-183)
+    def beginForwardPassCB(self) -> bool:
+        return bool(self._lib.mlc_hip_begin())
+
+    def flushForwardPassCB(self) -> bool:
+        return bool(self._lib.mlc_hip_flush())
+
+    def hasForwardPassCB(self) -> bool:
+        return bool(self._lib.mlc_hip_has_open_pass())
+
+    # -- paged flash attention (metal_runtime.hpp:510-523, 645-658)
+    def _attn(self, q, k_pages, v_pages, o, page_tables_flat, page_table_offsets, seq_lens,
+              q_positions, batch, num_heads, kv_heads, head_dim, page_size_tokens, apply_causal,
+              sync) -> bool:
+        flat = _u32(page_tables_flat)
+        off = _u32(page_table_offsets)
+        sl = _u32(seq_lens)
+        qp = _u32(q_positions)
+        # the reference rejects vectors of the wrong length (metal_runtime.mm:7747-7748)
+        if off.size != batch + 1 or sl.size != batch or qp.size != batch:
+            return False
+        flat_arg = flat if flat.size else np.zeros(1, np.uint32)
+        return bool(self._lib.mlc_hip_paged_attn_decode(
+            q, k_pages, v_pages, o, _ptr(flat_arg), flat.size, _ptr(off), _ptr(sl), _ptr(qp),
+            batch, num_heads, kv_heads, head_dim, page_size_tokens, int(bool(apply_causal)), sync))
+
+    def runPagedFlashAttention(self, q_buffer, k_pages_buffer, v_pages_buffer, o_buffer,
+                               page_tables_flat, page_table_offsets, seq_lens, q_positions,
+                               batch, num_heads, kv_heads, head_dim, page_size_tokens,
+                               apply_causal) -> bool:
+        return self._attn(q_buffer, k_pages_buffer, v_pages_buffer, o_buffer, page_tables_flat,
+                          page_table_offsets, seq_lens, q_positions, batch, num_heads, kv_heads,
+                          head_dim, page_size_tokens, apply_causal, 1)
+
+    def encodePagedFlashAttention(self, q_buf, k_pages_buf, v_pages_buf, o_buf, page_tables_flat,
+                                  page_table_offsets, seq_lens, q_positions, batch, num_heads,
+                                  kv_heads, head_dim, page_size_tokens, apply_causal) -> bool:
+        return self._attn(q_buf, k_pages_buf, v_pages_buf, o_buf, page_tables_flat,
+                          page_table_offsets, seq_lens, q_positions, batch, num_heads, kv_heads,
+                          head_dim, page_size_tokens, apply_causal, 0)
+
+    # -- batched paged KV write (metal_runtime.hpp:526-533, 680-687)
+    def _scatter_batched(self, page_storage, page_ids, slots_in_page, page_size_tokens,
+                         n_kv_heads, head_dim, batch, src, sync) -> bool:
+        pid = _u32(page_ids)
+        sl = _u32(slots_in_page)
+        if sync and (pid.size != batch or sl.size != batch):  # metal_runtime.mm:7243
+            return False
+        if pid.size < batch or sl.size < batch:
+            return False
+        return bool(self._lib.mlc_hip_scatter_kv_paged_batched_f16(
+            page_storage, _ptr(pid), _ptr(sl), page_size_tokens, n_kv_heads, head_dim, batch, src,
+            sync))
+
+    def scatterKVPagedBatched(self, page_storage_buffer, page_ids, slots_in_page,
+                              page_size_tokens, n_kv_heads, head_dim, batch, src_buffer) -> bool:
+        return self._scatter_batched(page_storage_buffer, page_ids, slots_in_page,
+                                     page_size_tokens, n_kv_heads, head_dim, batch, src_buffer, 1)
+
+    def encodeScatterKVPagedBatched(self, page_storage_buffer, page_ids, slots_in_page,
+                                    page_size_tokens, n_kv_heads, head_dim, batch,
+                                    src_buffer) -> bool:
+        return self._scatter_batched(page_storage_buffer, page_ids, slots_in_page,
+                                     page_size_tokens, n_kv_heads, head_dim, batch, src_buffer, 0)
+
+    # -- single-request scatter / gather (metal_runtime.hpp:619-626, 666-674)
+    def scatterKVPaged(self, page_storage_buffer, page_table, page_size_tokens, n_kv_heads,
+                       head_dim, tokens, start_slot, src_buffer, dtype_bytes) -> bool:
+        pt = _u32(page_table)
+        pt_arg = pt if pt.size else np.zeros(1, np.uint32)
+        return bool(self._lib.mlc_hip_scatter_kv_paged(
+            page_storage_buffer, _ptr(pt_arg), pt.size, page_size_tokens, n_kv_heads, head_dim,
+            tokens, start_slot, src_buffer, dtype_bytes))
+
+    def gatherKVPages(self, page_storage_buffer, page_table, page_size_tokens, n_kv_heads,
+                      head_dim, num_tokens, dst_buffer, dtype_bytes) -> bool:
+        pt = _u32(page_table)
+        pt_arg = pt if pt.size else np.zeros(1, np.uint32)
+        return bool(self._lib.mlc_hip_gather_kv_pages(
+            page_storage_buffer, _ptr(pt_arg), pt.size, page_size_tokens, n_kv_heads, head_dim,
+            num_tokens, dst_buffer, dtype_bytes))
+
+    # -- chunked prefill (no reference method; see include/mlc_hip.h)
+    def runPagedPrefillAttention(self, q_f16_buffer, k_pages_buffer, v_pages_buffer, o_buffer,
+                                 page_tables_flat, page_table_offsets, seq_lens, q_start, batch,
+                                 chunk, num_heads, kv_heads, head_dim, page_size_tokens,
+                                 sync: bool = True) -> bool:
+        flat = _u32(page_tables_flat)
+        off = _u32(page_table_offsets)
+        sl = _u32(seq_lens)
+        qs = _u32(q_start)
+        if off.size != batch + 1 or sl.size != batch or qs.size != batch:
+            return False
+        flat_arg = flat if flat.size else np.zeros(1, np.uint32)
+        return bool(self._lib.mlc_hip_paged_attn_prefill(
+            q_f16_buffer, k_pages_buffer, v_pages_buffer, o_buffer, _ptr(flat_arg), flat.size,
+            _ptr(off), _ptr(sl), _ptr(qs), batch, chunk, num_heads, kv_heads, head_dim,
+            page_size_tokens, int(bool(sync))))
+
+    # -- measurement helpers
+    def timerStart(self) -> bool:
+        return bool(self._lib.mlc_hip_timer_start())
+
+    def timerStopMs(self) -> float:
+        return float(self._lib.mlc_hip_timer_stop())
+
+    def lastDecodeLaunches(self) -> int:
+        return int(self._lib.mlc_hip_last_decode_launches())
+
+    def lastDecodeWorkItems(self) -> int:
+        return int(self._lib.mlc_hip_last_decode_work_items())
+
+    def setOption(self, name: str, value: int) -> bool:
+        return bool(self._lib.mlc_hip_set_option(name.encode(), int(value)))
+
+    def stream(self) -> int:
+        return self._lib.mlc_hip_stream() or 0

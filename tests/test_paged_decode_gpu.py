@@ -1,0 +1,231 @@
+"""Parity of the HIP paged decode attention against the CPU oracle (the executor-CPU
+ordering of the reference), through the C ABI.  Tolerance: per (request, head)
+cosine >= 0.9999 and max-abs <= 2e-3, as the benchmark definition states."""
+import numpy as np
+import pytest
+
+from paged_cases import (DeviceCase, assert_parity, baseline_config, make_case, oracle_decode,
+                         reference_scenarios)
+
+pytestmark = pytest.mark.gpu
+
+
+def _check(exe, case, sync=True):
+    print(f"[case] {case.name} B={case.batch} H={case.num_heads}/{case.kv_heads} D={case.head_dim} "
+          f"P={case.page_size} causal={case.apply_causal}", flush=True)
+    dev = DeviceCase(exe, case)
+    try:
+        got = dev.run(sync=sync)
+    finally:
+        dev.free()
+    want = oracle_decode(case)
+    assert want is not None
+    return assert_parity(got, want, case.head_dim, case.name), got, want
+
+
+@pytest.mark.parametrize("case", reference_scenarios(), ids=lambda c: c.name)
+def test_reference_scenarios(exe, case):
+    # tests/test_paged_flash.cpp:214-275 asks cosine >= 0.999; the bar here is tighter
+    _check(exe, case)
+
+
+@pytest.mark.parametrize("idx", [1, 2, 3])
+def test_baseline_configs(exe, idx):
+    _check(exe, baseline_config(idx))
+
+
+def test_baseline_config4_reduced_batch(exe):
+    # Llama-3-8B shape with the 1% x8 K rows; 8 requests keep the oracle to seconds
+    _check(exe, baseline_config(4, batch=8))
+
+
+def test_encode_variant_matches_run(exe):
+    case = baseline_config(2, batch=8)
+    dev = DeviceCase(exe, case)
+    try:
+        a = dev.run(sync=True)
+        b = dev.run(sync=False)
+    finally:
+        dev.free()
+    assert np.array_equal(a, b)
+
+
+def test_encode_needs_open_pass(exe):
+    case = make_case("closed", 1, 8, 2, 64, 64, [10])
+    dev = DeviceCase(exe, case)
+    try:
+        assert not exe.hasForwardPassCB()
+        ok = exe.encodePagedFlashAttention(dev.q_buf, dev.k_buf, dev.v_buf, dev.o_buf,
+                                           case.page_tables_flat, case.page_table_offsets,
+                                           case.seq_lens, case.q_positions, 1, 8, 2, 64, 64, True)
+        assert not ok  # metal_runtime.mm:7090
+    finally:
+        dev.free()
+
+
+@pytest.mark.parametrize("gq", [(8, 8), (8, 4), (8, 2), (8, 1), (32, 2), (12, 4), (6, 1)])
+@pytest.mark.parametrize("head_dim", [64, 128])
+def test_gqa_ratios(exe, gq, head_dim):
+    h, hkv = gq
+    case = make_case(f"gqa{h}_{hkv}_d{head_dim}", 3, h, hkv, head_dim, 64, [130, 64, 257], seed=h * 7 + hkv)
+    _check(exe, case)
+
+
+@pytest.mark.parametrize("head_dim,page", [(32, 16), (96, 64), (256, 64), (64, 4), (128, 16), (4, 4),
+                                           (64, 128), (128, 32), (64, 192)])
+def test_other_shapes(exe, head_dim, page):
+    case = make_case(f"d{head_dim}_p{page}", 3, 8, 2, head_dim, page, [37, 1, 200], seed=head_dim + page)
+    _check(exe, case)
+
+
+def test_edge_lengths(exe):
+    # empty request, single token, exactly one page, page + 1, one tile + 1
+    case = make_case("edges", 6, 32, 4, 64, 64, [0, 1, 64, 65, 63, 129])
+    rep, got, want = _check(exe, case)
+    assert np.all(got[0] == 0.0)  # metal_runtime.mm:2254-2257
+    # S == 1 -> O is exactly V[0] (softmax of one score)
+    v = case.v_pages.view(np.float16).reshape(-1, 64, 4, 64)
+    pid = case.page_tables_flat[case.page_table_offsets[1]]
+    for h in range(32):
+        assert np.array_equal(got[1, h], v[pid, 0, h // 8].astype(np.float32))
+
+
+def test_causal_positions(exe):
+    # q_position in the middle of the cache (chunked-prefill style rows) and at 0
+    S = [300, 300, 300, 300, 64, 130]
+    case = make_case("causal_mid", 6, 8, 2, 64, 64, S, q_positions=[0, 63, 64, 150, 10, 129])
+    _check(exe, case)
+    case_nc = make_case("noncausal_mid", 6, 8, 2, 64, 64, S, q_positions=[0, 63, 64, 150, 10, 129],
+                        causal=False)
+    _check(exe, case_nc)
+
+
+def test_unused_tail_is_never_read(exe):
+    # rows past seq_len (rest of the last page, and whole unused pages) hold NaN
+    case = make_case("nan_tail", 4, 32, 4, 64, 64, [100, 64, 1, 200], capacity_pages=16, seed=5)
+    k = case.k_pages.view(np.float16).reshape(16, 64, 4 * 64)
+    v = case.v_pages.view(np.float16).reshape(16, 64, 4 * 64)
+    used = np.zeros((16, 64), bool)
+    for r in range(4):
+        for pos in range(int(case.seq_lens[r])):
+            used[case.page_tables_flat[case.page_table_offsets[r] + pos // 64], pos % 64] = True
+    k[~used] = np.nan
+    v[~used] = np.nan
+    _check(exe, case)
+
+
+def test_page_permutation_invariance(exe):
+    # moving the pages (with their data) to other ids leaves O bit-identical
+    a = make_case("perm_a", 2, 32, 4, 64, 64, [500, 77], capacity_pages=32, permute=False, seed=9)
+    perm = np.random.default_rng(3).permutation(32).astype(np.uint32)
+    b = make_case("perm_b", 2, 32, 4, 64, 64, [500, 77], capacity_pages=32, permute=False, seed=9)
+    kb = b.k_pages.reshape(32, -1).copy()
+    vb = b.v_pages.reshape(32, -1).copy()
+    b.k_pages = np.empty_like(kb)
+    b.v_pages = np.empty_like(vb)
+    b.k_pages[perm] = kb
+    b.v_pages[perm] = vb
+    b.k_pages = b.k_pages.ravel()
+    b.v_pages = b.v_pages.ravel()
+    b.page_tables_flat = perm[a.page_tables_flat]
+    _, got_a, _ = _check(exe, a)
+    _, got_b, _ = _check(exe, b)
+    assert np.array_equal(got_a, got_b)
+
+
+def test_split_k_targets_agree(exe):
+    # the same batch planned as 1 item per (request, kv head) and as many small items
+    case = baseline_config(2, batch=6)
+    want = oracle_decode(case)
+    outs = []
+    for target in (1, 64, 100000):
+        assert exe.setOption("decode_target_items", target)
+        dev = DeviceCase(exe, case)
+        try:
+            outs.append(dev.run())
+            print("items", exe.lastDecodeWorkItems(), "launches", exe.lastDecodeLaunches(), flush=True)
+        finally:
+            dev.free()
+        assert_parity(outs[-1], want, 64, f"target={target}")
+    exe.setOption("decode_target_items", 0)
+    assert np.max(np.abs(outs[0] - outs[2])) < 1e-5
+
+
+def test_generic_kernel_agrees_with_fast(exe):
+    case = baseline_config(2, batch=4)
+    dev = DeviceCase(exe, case)
+    try:
+        fast = dev.run()
+        assert exe.setOption("decode_force_generic", 1)
+        gen = dev.run()
+    finally:
+        exe.setOption("decode_force_generic", 0)
+        dev.free()
+    assert np.max(np.abs(fast - gen)) < 1e-5
+    assert_parity(gen, oracle_decode(case), 64, "generic")
+
+
+def test_plan_cache_across_layers_and_steps(exe):
+    # same tables, different K/V pools (layers); then changed tables (next step)
+    c1 = baseline_config(2, batch=4, seed=1)
+    c2 = baseline_config(2, batch=4, seed=1)
+    rng = np.random.default_rng(77)
+    c2.k_pages = rng.standard_normal(c2.k_pages.size, dtype=np.float32).astype(np.float16).view(np.uint16)
+    c2.v_pages = rng.standard_normal(c2.v_pages.size, dtype=np.float32).astype(np.float16).view(np.uint16)
+    _check(exe, c1)
+    _check(exe, c2)
+    c3 = baseline_config(2, batch=4, seed=2)
+    _check(exe, c3)
+    _check(exe, c1)
+
+
+def test_stress_online_rescale(exe):
+    # compiler/main.cpp:4039-4065: q = 1, K[s] = 0.1*s/D so scores climb with position
+    # and every tile raises the running maximum; gate there is max_abs <= 1e-5
+    H, Hkv, D, S = 32, 4, 64, 2048
+    case = make_case("stress_online", 1, H, Hkv, D, 64, [S], permute=False, seed=42)
+    case.q[:] = 1.0
+    k = case.k_pages.view(np.float16).reshape(-1, Hkv * D)
+    for s in range(S):
+        k[s, :] = np.float16(0.1 * s / D)
+    dev = DeviceCase(exe, case)
+    try:
+        got = dev.run()
+    finally:
+        dev.free()
+    want = oracle_decode(case)
+    rep = assert_parity(got, want, D, "stress")
+    assert rep["max_abs"] <= 1e-5, rep
+
+
+def test_bad_arguments_are_rejected(exe):
+    case = make_case("bad", 2, 8, 2, 64, 64, [10, 20])
+    dev = DeviceCase(exe, case)
+    try:
+        base = dict(q=dev.q_buf, k=dev.k_buf, v=dev.v_buf, o=dev.o_buf, flat=case.page_tables_flat,
+                    off=case.page_table_offsets, sl=case.seq_lens, qp=case.q_positions, B=2, H=8,
+                    Hkv=2, D=64, P=64)
+
+        def run(**kw):
+            a = {**base, **kw}
+            return exe.runPagedFlashAttention(a["q"], a["k"], a["v"], a["o"], a["flat"], a["off"],
+                                              a["sl"], a["qp"], a["B"], a["H"], a["Hkv"], a["D"],
+                                              a["P"], True)
+        assert run()
+        # metal_runtime.mm:7742-7750
+        assert not run(q=0)
+        assert not run(o=0)
+        assert not run(B=0)
+        assert not run(Hkv=3)
+        assert not run(Hkv=0)
+        assert not run(D=512)
+        assert not run(P=0)
+        assert not run(off=case.page_table_offsets[:2])
+        assert not run(sl=case.seq_lens[:1])
+        assert not run(flat=case.page_tables_flat[:1])
+        # beyond the reference: a table that does not cover its sequence
+        assert not run(sl=np.array([10, 2000], np.uint32))
+        # a page id outside a pool this library allocated
+        assert not run(flat=np.array([0, 999], np.uint32))
+    finally:
+        dev.free()
