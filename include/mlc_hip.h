@@ -158,9 +158,11 @@ float mlc_hip_timer_stop(void);
 int mlc_hip_last_decode_launches(void);
 int mlc_hip_last_decode_work_items(void);
 
-/* Tunables: "decode_target_items" (split-K work items aimed for per launch),
- * "decode_force_generic" (1 = always use the shape-agnostic kernel).
- * Returns 0 for an unknown name. */
+/* Tunables: "decode_target_items" (split-K work items aimed for per launch, 0 =
+ * automatic), "decode_heads_per_wave" (1, 2, 4 or 8: the most query heads one
+ * wavefront handles; the GQA group is spread over group/that many waves of a
+ * workgroup), "decode_force_generic" (1 = always use the shape-agnostic kernel).
+ * Returns 0 for an unknown name or value. */
 int mlc_hip_set_option(const char* name, long value);
 
 #ifdef __cplusplus

@@ -3,6 +3,7 @@
   libmlc_hip.so       HIP kernels + the C ABI declared in include/mlc_hip.h
   libhip_executor.so  the C++ HipExecutor class (mirror of the reference's
                       MetalExecutor paged-path methods) on top of that ABI
+  libmlc_bench.so     native benchmark loop that calls the ABI (no kernels)
 """
 from __future__ import annotations
 
@@ -14,12 +15,13 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(CSRC, "libmlc_hip.so")
 EXECUTOR_LIB_PATH = os.path.join(CSRC, "libhip_executor.so")
+BENCH_LIB_PATH = os.path.join(CSRC, "libmlc_bench.so")
 
 # Packed FP32 instructions are switched off on purpose (see DESIGN notes in the
 # repository); the host pass prints a harmless "not a recognized feature" warning.
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
-    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-fno-honor-nans",
 ]
 
 
@@ -37,12 +39,29 @@ def _run(cmd: list[str]) -> None:
 
 
 def build_all(verbose: bool = False) -> None:
+    """Compiles the decode-kernel variants and the runtime in parallel, then links them."""
+    from concurrent.futures import ThreadPoolExecutor
+
     cc = hipcc()
-    _run([cc, *HIPCC_FLAGS, "-shared", os.path.join(CSRC, "mlc_hip.hip"), "-o", LIB_PATH])
+    obj_dir = os.path.join(CSRC, "build")
+    os.makedirs(obj_dir, exist_ok=True)
+    jobs = []
+    for d in (64, 128):
+        for h in (1, 2, 4, 8):
+            obj = os.path.join(obj_dir, f"decode_d{d}_h{h}.o")
+            jobs.append(([cc, *HIPCC_FLAGS, f"-DMLC_D={d}", f"-DMLC_HPW={h}", "-c",
+                          os.path.join(CSRC, "paged_decode_inst.hip"), "-o", obj], obj))
+    rt_obj = os.path.join(obj_dir, "mlc_hip.o")
+    jobs.append(([cc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, "mlc_hip.hip"), "-o", rt_obj], rt_obj))
+    with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
+        list(pool.map(lambda j: _run(j[0]), jobs))
+    _run([cc, "--offload-arch=gfx950", "-shared", "-fPIC", *[j[1] for j in jobs], "-o", LIB_PATH])
     _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", os.path.join(CSRC, "hip_executor.cpp"),
           "-o", EXECUTOR_LIB_PATH, "-L" + CSRC, "-lmlc_hip", "-Wl,-rpath,$ORIGIN"])
+    _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", os.path.join(CSRC, "bench_loop.cpp"),
+          "-o", BENCH_LIB_PATH, "-L" + CSRC, "-lmlc_hip", "-Wl,-rpath,$ORIGIN"])
     if verbose:
-        print("built", LIB_PATH, "and", EXECUTOR_LIB_PATH)
+        print("built", LIB_PATH, EXECUTOR_LIB_PATH, BENCH_LIB_PATH)
 
 
 if __name__ == "__main__":

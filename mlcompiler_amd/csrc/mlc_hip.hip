@@ -17,8 +17,17 @@
 #include <vector>
 
 #include "paged_copy_kernels.h"
+#include "paged_decode_generic.h"
 #include "paged_decode_kernels.h"
 #include "paged_prefill_kernels.h"
+
+namespace mlc_hip {
+// Defined in paged_decode_inst.hip, one object per (head_dim, heads-per-wave).
+#define MLC_DECL(d, h) bool launch_decode_fast_##d##_##h(int, int, bool, const DecodeArgs&, hipStream_t);
+MLC_DECL(64, 1) MLC_DECL(64, 2) MLC_DECL(64, 4) MLC_DECL(64, 8)
+MLC_DECL(128, 1) MLC_DECL(128, 2) MLC_DECL(128, 4) MLC_DECL(128, 8)
+#undef MLC_DECL
+}  // namespace mlc_hip
 
 namespace {
 
@@ -55,12 +64,12 @@ struct DecodePlan {
     std::vector<uint32_t> pt_flat, pt_off, seq_lens, q_pos;
     size_t B = 0, H = 0, Hkv = 0, D = 0, P = 0;
     int causal = 0;
-    long target_items = 0, force_generic = 0;
+    long target_items = 0, force_generic = 0, hpw_max = 0, tile_rows = 0;
     // result
     bool fast = false;
-    int hpw = 0;
-    uint32_t n_items = 0, n_merge = 0, n_part = 0;
-    size_t off_items = 0, off_merge = 0, off_ptoff = 0, off_limits = 0;  // byte offsets in blob
+    int hpw = 0, nw = 0, ns = 0;
+    uint32_t n_items = 0, n_part = 0;
+    size_t off_items = 0, off_ptoff = 0, off_limits = 0;  // byte offsets in blob
     int slot = -1;
 };
 
@@ -79,10 +88,14 @@ struct Ctx {
     int plan_next = 0;
     DecodePlan plan;
     float* part_o = nullptr;
-    float2* part_ml = nullptr;
-    size_t part_o_cap = 0, part_ml_cap = 0;  // in elements
-    long opt_target_items = 0;               // 0 = automatic
+    float* part_ml = nullptr;
+    uint32_t* counters = nullptr;
+    size_t part_o_cap = 0, part_ml_cap = 0, counters_cap = 0;  // in elements
+    long opt_target_items = 0;                                 // 0 = automatic
     long opt_force_generic = 0;
+    long opt_hpw_max = 4;                                      // query heads per wave, at most
+    long opt_tile_rows = 4;                                    // wave rows that share an item's tiles
+    long opt_pv_fp16 = 1;                                      // softmax weights rounded to fp16 for P.V
     int last_launches = 0;
     int last_items = 0;
     int n_cu = 256;
@@ -159,18 +172,13 @@ int finish(int sync) {
 
 // ---------------------------------------------------------------- decode plan
 
-int gcd_pow2_cap8(size_t group) {
-    int h = 8;
-    while (h > 1 && (group % (size_t)h) != 0) h >>= 1;
-    return h;
-}
-
 bool plan_matches(const DecodePlan& p, const uint32_t* flat, size_t n_flat, const uint32_t* off,
                   const uint32_t* seq, const uint32_t* qpos, size_t B, size_t H, size_t Hkv,
                   size_t D, size_t P, int causal) {
     if (!p.valid || p.B != B || p.H != H || p.Hkv != Hkv || p.D != D || p.P != P ||
         p.causal != causal || p.target_items != g.opt_target_items ||
-        p.force_generic != g.opt_force_generic)
+        p.force_generic != g.opt_force_generic || p.hpw_max != g.opt_hpw_max ||
+        p.tile_rows != g.opt_tile_rows)
         return false;
     if (p.pt_flat.size() != n_flat) return false;
     if (n_flat && std::memcmp(p.pt_flat.data(), flat, n_flat * 4) != 0) return false;
@@ -198,6 +206,8 @@ int build_plan(const uint32_t* flat, size_t n_flat, const uint32_t* off, const u
     p.B = B; p.H = H; p.Hkv = Hkv; p.D = D; p.P = P; p.causal = causal;
     p.target_items = g.opt_target_items;
     p.force_generic = g.opt_force_generic;
+    p.hpw_max = g.opt_hpw_max;
+    p.tile_rows = g.opt_tile_rows;
 
     std::vector<uint32_t> limits(B);
     for (size_t r = 0; r < B; ++r) {
@@ -208,47 +218,68 @@ int build_plan(const uint32_t* flat, size_t n_flat, const uint32_t* off, const u
 
     const size_t tile = (D == 64) ? 64 : 32;
     p.fast = !g.opt_force_generic && pointers_aligned && (D == 64 || D == 128) && (P % tile) == 0;
+    const size_t G = H / Hkv;
+    if (p.fast) {
+        // query heads per wave (power of two dividing G), waves per workgroup = G / that
+        int hpw = 8;
+        while (hpw > 1 && (hpw > g.opt_hpw_max || (G % (size_t)hpw) != 0)) hpw >>= 1;
+        size_t nw = G / (size_t)hpw;
+        if (nw > 4 || nw == 3) {  // too many / odd wave counts: use the widest wave
+            hpw = 8;
+            while (hpw > 1 && (G % (size_t)hpw) != 0) hpw >>= 1;
+            nw = G / (size_t)hpw;
+        }
+        if (nw > 4 || nw == 3) p.fast = false;
+        p.hpw = hpw;
+        p.nw = (int)nw;
+        // tile rows per workgroup: at most 8 waves per workgroup
+        int ns = (int)g.opt_tile_rows;
+        while (ns > 1 && (size_t)ns * nw > 8) ns >>= 1;
+        p.ns = ns;
+    }
     const size_t flat_bytes = align_up(n_flat * 4, 16);
 
     std::vector<DecodeWorkItem> items;
-    std::vector<MergeEntry> merges;
     p.n_part = 0;
     if (p.fast) {
-        const size_t G = H / Hkv;
-        p.hpw = gcd_pow2_cap8(G);
-        const size_t NG = G / (size_t)p.hpw;
         size_t total_tiles = 0;
         for (size_t r = 0; r < B; ++r) total_tiles += (limits[r] + tile - 1) / tile;
-        total_tiles *= Hkv * NG;
-        // Aim for a few resident waves per SIMD on every CU; never split below one tile.
-        size_t target = g.opt_target_items > 0 ? (size_t)g.opt_target_items : (size_t)g.n_cu * 8;
+        total_tiles *= Hkv;
+        // Work items (= workgroups) aimed for: enough to give every SIMD two resident waves.
+        const size_t slots = (size_t)g.n_cu * 8 / (size_t)(p.nw * p.ns);
+        size_t target = g.opt_target_items > 0 ? (size_t)g.opt_target_items : slots;
         size_t chunk = std::max<size_t>(1, (total_tiles + target - 1) / target);
+        for (size_t r = 0; r < B; ++r) {  // the merge pass handles at most kMaxSplits partials
+            const size_t tiles_r = (limits[r] + tile - 1) / tile;
+            chunk = std::max(chunk, (tiles_r + kMaxSplits - 1) / kMaxSplits);
+        }
         for (size_t r = 0; r < B; ++r) {
             const size_t tiles_r = (limits[r] + tile - 1) / tile;
             const size_t ns = std::max<size_t>(1, (tiles_r + chunk - 1) / chunk);
             const size_t per = (tiles_r + ns - 1) / ns;
-            const size_t ns_eff = tiles_r == 0 ? 1 : (tiles_r + per - 1) / per;
+            size_t ns_eff = tiles_r == 0 ? 1 : (tiles_r + per - 1) / per;
+            if (ns_eff > 0xFFFF) return fail("decode: too many splits");
             for (size_t kvh = 0; kvh < Hkv; ++kvh) {
-                for (size_t hg = 0; hg < NG; ++hg) {
-                    const uint32_t head0 = (uint32_t)(kvh * G + hg * p.hpw);
-                    uint32_t first_part = kNoPartial;
-                    if (ns_eff > 1) {
-                        first_part = p.n_part;
-                        merges.push_back({(uint32_t)r, head0, first_part, (uint32_t)ns_eff});
-                        p.n_part += (uint32_t)ns_eff;
+                uint32_t first_part = kNoPartial;
+                if (ns_eff > 1) {
+                    first_part = p.n_part;
+                    p.n_part += (uint32_t)ns_eff;
+                }
+                for (size_t s = 0; s < ns_eff; ++s) {
+                    DecodeWorkItem it;
+                    it.req = (uint32_t)r;
+                    it.kv_head = (uint32_t)kvh;
+                    it.pt_base = off[r];
+                    it.tok_begin = (uint32_t)std::min<size_t>(s * per * tile, limits[r]);
+                    it.tok_end = (uint32_t)std::min<size_t>((s + 1) * per * tile, limits[r]);
+                    for (size_t w = 0; w < 4; ++w) {
+                        const size_t t0 = it.tok_begin + w * tile;
+                        it.first_pages[w] = t0 < it.tok_end ? flat[off[r] + t0 / P] : 0;
                     }
-                    for (size_t s = 0; s < ns_eff; ++s) {
-                        DecodeWorkItem it;
-                        it.req = (uint32_t)r;
-                        it.head0 = head0;
-                        it.kv_head = (uint32_t)kvh;
-                        it.pt_base = off[r];
-                        it.tok_begin = (uint32_t)std::min<size_t>(s * per * tile, limits[r]);
-                        it.tok_end = (uint32_t)std::min<size_t>((s + 1) * per * tile, limits[r]);
-                        it.part_idx = ns_eff > 1 ? first_part + (uint32_t)s : kNoPartial;
-                        it.pad = 0;
-                        items.push_back(it);
-                    }
+                    it.part_first = first_part;
+                    it.split = (uint32_t)s | ((uint32_t)ns_eff << 16);
+                    it.pad = 0;
+                    items.push_back(it);
                 }
             }
         }
@@ -258,21 +289,18 @@ int build_plan(const uint32_t* flat, size_t n_flat, const uint32_t* off, const u
             return (x.tok_end - x.tok_begin) > (y.tok_end - y.tok_begin);
         });
         p.n_items = (uint32_t)items.size();
-        p.n_merge = (uint32_t)merges.size();
         p.off_items = flat_bytes;
-        p.off_merge = p.off_items + items.size() * sizeof(DecodeWorkItem);
-        const size_t total = p.off_merge + merges.size() * sizeof(MergeEntry);
+        const size_t total = p.off_items + items.size() * sizeof(DecodeWorkItem);
         MetaSlot& s = g.plan_slots[g.plan_next];
         if (!slot_reserve(s, std::max<size_t>(total, 16))) return 0;
         char* h = static_cast<char*>(s.host);
         if (n_flat) std::memcpy(h, flat, n_flat * 4);
         if (!items.empty()) std::memcpy(h + p.off_items, items.data(), items.size() * sizeof(DecodeWorkItem));
-        if (!merges.empty()) std::memcpy(h + p.off_merge, merges.data(), merges.size() * sizeof(MergeEntry));
         if (!slot_upload(s, std::max<size_t>(total, 16))) return 0;
     } else {
         p.hpw = 0;
+        p.nw = 0;
         p.n_items = (uint32_t)(B * H);
-        p.n_merge = 0;
         p.off_ptoff = flat_bytes;
         p.off_limits = p.off_ptoff + align_up(B * 4, 16);
         const size_t total = p.off_limits + align_up(B * 4, 16);
@@ -290,44 +318,50 @@ int build_plan(const uint32_t* flat, size_t n_flat, const uint32_t* off, const u
     return 1;
 }
 
-int ensure_partials(size_t n_part, int hpw, size_t D) {
-    const size_t need_o = n_part * (size_t)hpw * D;
-    const size_t need_ml = n_part * (size_t)hpw;
-    if (need_o > g.part_o_cap || need_ml > g.part_ml_cap) {
+int ensure_partials(size_t n_part, size_t G, size_t D, size_t nw) {
+    const size_t need_o = n_part * G * D;
+    const size_t need_ml = n_part * G * 2;
+    const size_t need_c = n_part * nw;
+    if (need_o > g.part_o_cap || need_ml > g.part_ml_cap || need_c > g.counters_cap) {
         HIP_OK(hipStreamSynchronize(g.stream));
         if (g.part_o) HIP_OK(hipFree(g.part_o));
         if (g.part_ml) HIP_OK(hipFree(g.part_ml));
+        if (g.counters) HIP_OK(hipFree(g.counters));
         g.part_o = nullptr;
         g.part_ml = nullptr;
-        g.part_o_cap = g.part_ml_cap = 0;
+        g.counters = nullptr;
+        g.part_o_cap = g.part_ml_cap = g.counters_cap = 0;
         const size_t cap_o = std::max<size_t>(need_o * 2, 1 << 20);
         const size_t cap_ml = std::max<size_t>(need_ml * 2, 1 << 14);
+        const size_t cap_c = std::max<size_t>(need_c * 2, 1 << 14);
         HIP_OK(hipMalloc(reinterpret_cast<void**>(&g.part_o), cap_o * sizeof(float)));
-        HIP_OK(hipMalloc(reinterpret_cast<void**>(&g.part_ml), cap_ml * sizeof(float2)));
+        HIP_OK(hipMalloc(reinterpret_cast<void**>(&g.part_ml), cap_ml * sizeof(float)));
+        HIP_OK(hipMalloc(reinterpret_cast<void**>(&g.counters), cap_c * sizeof(uint32_t)));
+        // Arrival counters start at zero; the last arriver of every group puts its counter
+        // back to zero, so they stay zero between launches.
+        HIP_OK(hipMemsetAsync(g.counters, 0, cap_c * sizeof(uint32_t), g.stream));
         g.part_o_cap = cap_o;
         g.part_ml_cap = cap_ml;
+        g.counters_cap = cap_c;
     }
     return 1;
 }
 
-template <int D>
-void launch_fast(int hpw, const DecodeArgs& a) {
-    const dim3 grid(a.n_items), block(64);
-    switch (hpw) {
-        case 8: hipLaunchKernelGGL((paged_decode_fast_kernel<D, 8>), grid, block, 0, g.stream, a); break;
-        case 4: hipLaunchKernelGGL((paged_decode_fast_kernel<D, 4>), grid, block, 0, g.stream, a); break;
-        case 2: hipLaunchKernelGGL((paged_decode_fast_kernel<D, 2>), grid, block, 0, g.stream, a); break;
-        default: hipLaunchKernelGGL((paged_decode_fast_kernel<D, 1>), grid, block, 0, g.stream, a); break;
+bool launch_fast(size_t D, int hpw, int nw, int ns, const DecodeArgs& a) {
+    const bool pv16 = g.opt_pv_fp16 != 0;
+    if (D == 64) {
+        switch (hpw) {
+            case 8: return launch_decode_fast_64_8(nw, ns, pv16, a, g.stream);
+            case 4: return launch_decode_fast_64_4(nw, ns, pv16, a, g.stream);
+            case 2: return launch_decode_fast_64_2(nw, ns, pv16, a, g.stream);
+            default: return launch_decode_fast_64_1(nw, ns, pv16, a, g.stream);
+        }
     }
-}
-
-void launch_merge(int hpw, uint32_t n_merge, const MergeEntry* e, float* o, uint32_t H, uint32_t D) {
-    const dim3 grid(n_merge, (unsigned)hpw), block(D <= 64 ? 64 : 128);
     switch (hpw) {
-        case 8: hipLaunchKernelGGL((paged_decode_merge_kernel<8>), grid, block, 0, g.stream, e, g.part_o, g.part_ml, o, H, D); break;
-        case 4: hipLaunchKernelGGL((paged_decode_merge_kernel<4>), grid, block, 0, g.stream, e, g.part_o, g.part_ml, o, H, D); break;
-        case 2: hipLaunchKernelGGL((paged_decode_merge_kernel<2>), grid, block, 0, g.stream, e, g.part_o, g.part_ml, o, H, D); break;
-        default: hipLaunchKernelGGL((paged_decode_merge_kernel<1>), grid, block, 0, g.stream, e, g.part_o, g.part_ml, o, H, D); break;
+        case 8: return launch_decode_fast_128_8(nw, ns, pv16, a, g.stream);
+        case 4: return launch_decode_fast_128_4(nw, ns, pv16, a, g.stream);
+        case 2: return launch_decode_fast_128_2(nw, ns, pv16, a, g.stream);
+        default: return launch_decode_fast_128_1(nw, ns, pv16, a, g.stream);
     }
 }
 
@@ -491,7 +525,8 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
     g.last_launches = 0;
     g.last_items = (int)p.n_items;
     if (p.fast) {
-        if (p.n_part && !ensure_partials(p.n_part, p.hpw, head_dim)) return 0;
+        if (p.n_part && !ensure_partials(p.n_part, num_heads / kv_heads, head_dim, (size_t)p.nw))
+            return 0;
         DecodeArgs a;
         a.q = static_cast<const float*>(q);
         a.k_pages = static_cast<const uint4*>(k_pages);
@@ -501,18 +536,14 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
         a.items = reinterpret_cast<const DecodeWorkItem*>(dev + p.off_items);
         a.part_o = g.part_o;
         a.part_ml = g.part_ml;
+        a.counters = g.counters;
         a.num_heads = (uint32_t)num_heads;
         a.kv_heads = (uint32_t)kv_heads;
         a.page_size = (uint32_t)page_size_tokens;
         a.n_items = p.n_items;
         a.scale_log2e = scale_log2e;
-        if (head_dim == 64) launch_fast<64>(p.hpw, a); else launch_fast<128>(p.hpw, a);
+        if (!launch_fast(head_dim, p.hpw, p.nw, p.ns, a)) return fail("decode: kernel variant not built");
         ++g.last_launches;
-        if (p.n_merge) {
-            launch_merge(p.hpw, p.n_merge, reinterpret_cast<const MergeEntry*>(dev + p.off_merge),
-                         a.o, a.num_heads, (uint32_t)head_dim);
-            ++g.last_launches;
-        }
     } else {
         GenericArgs a;
         a.q = static_cast<const float*>(q);
@@ -785,6 +816,17 @@ int mlc_hip_set_option(const char* name, long value) {
     if (!name) return 0;
     if (!std::strcmp(name, "decode_target_items")) { g.opt_target_items = value; return 1; }
     if (!std::strcmp(name, "decode_force_generic")) { g.opt_force_generic = value; return 1; }
+    if (!std::strcmp(name, "decode_pv_fp16")) { g.opt_pv_fp16 = value ? 1 : 0; return 1; }
+    if (!std::strcmp(name, "decode_tile_rows")) {
+        if (value != 1 && value != 2 && value != 4) return 0;
+        g.opt_tile_rows = value;
+        return 1;
+    }
+    if (!std::strcmp(name, "decode_heads_per_wave")) {
+        if (value != 1 && value != 2 && value != 4 && value != 8) return 0;
+        g.opt_hpw_max = value;
+        return 1;
+    }
     return 0;
 }
 

@@ -4,36 +4,38 @@
 // (compiler/runtime/metal_runtime.mm:2216-2335): for each (request, query head)
 //   O = softmax(q . K^T / sqrt(D), causal: kv_pos <= q_pos) . V
 // with K/V rows read through the request's page table from fp16 pages laid out
-// [page][slot][kv_head][dim], fp32 arithmetic and fp32 output.
+// [page][slot][kv_head][dim], fp32 accumulation and fp32 output.
 //
 // Layout of the work: the host flattens the batch into WORK ITEMS
-// (request, kv head, head group, token range) of roughly equal length -- split-K
-// over pages -- and launches one 64-lane wavefront per item.  All query heads
-// that share the KV head (GQA) are processed by the same wave, so every K/V byte
-// is fetched from HBM once.  Items that cover a whole request write O directly;
-// split requests write un-normalised (o, m, l) partials that a small second
-// kernel merges.
+// (request, kv head, token range) of roughly equal length -- split-K over pages --
+// and launches one workgroup per item.  A workgroup has NW x NS wavefronts: the
+// GQA group of the KV head is spread over NW waves (HPW query heads each, so
+// every K/V byte is fetched from HBM once and re-read from the CU's vector cache
+// by the other head waves), and the item's tiles are dealt round-robin to NS
+// wave rows.  Partial softmax states of the NS rows are merged through LDS; an
+// item that covers its whole request writes O directly, split requests publish
+// (o, m, l) partials and the last workgroup to arrive merges them.
 //
-// Lane layout of the fast kernel (D = 64 or 128):
+// Lane layout (D = 64 or 128):
 //   a K (or V) row of one KV head is D halves = D/8 16-byte chunks; lane
 //   (r, c) = (lane / CPR, lane % CPR), CPR = D/8, loads chunk c of row r of a
 //   "row group" of RPI = 64/CPR consecutive tokens, so one global_load_dwordx4
 //   per wave reads RPI whole rows, fully coalesced.  A tile is 8 row groups
 //   (64 tokens for D=64, 32 for D=128).
-//   QK: every lane forms the partial dot over its 8 dims for HPW heads x 8 row
-//   groups, then a 3-step reduce-scatter over the 8 c-lanes (DPP half-mirror,
-//   quad xor 2, quad xor 1 fused into v_add_f32) leaves lane (r, c) holding the
-//   complete scores of ONE token for all HPW heads.  To keep that exchange free
-//   of selects, register j' of lane c holds row group j' ^ g(c), g(c) = c ^
-//   ((c & 4) ? 3 : 0): the swizzle is applied to the load address, which costs
-//   nothing.
+//   QK: every lane forms the partial dot over its 8 dims for 8 row groups, then a
+//   3-step reduce-scatter over the 8 c-lanes (DPP half-mirror, quad xor 2, quad
+//   xor 1 fused into v_add_f32) leaves lane (r, c) holding the complete scores of
+//   ONE token for all HPW heads.  To keep that exchange free of selects, register
+//   j' of lane c holds row group j' ^ g(c), g(c) = c ^ ((c & 4) ? 3 : 0): the
+//   swizzle is applied to the load address, which costs nothing.
 //   Softmax: exp2 with log2(e)/sqrt(D) folded into q; the running reference
-//   maximum is kept per r-set (the 8 tokens x 8 tiles a row of lanes owns) and
-//   only raised when a tile exceeds it by more than 2^8 (exact math, any
-//   reference works; this removes almost all accumulator rescales).
-//   PV: p is gathered back over the same 8 lanes (7 DPP moves per head) and
-//   applied to the V rows held in the same (r, c) layout; accumulators are
-//   [HPW][8 dims] per lane, reduced over r once, at the end of the item.
+//   maximum is kept per r-set (the tokens a row of lanes owns) and only raised
+//   when a tile exceeds it by more than 2^8 (exact math, any reference works;
+//   this removes almost all accumulator rescales).
+//   PV: weights are rounded to fp16 (and the normaliser is summed from the
+//   rounded values), gathered back over the same 8 lanes with DPP moves and
+//   applied with v_dot2_f32_f16 to V rows held in the same (r, c) layout;
+//   accumulators are fp32 [HPW][8 dims] per lane, reduced over r once per item.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -42,16 +44,19 @@
 namespace mlc_hip {
 
 struct DecodeWorkItem {
-    uint32_t req;        // request index
-    uint32_t head0;      // first query head handled by this wave
-    uint32_t kv_head;    // KV head those query heads read
-    uint32_t pt_base;    // offset of the request's page ids in page_tables_flat
-    uint32_t tok_begin;  // first kv position (multiple of the tile size)
-    uint32_t tok_end;    // one past the last visible kv position of this item
-    uint32_t part_idx;   // partial slot, or kNoPartial to write O directly
+    uint32_t req;         // request index
+    uint32_t kv_head;     // KV head; the workgroup's waves cover its query-head group
+    uint32_t pt_base;     // offset of the request's page ids in page_tables_flat
+    uint32_t tok_begin;   // first kv position (multiple of the tile size)
+    uint32_t tok_end;     // one past the last visible kv position of this item
+    uint32_t part_first;  // first partial slot of this (request, kv head), or kNoPartial
+    uint32_t split;       // this item's split index | number of splits << 16
+    uint32_t first_pages[4];  // page id of the first tile of each tile row (saves a dependent load)
     uint32_t pad;
 };
+static_assert(sizeof(DecodeWorkItem) == 48, "work items are uploaded as raw bytes");
 static constexpr uint32_t kNoPartial = 0xFFFFFFFFu;
+static constexpr uint32_t kMaxSplits = 64;  // partial states merged by one wave pass
 
 struct DecodeArgs {
     const float* q;             // [B][H][D]
@@ -60,8 +65,9 @@ struct DecodeArgs {
     float* o;                   // [B][H][D]
     const uint32_t* pt_flat;    // device copy of page_tables_flat
     const DecodeWorkItem* items;
-    float* part_o;              // [n_part][HPW][D] un-normalised partial outputs
-    float2* part_ml;            // [n_part][HPW]    (m in log2 units, l)
+    float* part_o;              // [n_part][G][D] un-normalised partial outputs
+    float* part_ml;             // [n_part][G][2] (m in log2 units, l)
+    uint32_t* counters;         // [n_part][NW] arrival counters, zero between launches
     uint32_t num_heads;
     uint32_t kv_heads;
     uint32_t page_size;         // tokens per page
@@ -70,6 +76,7 @@ struct DecodeArgs {
 };
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 
 // DPP controls (GFX9 encoding)
 static constexpr int kDppQuadXor1 = 0xB1;     // quad_perm:[1,0,3,2]
@@ -82,37 +89,105 @@ template <int CTRL>
 __device__ __forceinline__ float dpp_f(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
 }
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
+
+// Device-scope accesses: the store is written through to memory, the load bypasses the
+// (per-XCD, mutually non-coherent) L2 caches.
+__device__ __forceinline__ void st_dev(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float ld_dev(const float* p) {
+    return __hip_atomic_load(const_cast<float*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// plain maximum; the file is compiled with -fno-honor-nans so no NaN-quieting moves are added
+__device__ __forceinline__ float max_nn(float a, float b) { return __builtin_fmaxf(a, b); }
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) v = max_nn(v, __shfl_xor(v, off));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) v += __shfl_xor(v, off);
+    return v;
+}
 
 // -inf substitute for running maxima: finite, so (m - m) and exp2(-inf - m) stay NaN-free.
 static constexpr float kNegBig = -1.0e30f;
 // A tile may exceed the running reference by 2^kLazyTau before accumulators are rescaled.
 static constexpr float kLazyTau = 8.0f;
 
-template <int D, int HPW>
-__global__ __launch_bounds__(64) void paged_decode_fast_kernel(const DecodeArgs a) {
+template <int D, int HPW, int NW, int NS, bool PV16>
+__global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const DecodeArgs a) {
     static_assert(D == 64 || D == 128, "fast path covers head_dim 64 and 128");
-    constexpr int CPR = D / 8;       // 16-byte chunks per row
-    constexpr int RPI = 64 / CPR;    // rows fetched by one wave-wide load
-    constexpr int TT = 8 * RPI;      // tokens per tile
+    constexpr int CPR = D / 8;         // 16-byte chunks per row
+    constexpr int RPI = 64 / CPR;      // rows fetched by one wave-wide load
+    constexpr int TT = 8 * RPI;        // tokens per tile
     constexpr int OPL = HPW * D / 64;  // outputs per lane in the epilogue
+    constexpr int HPK = D / 64;        // epilogue registers per head: idx = k*64+lane -> h = k/HPK
+    constexpr int G = HPW * NW;        // query heads per KV head
+    constexpr int NWAVES = NW * NS;
 
-    __shared__ float s_acc[RPI * HPW * D];
+    __shared__ float s_acc_all[NWAVES][RPI * HPW * D];
+    __shared__ float s_ml[NWAVES][HPW][2];
 
     const uint32_t item_idx = blockIdx.x;
     if (item_idx >= a.n_items) return;
     const DecodeWorkItem it = a.items[item_idx];
-    const int lane = threadIdx.x;
+    const int wave = threadIdx.x / 64;
+    const int lane = threadIdx.x % 64;
+    const int hg = wave % NW;   // head group of this wave
+    const int sub = wave / NW;  // tile row of this wave
+    float* s_acc = s_acc_all[wave];
     const int c = lane % CPR;
     const int r = lane / CPR;
     const int c7 = c & 7;
     const int gsw = c7 ^ ((c7 & 4) ? 3 : 0);  // row-group swizzle g(c)
+    const uint32_t head0 = it.kv_head * G + hg * HPW;
+
+    const uint32_t row_u4 = a.kv_heads * CPR;  // 16-byte chunks per token row (all KV heads)
+    const uint32_t lane_u4 = it.kv_head * CPR + c;
+
+    // The 8 rows this lane reads in a tile; rows past the visible end are clamped onto the
+    // last visible row (in bounds, masked out of the softmax below).
+    auto load_tile = [&](const uint4* pages, uint32_t page_id, uint32_t tile_start,
+                         uint4 (&reg)[8]) {
+        const uint32_t slot0 = tile_start % a.page_size;
+        const uint32_t last = it.tok_end - 1u - tile_start;  // last visible row of the tile
+        const uint4* base = pages + ((size_t)page_id * a.page_size + slot0) * row_u4 + lane_u4;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            uint32_t t = (uint32_t)((j ^ gsw) * RPI + r);
+            t = t < last ? t : last;
+            reg[j] = base[(size_t)t * row_u4];
+        }
+    };
+    auto page_of = [&](uint32_t tile_start) {
+        return a.pt_flat[it.pt_base + tile_start / a.page_size];
+    };
+
+    constexpr uint32_t STEP = TT * NS;  // this wave's tiles are STEP tokens apart
+    const uint32_t my_begin = it.tok_begin + (uint32_t)sub * TT;
+    uint4 kreg[8], vreg[8];
+    if (my_begin < it.tok_end) {
+        const uint32_t pg = it.first_pages[sub];
+        load_tile(a.k_pages, pg, my_begin, kreg);
+        load_tile(a.v_pages, pg, my_begin, vreg);
+    }
+    uint32_t next_page = 0;
+    if (my_begin + STEP < it.tok_end) next_page = page_of(my_begin + STEP);
 
     // q for this wave's heads, dims c*8 .. c*8+7, pre-scaled.
     float qv[HPW][8];
     {
-        const float* qbase = a.q + ((size_t)it.req * a.num_heads + it.head0) * D + c * 8;
+        const float* qbase = a.q + ((size_t)it.req * a.num_heads + head0) * D + c * 8;
 #pragma unroll
         for (int h = 0; h < HPW; ++h) {
             const float4 lo = *reinterpret_cast<const float4*>(qbase + h * D);
@@ -134,34 +209,11 @@ __global__ __launch_bounds__(64) void paged_decode_fast_kernel(const DecodeArgs 
         for (int i = 0; i < 8; ++i) acc[h][i] = 0.f;
     }
 
-    const uint32_t row_u4 = a.kv_heads * CPR;  // 16-byte chunks per token row (all KV heads)
-    const uint32_t lane_u4 = it.kv_head * CPR + c;
-
-    // Addresses of the 8 rows this lane reads in a tile; rows past the visible end are
-    // clamped onto the last visible row (in bounds, masked out of the softmax below).
-    auto load_tile = [&](const uint4* pages, uint32_t tile_start, uint4 (&reg)[8]) {
-        const uint32_t page_idx = tile_start / a.page_size;
-        const uint32_t slot0 = tile_start - page_idx * a.page_size;
-        const uint32_t page_id = a.pt_flat[it.pt_base + page_idx];
-        const uint32_t last = it.tok_end - 1u - tile_start;  // last visible row of the tile
-        const uint4* base = pages + ((size_t)page_id * a.page_size + slot0) * row_u4 + lane_u4;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            uint32_t t = (uint32_t)((j ^ gsw) * RPI + r);
-            t = t < last ? t : last;
-            reg[j] = base[(size_t)t * row_u4];
-        }
-    };
-
-    uint4 kreg[8], vreg[8];
-    if (it.tok_begin < it.tok_end) {
-        load_tile(a.k_pages, it.tok_begin, kreg);
-        load_tile(a.v_pages, it.tok_begin, vreg);
-    }
-
-    for (uint32_t tile_start = it.tok_begin; tile_start < it.tok_end; tile_start += TT) {
-        const uint32_t next = tile_start + TT;
+    for (uint32_t tile_start = my_begin; tile_start < it.tok_end; tile_start += STEP) {
+        const uint32_t next = tile_start + STEP;
         const bool has_next = next < it.tok_end;
+        const uint32_t page_n = next_page;
+        if (next + STEP < it.tok_end) next_page = page_of(next + STEP);
 
         // ---- QK: per head, partial dots over this lane's 8 dims for the 8 row groups,
         // then a reduce-scatter over the 8 c-lanes (lane keeps row group g(c)).
@@ -185,7 +237,7 @@ __global__ __launch_bounds__(64) void paged_decode_fast_kernel(const DecodeArgs 
             if (CPR == 16) s += dpp_f<kDppRowRor8>(s);
             sc[h] = s;
         }
-        if (has_next) load_tile(a.k_pages, next, kreg);
+        if (has_next) load_tile(a.k_pages, page_n, next, kreg);
 
         // ---- mask, tile maximum over the r-set, lazy reference update
         const uint32_t my_tok = tile_start + (uint32_t)(gsw * RPI + r);
@@ -196,17 +248,17 @@ __global__ __launch_bounds__(64) void paged_decode_fast_kernel(const DecodeArgs 
         for (int h = 0; h < HPW; ++h) {
             sc[h] = visible ? sc[h] : -INFINITY;
             float m = sc[h];
-            m = fmaxf(m, dpp_f<kDppQuadXor1>(m));
-            m = fmaxf(m, dpp_f<kDppQuadXor2>(m));
-            m = fmaxf(m, dpp_f<kDppHalfMirror>(m));
-            if (CPR == 16) m = fmaxf(m, dpp_f<kDppRowRor8>(m));
+            m = max_nn(m, dpp_f<kDppQuadXor1>(m));
+            m = max_nn(m, dpp_f<kDppQuadXor2>(m));
+            m = max_nn(m, dpp_f<kDppHalfMirror>(m));
+            if (CPR == 16) m = max_nn(m, dpp_f<kDppRowRor8>(m));
             tmax[h] = m;
             raise |= (m > m_ref[h] + kLazyTau);
         }
         if (__any(raise)) {
 #pragma unroll
             for (int h = 0; h < HPW; ++h) {
-                const float m_new = fmaxf(m_ref[h], tmax[h]);
+                const float m_new = max_nn(m_ref[h], tmax[h]);
                 const float alpha = fast_exp2(m_ref[h] - m_new);
                 m_ref[h] = m_new;
                 l_sum[h] *= alpha;
@@ -214,200 +266,274 @@ __global__ __launch_bounds__(64) void paged_decode_fast_kernel(const DecodeArgs 
                 for (int i = 0; i < 8; ++i) acc[h][i] *= alpha;
             }
         }
-        float p[HPW];
-#pragma unroll
-        for (int h = 0; h < HPW; ++h) {
-            p[h] = fast_exp2(sc[h] - m_ref[h]);
-            l_sum[h] += p[h];
-        }
 
-        // ---- PV: register j of this lane holds the V row whose weight lives in the
-        // lane at swizzle distance j; fetch it with DPP moves.
+        if constexpr (PV16) {
+            // ---- weights rounded to fp16 (the sum l uses the rounded values, so the result
+            // is an exactly normalised average with weights perturbed by <= 2^-11), packed
+            // two heads to a register.
+            uint32_t pp[(HPW + 1) / 2];
 #pragma unroll
-        for (int h = 0; h < HPW; ++h) {
-            float pj[8];
-            pj[0] = p[h];
-            pj[1] = dpp_f<kDppQuadXor1>(p[h]);
-            pj[2] = dpp_f<kDppQuadXor2>(p[h]);
-            pj[3] = dpp_f<kDppQuadXor3>(p[h]);
-            pj[4] = dpp_f<kDppHalfMirror>(p[h]);
-            pj[5] = dpp_f<kDppQuadXor1>(pj[4]);
-            pj[6] = dpp_f<kDppQuadXor2>(pj[4]);
-            pj[7] = dpp_f<kDppQuadXor3>(pj[4]);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const half8_t vh = __builtin_bit_cast(half8_t, vreg[j]);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) acc[h][i] = fmaf(pj[j], (float)vh[i], acc[h][i]);
+            for (int h2 = 0; h2 < (HPW + 1) / 2; ++h2) {
+                const _Float16 p0 = (_Float16)fast_exp2(sc[2 * h2] - m_ref[2 * h2]);
+                l_sum[2 * h2] += (float)p0;
+                _Float16 p1 = (_Float16)0.f;
+                if (2 * h2 + 1 < HPW) {
+                    p1 = (_Float16)fast_exp2(sc[2 * h2 + 1] - m_ref[2 * h2 + 1]);
+                    l_sum[2 * h2 + 1] += (float)p1;
+                }
+                half2_t pk = {p0, p1};
+                pp[h2] = __builtin_bit_cast(uint32_t, pk);
             }
+            // ---- PV with v_dot2_f32_f16: register j of this lane holds the V row whose
+            // weight lives in the lane at swizzle distance j.  V rows are paired (j, j+1)
+            // per dim, the weights of the same two rows are paired per head.
+            uint32_t vp[4][8];  // [row pair][dim] = (v[2k][i], v[2k+1][i])
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t* va = reinterpret_cast<const uint32_t*>(&vreg[2 * k]);
+                const uint32_t* vb = reinterpret_cast<const uint32_t*>(&vreg[2 * k + 1]);
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    // dims 2w (low halves) and 2w+1 (high halves) of both rows
+                    vp[k][2 * w] = __builtin_amdgcn_perm(vb[w], va[w], 0x05040100u);
+                    vp[k][2 * w + 1] = __builtin_amdgcn_perm(vb[w], va[w], 0x07060302u);
+                }
+            }
+            if (has_next) load_tile(a.v_pages, page_n, next, vreg);  // vreg is dead once packed
+#pragma unroll
+            for (int h2 = 0; h2 < (HPW + 1) / 2; ++h2) {
+                uint32_t g8[8];
+                g8[0] = pp[h2];
+                g8[1] = dpp_u<kDppQuadXor1>(pp[h2]);
+                g8[2] = dpp_u<kDppQuadXor2>(pp[h2]);
+                g8[3] = dpp_u<kDppQuadXor3>(pp[h2]);
+                g8[4] = dpp_u<kDppHalfMirror>(pp[h2]);
+                g8[5] = dpp_u<kDppQuadXor1>(g8[4]);
+                g8[6] = dpp_u<kDppQuadXor2>(g8[4]);
+                g8[7] = dpp_u<kDppQuadXor3>(g8[4]);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    // (p[h][row 2k], p[h][row 2k+1]) for the two heads packed in g8
+                    const uint32_t w0 = __builtin_amdgcn_perm(g8[2 * k + 1], g8[2 * k], 0x05040100u);
+                    const half2_t pw0 = __builtin_bit_cast(half2_t, w0);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i)
+                        acc[2 * h2][i] = __builtin_amdgcn_fdot2(
+                            __builtin_bit_cast(half2_t, vp[k][i]), pw0, acc[2 * h2][i], false);
+                    if (2 * h2 + 1 < HPW) {
+                        const uint32_t w1 =
+                            __builtin_amdgcn_perm(g8[2 * k + 1], g8[2 * k], 0x07060302u);
+                        const half2_t pw1 = __builtin_bit_cast(half2_t, w1);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i)
+                            acc[2 * h2 + 1][i] = __builtin_amdgcn_fdot2(
+                                __builtin_bit_cast(half2_t, vp[k][i]), pw1, acc[2 * h2 + 1][i],
+                                false);
+                    }
+                }
+            }
+        } else {
+            // ---- exact fp32 weights: gather them over the 8 lanes, fp16 V widened in the FMA
+            float p[HPW];
+#pragma unroll
+            for (int h = 0; h < HPW; ++h) {
+                p[h] = fast_exp2(sc[h] - m_ref[h]);
+                l_sum[h] += p[h];
+            }
+#pragma unroll
+            for (int h = 0; h < HPW; ++h) {
+                float pj[8];
+                pj[0] = p[h];
+                pj[1] = dpp_f<kDppQuadXor1>(p[h]);
+                pj[2] = dpp_f<kDppQuadXor2>(p[h]);
+                pj[3] = dpp_f<kDppQuadXor3>(p[h]);
+                pj[4] = dpp_f<kDppHalfMirror>(p[h]);
+                pj[5] = dpp_f<kDppQuadXor1>(pj[4]);
+                pj[6] = dpp_f<kDppQuadXor2>(pj[4]);
+                pj[7] = dpp_f<kDppQuadXor3>(pj[4]);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const half8_t vh = __builtin_bit_cast(half8_t, vreg[j]);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) acc[h][i] = fmaf(pj[j], (float)vh[i], acc[h][i]);
+                }
+            }
+            if (has_next) load_tile(a.v_pages, page_n, next, vreg);
         }
-        if (has_next) load_tile(a.v_pages, next, vreg);
     }
 
-    // ---- epilogue: bring the RPI r-sets onto one reference, sum over r through LDS
+    // ---- epilogue 1: bring the RPI r-sets of this wave onto one reference, sum over r
+    // through this wave's LDS region.
     float m_all[HPW], l_all[HPW];
 #pragma unroll
     for (int h = 0; h < HPW; ++h) {
         float m = m_ref[h];
 #pragma unroll
-        for (int off = CPR; off < 64; off <<= 1) m = fmaxf(m, __shfl_xor(m, off));
+        for (int off = CPR; off < 64; off <<= 1) m = max_nn(m, __shfl_xor(m, off));
         m_all[h] = m;
         const float w = fast_exp2(m_ref[h] - m);
         // with CPR == 16 every token's weight sits in two lanes (c and c^8): count it once
-        float l = (CPR == 16 && (c & 8)) ? 0.f : l_sum[h] * w;
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) l += __shfl_xor(l, off);
-        l_all[h] = l;
+        l_all[h] = wave_sum((CPR == 16 && (c & 8)) ? 0.f : l_sum[h] * w);
         float4* dst = reinterpret_cast<float4*>(&s_acc[((r * HPW + h) * CPR + c) * 8]);
         dst[0] = make_float4(acc[h][0] * w, acc[h][1] * w, acc[h][2] * w, acc[h][3] * w);
         dst[1] = make_float4(acc[h][4] * w, acc[h][5] * w, acc[h][6] * w, acc[h][7] * w);
     }
-    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
+    // Output k of this lane is element idx = k*64 + lane of [HPW][D]: head k / HPK.
+    float o_un[OPL];
 #pragma unroll
     for (int k = 0; k < OPL; ++k) {
-        const int idx = k * 64 + lane;  // index into [HPW][D]
-        const int h = idx / D;
-        const int d = idx % D;
+        const int idx = k * 64 + lane;
         float sum = 0.f;
 #pragma unroll
-        for (int rr = 0; rr < RPI; ++rr) sum += s_acc[(rr * HPW + h) * D + d];
-        // m_all[h], l_all[h] for a run-time h: select without indexing registers dynamically
-        float mh = m_all[0], l = l_all[0];
-#pragma unroll
-        for (int hh = 1; hh < HPW; ++hh) {
-            mh = (h == hh) ? m_all[hh] : mh;
-            l = (h == hh) ? l_all[hh] : l;
-        }
-        if (it.part_idx == kNoPartial) {
-            const float inv = l > 0.f ? 1.0f / l : 0.f;
-            a.o[((size_t)it.req * a.num_heads + it.head0 + h) * D + d] = sum * inv;
-        } else {
-            a.part_o[((size_t)it.part_idx * HPW + h) * D + d] = sum;
-            if (d == 0) a.part_ml[(size_t)it.part_idx * HPW + h] = make_float2(mh, l);
-        }
+        for (int rr = 0; rr < RPI; ++rr) sum += s_acc[rr * HPW * D + idx];
+        o_un[k] = sum;
     }
-}
 
-// Merges the split-K partials of one (request, head group): grid = number of
-// merge entries, block = D threads... one thread per output dim, loop over heads.
-struct MergeEntry {
-    uint32_t req;
-    uint32_t head0;
-    uint32_t first_part;
-    uint32_t n_parts;
-};
-
-template <int HPW>
-__global__ void paged_decode_merge_kernel(const MergeEntry* entries, const float* part_o,
-                                          const float2* part_ml, float* o, uint32_t num_heads,
-                                          uint32_t head_dim) {
-    const MergeEntry e = entries[blockIdx.x];
-    const uint32_t h = blockIdx.y;
-    const float2* ml = part_ml + (size_t)e.first_part * HPW + h;
-    float m = kNegBig;
-    for (uint32_t s = 0; s < e.n_parts; ++s) m = fmaxf(m, ml[(size_t)s * HPW].x);
-    float l = 0.f;
-    for (uint32_t s = 0; s < e.n_parts; ++s) {
-        const float2 v = ml[(size_t)s * HPW];
-        l += v.y * fast_exp2(v.x - m);
-    }
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
-    for (uint32_t d = threadIdx.x; d < head_dim; d += blockDim.x) {
-        float acc = 0.f;
-        for (uint32_t s = 0; s < e.n_parts; ++s) {
-            const float w = fast_exp2(ml[(size_t)s * HPW].x - m);
-            acc += w * part_o[(((size_t)e.first_part + s) * HPW + h) * head_dim + d];
+    // ---- epilogue 2: merge the NS tile rows of the workgroup through LDS
+    if constexpr (NS > 1) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int k = 0; k < OPL; ++k) s_acc[k * 64 + lane] = o_un[k];
+        if (lane < HPW) {
+            // m_all / l_all are wave-uniform: pick this lane's head without dynamic indexing
+            float mh = m_all[0], lh = l_all[0];
+#pragma unroll
+            for (int hh = 1; hh < HPW; ++hh) {
+                mh = (lane == hh) ? m_all[hh] : mh;
+                lh = (lane == hh) ? l_all[hh] : lh;
+            }
+            s_ml[wave][lane][0] = mh;
+            s_ml[wave][lane][1] = lh;
         }
-        o[((size_t)e.req * num_heads + e.head0 + h) * head_dim + d] = acc * inv;
-    }
-}
-
-// Shape-agnostic kernel: any head_dim <= 256, any page size, any GQA ratio.  One
-// wave per (request, query head); lanes own tokens for QK and dims for PV.  Used
-// for the shapes the fast kernel does not cover (small pages, odd head sizes).
-struct GenericArgs {
-    const float* q;
-    const _Float16* k_pages;
-    const _Float16* v_pages;
-    float* o;
-    const uint32_t* pt_flat;
-    const uint32_t* pt_off;    // [B]
-    const uint32_t* limits;    // [B] visible kv positions (causal rule applied)
-    uint32_t num_heads;
-    uint32_t kv_heads;
-    uint32_t head_dim;
-    uint32_t page_size;
-    float scale_log2e;
-};
-
-__global__ __launch_bounds__(64) void paged_decode_generic_kernel(const GenericArgs a) {
-    const uint32_t req = blockIdx.x / a.num_heads;
-    const uint32_t head = blockIdx.x % a.num_heads;
-    const uint32_t kvh = (uint32_t)(((uint64_t)head * a.kv_heads) / a.num_heads);
-    const uint32_t D = a.head_dim;
-    const uint32_t limit = a.limits[req];
-    const uint32_t pt_base = a.pt_off[req];
-    const int lane = threadIdx.x;
-    __shared__ float s_q[256];
-    const float* qrow = a.q + ((size_t)req * a.num_heads + head) * D;
-    for (uint32_t d = lane; d < D; d += 64) s_q[d] = qrow[d] * a.scale_log2e;
-    __syncthreads();
-
-    constexpr int DPL = 4;  // dims per lane: covers head_dim <= 256
-    float oacc[DPL] = {0.f, 0.f, 0.f, 0.f};
-    float m = kNegBig, l = 0.f;
-    const size_t row_elems = (size_t)a.kv_heads * D;
-
-    for (uint32_t t0 = 0; t0 < limit; t0 += 64) {
-        const uint32_t pos = t0 + lane;
-        const bool visible = pos < limit;
-        size_t row = 0;
-        float s = -INFINITY;
-        if (visible) {
-            const uint32_t page_idx = pos / a.page_size;
-            const uint32_t slot = pos - page_idx * a.page_size;
-            const uint32_t page_id = a.pt_flat[pt_base + page_idx];
-            row = ((size_t)page_id * a.page_size + slot) * row_elems + (size_t)kvh * D;
-            const _Float16* kr = a.k_pages + row;
-            float dot = 0.f;
-            for (uint32_t d = 0; d < D; ++d) dot = fmaf(s_q[d], (float)kr[d], dot);
-            s = dot;
-        }
-        float tmax = s;
+        __syncthreads();
+        if (sub != 0) return;
 #pragma unroll
-        for (int off = 1; off < 64; off <<= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, off));
-        const float m_new = fmaxf(m, tmax);
-        const float alpha = fast_exp2(m - m_new);
-        const float p = fast_exp2(s - m_new);  // s = -inf -> 0
-        float psum = p;
+        for (int h = 0; h < HPW; ++h) {
+            float m = kNegBig;
 #pragma unroll
-        for (int off = 1; off < 64; off <<= 1) psum += __shfl_xor(psum, off);
-        l = l * alpha + psum;
-        m = m_new;
+            for (int s = 0; s < NS; ++s) m = max_nn(m, s_ml[s * NW + hg][h][0]);
+            float l = 0.f;
+            float w[NS];
 #pragma unroll
-        for (int k = 0; k < DPL; ++k) oacc[k] *= alpha;
-        const uint32_t n_here = (limit - t0) < 64u ? (limit - t0) : 64u;
-        const uint32_t row_lo = (uint32_t)(row & 0xFFFFFFFFu);
-        const uint32_t row_hi = (uint32_t)(row >> 32);
-        for (uint32_t t = 0; t < n_here; ++t) {
-            const float pt = __shfl(p, (int)t);
-            const size_t rt = ((size_t)__shfl((int)row_hi, (int)t) << 32) |
-                              (uint32_t)__shfl((int)row_lo, (int)t);
-            const _Float16* vr = a.v_pages + rt;
+            for (int s = 0; s < NS; ++s) {
+                w[s] = fast_exp2(s_ml[s * NW + hg][h][0] - m);
+                l += w[s] * s_ml[s * NW + hg][h][1];
+            }
+            m_all[h] = m;
+            l_all[h] = l;
 #pragma unroll
-            for (int k = 0; k < DPL; ++k) {
-                const uint32_t d = lane + 64u * k;
-                if (d < D) oacc[k] = fmaf(pt, (float)vr[d], oacc[k]);
+            for (int kk = 0; kk < HPK; ++kk) {
+                const int k = h * HPK + kk;
+                float sum = 0.f;
+#pragma unroll
+                for (int s = 0; s < NS; ++s) sum += w[s] * s_acc_all[s * NW + hg][k * 64 + lane];
+                o_un[k] = sum;
             }
         }
     }
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
-    float* orow = a.o + ((size_t)req * a.num_heads + head) * D;
+
+    if (it.part_first == kNoPartial) {
 #pragma unroll
-    for (int k = 0; k < DPL; ++k) {
-        const uint32_t d = lane + 64u * k;
-        if (d < D) orow[d] = oacc[k] * inv;
+        for (int k = 0; k < OPL; ++k) {
+            const float l = l_all[k / HPK];
+            const float inv = l > 0.f ? 1.0f / l : 0.f;
+            a.o[((size_t)it.req * a.num_heads + head0) * D + k * 64 + lane] = o_un[k] * inv;
+        }
+        return;
+    }
+
+    // ---- split request: publish this item's partial, the last arriver merges all of them.
+    // Partials are written and read with device-scope (write-through / cache-bypassing)
+    // accesses, so no L2 write-back or invalidate is needed around the arrival counter:
+    // waiting for the stores to complete before the counter is bumped is enough.
+    const uint32_t n_splits = it.split >> 16;
+    const uint32_t my_split = it.split & 0xFFFFu;
+    {
+        const size_t slot = (size_t)it.part_first + my_split;
+        float* po = a.part_o + (slot * G + hg * HPW) * D;
+        float* ml = a.part_ml + (slot * G + hg * HPW) * 2;
+#pragma unroll
+        for (int k = 0; k < OPL; ++k) st_dev(po + k * 64 + lane, o_un[k]);
+        if (lane < HPW) {
+            float mh = m_all[0], lh = l_all[0];
+#pragma unroll
+            for (int hh = 1; hh < HPW; ++hh) {
+                mh = (lane == hh) ? m_all[hh] : mh;
+                lh = (lane == hh) ? l_all[hh] : lh;
+            }
+            st_dev(ml + lane * 2, mh);
+            st_dev(ml + lane * 2 + 1, lh);
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // stores complete (vmcnt 0)
+    uint32_t ticket = 0;
+    uint32_t* counter = &a.counters[(size_t)it.part_first * NW + hg];
+    if (lane == 0)
+        ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    ticket = __shfl(ticket, 0);
+    if (ticket != n_splits - 1) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    if (lane == 0)  // ready for the next launch
+        __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+    // Lane s holds the (m, l) of split s for every head; all loads are issued before any
+    // is consumed, so the merge costs about one memory round trip.
+    const float* ml_base = a.part_ml + ((size_t)it.part_first * G + hg * HPW) * 2;
+    const float* po_base = a.part_o + ((size_t)it.part_first * G + hg * HPW) * D;
+    float ms[HPW], ls[HPW];
+#pragma unroll
+    for (int h = 0; h < HPW; ++h) {
+        ms[h] = kNegBig;
+        ls[h] = 0.f;
+        if ((uint32_t)lane < n_splits) {
+            ms[h] = ld_dev(ml_base + ((size_t)lane * G + h) * 2);
+            ls[h] = ld_dev(ml_base + ((size_t)lane * G + h) * 2 + 1);
+        }
+    }
+    constexpr int UNR = 8;
+    float acc_o[OPL];
+#pragma unroll
+    for (int k = 0; k < OPL; ++k) acc_o[k] = 0.f;
+    float wgt[HPW], l_fin[HPW];
+    bool have_w = false;
+    for (uint32_t s0 = 0; s0 < n_splits; s0 += UNR) {
+        float pv[UNR][OPL];
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+#pragma unroll
+            for (int k = 0; k < OPL; ++k) {
+                pv[u][k] = 0.f;
+                if (s0 + u < n_splits) pv[u][k] = ld_dev(po_base + (size_t)(s0 + u) * G * D + k * 64 + lane);
+            }
+        }
+        if (!have_w) {
+#pragma unroll
+            for (int h = 0; h < HPW; ++h) {
+                const float m = wave_max(ms[h]);
+                wgt[h] = fast_exp2(ms[h] - m);  // lanes >= n_splits: exp2(-1e30 - m) = 0
+                l_fin[h] = wave_sum(wgt[h] * ls[h]);
+            }
+            have_w = true;
+        }
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+            if (s0 + u < n_splits) {
+#pragma unroll
+                for (int k = 0; k < OPL; ++k)
+                    acc_o[k] += __shfl(wgt[k / HPK], (int)(s0 + u)) * pv[u][k];
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < OPL; ++k) {
+        const float l = l_fin[k / HPK];
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        a.o[((size_t)it.req * a.num_heads + head0) * D + k * 64 + lane] = acc_o[k] * inv;
     }
 }
 
