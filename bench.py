@@ -129,6 +129,28 @@ def main() -> int:
         k_bufs.append(kb)
         v_bufs.append(vb)
 
+    import ctypes as C
+    from mlcompiler_amd.build import BENCH_LIB_PATH
+    bl = C.CDLL(BENCH_LIB_PATH)   # native loop around the C ABI (no Python between launches)
+    u32p = C.POINTER(C.c_uint32)
+    meta = [np.ascontiguousarray(x, np.uint32) for x in
+            (c.page_tables_flat, c.page_table_offsets, c.seq_lens, c.q_positions)]
+    kp = (C.c_void_p * n_layers)(*k_bufs)
+    vp = (C.c_void_p * n_layers)(*v_bufs)
+
+    def native_loop(steps: int):
+        ms, wall_s = C.c_float(), C.c_double()
+        ok = bl.mlc_bench_decode_loop(
+            C.c_void_p(q_buf), kp, vp, C.c_size_t(n_layers), C.c_void_p(o_buf),
+            meta[0].ctypes.data_as(u32p), C.c_size_t(meta[0].size), meta[1].ctypes.data_as(u32p),
+            meta[2].ctypes.data_as(u32p), meta[3].ctypes.data_as(u32p), C.c_size_t(c.batch),
+            C.c_size_t(c.num_heads), C.c_size_t(c.kv_heads), C.c_size_t(c.head_dim),
+            C.c_size_t(c.page_size), C.c_int(int(c.apply_causal)), C.c_size_t(steps),
+            C.byref(ms), C.byref(wall_s))
+        if not ok:
+            raise RuntimeError("decode loop failed: " + exe.lastError())
+        return ms.value, wall_s.value
+
     def step(layer: int) -> None:
         ok = exe.encodePagedFlashAttention(q_buf, k_bufs[layer], v_bufs[layer], o_buf,
                                            c.page_tables_flat, c.page_table_offsets, c.seq_lens,
@@ -137,20 +159,13 @@ def main() -> int:
         if not ok:
             raise RuntimeError("encodePagedFlashAttention failed: " + exe.lastError())
 
-    exe.beginForwardPassCB()
-    for i in range(args.warmup):
-        step(i % n_layers)
-    assert exe.flushForwardPassCB(), exe.lastError()
+    if args.warmup:
+        native_loop(args.warmup)
 
-    # ---- timed region: exactly --steps steps, device idle on both sides
-    exe.beginForwardPassCB()
-    t0 = time.perf_counter()
-    exe.timerStart()
-    for i in range(args.steps):
-        step(i % n_layers)
-    ev_ms = exe.timerStopMs()                 # HIP events on the kernel's stream
-    assert exe.flushForwardPassCB(), exe.lastError()
-    wall = time.perf_counter() - t0
+    # ---- timed region: exactly --steps steps, device idle on both sides (the loop starts
+    # on an idle stream and returns after the stream has drained); HIP events bracket the
+    # same region on the kernels' stream.
+    ev_ms, wall = native_loop(args.steps)
     launches = exe.lastDecodeLaunches()
     items = exe.lastDecodeWorkItems()
 

@@ -158,10 +158,15 @@ float mlc_hip_timer_stop(void);
 int mlc_hip_last_decode_launches(void);
 int mlc_hip_last_decode_work_items(void);
 
-/* Tunables: "decode_target_items" (split-K work items aimed for per launch, 0 =
- * automatic), "decode_heads_per_wave" (1, 2, 4 or 8: the most query heads one
- * wavefront handles; the GQA group is spread over group/that many waves of a
- * workgroup), "decode_force_generic" (1 = always use the shape-agnostic kernel).
+/* Tunables (0 selects the automatic choice where noted):
+ *   "decode_target_items"   split-K work items aimed for per launch (0 = automatic)
+ *   "decode_heads_per_wave" 1, 2, 4 or 8: the most query heads one wavefront handles;
+ *                           the GQA group is spread over group/that many waves (0 = automatic)
+ *   "decode_tile_rows"      1 or 2: wave rows of a workgroup that share an item's tiles
+ *   "decode_buffers"        1 or 2 LDS staging buffers per workgroup (0 = automatic)
+ *   "decode_pv_fp16"        1 = softmax weights rounded to fp16 for the P.V product
+ *                           (v_dot2_f32_f16, fp32 accumulate), 0 = fp32 weights
+ *   "decode_force_generic"  1 = always use the shape-agnostic kernel
  * Returns 0 for an unknown name or value. */
 int mlc_hip_set_option(const char* name, long value);
 

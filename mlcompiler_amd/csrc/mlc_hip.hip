@@ -23,7 +23,7 @@
 
 namespace mlc_hip {
 // Defined in paged_decode_inst.hip, one object per (head_dim, heads-per-wave).
-#define MLC_DECL(d, h) bool launch_decode_fast_##d##_##h(int, int, bool, const DecodeArgs&, hipStream_t);
+#define MLC_DECL(d, h) bool launch_decode_fast_##d##_##h(int, int, int, bool, const DecodeArgs&, hipStream_t);
 MLC_DECL(64, 1) MLC_DECL(64, 2) MLC_DECL(64, 4) MLC_DECL(64, 8)
 MLC_DECL(128, 1) MLC_DECL(128, 2) MLC_DECL(128, 4) MLC_DECL(128, 8)
 #undef MLC_DECL
@@ -64,10 +64,10 @@ struct DecodePlan {
     std::vector<uint32_t> pt_flat, pt_off, seq_lens, q_pos;
     size_t B = 0, H = 0, Hkv = 0, D = 0, P = 0;
     int causal = 0;
-    long target_items = 0, force_generic = 0, hpw_max = 0, tile_rows = 0;
+    long target_items = 0, force_generic = 0, hpw_max = 0, tile_rows = 0, buffers = 0;
     // result
     bool fast = false;
-    int hpw = 0, nw = 0, ns = 0;
+    int hpw = 0, nw = 0, ns = 0, nbuf = 2;
     uint32_t n_items = 0, n_part = 0;
     size_t off_items = 0, off_ptoff = 0, off_limits = 0;  // byte offsets in blob
     int slot = -1;
@@ -93,8 +93,9 @@ struct Ctx {
     size_t part_o_cap = 0, part_ml_cap = 0, counters_cap = 0;  // in elements
     long opt_target_items = 0;                                 // 0 = automatic
     long opt_force_generic = 0;
-    long opt_hpw_max = 4;                                      // query heads per wave, at most
-    long opt_tile_rows = 4;                                    // wave rows that share an item's tiles
+    long opt_hpw_max = 0;                                      // query heads per wave, at most (0 = automatic)
+    long opt_buffers = 0;                                      // LDS staging buffers per workgroup (1, 2; 0 = automatic)
+    long opt_tile_rows = 1;                                    // wave rows that share an item's tiles
     long opt_pv_fp16 = 1;                                      // softmax weights rounded to fp16 for P.V
     int last_launches = 0;
     int last_items = 0;
@@ -178,7 +179,7 @@ bool plan_matches(const DecodePlan& p, const uint32_t* flat, size_t n_flat, cons
     if (!p.valid || p.B != B || p.H != H || p.Hkv != Hkv || p.D != D || p.P != P ||
         p.causal != causal || p.target_items != g.opt_target_items ||
         p.force_generic != g.opt_force_generic || p.hpw_max != g.opt_hpw_max ||
-        p.tile_rows != g.opt_tile_rows)
+        p.tile_rows != g.opt_tile_rows || p.buffers != g.opt_buffers)
         return false;
     if (p.pt_flat.size() != n_flat) return false;
     if (n_flat && std::memcmp(p.pt_flat.data(), flat, n_flat * 4) != 0) return false;
@@ -208,6 +209,7 @@ int build_plan(const uint32_t* flat, size_t n_flat, const uint32_t* off, const u
     p.force_generic = g.opt_force_generic;
     p.hpw_max = g.opt_hpw_max;
     p.tile_rows = g.opt_tile_rows;
+    p.buffers = g.opt_buffers;
 
     std::vector<uint32_t> limits(B);
     for (size_t r = 0; r < B; ++r) {
@@ -221,8 +223,12 @@ int build_plan(const uint32_t* flat, size_t n_flat, const uint32_t* off, const u
     const size_t G = H / Hkv;
     if (p.fast) {
         // query heads per wave (power of two dividing G), waves per workgroup = G / that
+        // Measured on MI355X: a wave issues one VALU instruction every ~5 cycles and a SIMD
+        // needs two or more waves in flight to use its ALUs, so wide GQA groups are spread
+        // over four waves (2 heads each); narrower groups keep 4 heads per wave.
+        const long hpw_cap = g.opt_hpw_max > 0 ? g.opt_hpw_max : (G >= 8 ? 2 : 4);
         int hpw = 8;
-        while (hpw > 1 && (hpw > g.opt_hpw_max || (G % (size_t)hpw) != 0)) hpw >>= 1;
+        while (hpw > 1 && (hpw > hpw_cap || (G % (size_t)hpw) != 0)) hpw >>= 1;
         size_t nw = G / (size_t)hpw;
         if (nw > 4 || nw == 3) {  // too many / odd wave counts: use the widest wave
             hpw = 8;
@@ -232,10 +238,13 @@ int build_plan(const uint32_t* flat, size_t n_flat, const uint32_t* off, const u
         if (nw > 4 || nw == 3) p.fast = false;
         p.hpw = hpw;
         p.nw = (int)nw;
-        // tile rows per workgroup: at most 8 waves per workgroup
+        // tile rows per workgroup, within the workgroup's LDS budget
         int ns = (int)g.opt_tile_rows;
-        while (ns > 1 && (size_t)ns * nw > 8) ns >>= 1;
+        const int nbuf = g.opt_buffers > 0 ? (int)g.opt_buffers : 2;  // refined below
+        while (ns > 1 && decode_lds_bytes((int)D, hpw, (int)nw, ns, nbuf) > kMaxStaticLds) ns >>= 1;
+        if (decode_lds_bytes((int)D, hpw, (int)nw, ns, nbuf) > kMaxStaticLds) p.fast = false;
         p.ns = ns;
+        p.nbuf = nbuf;
     }
     const size_t flat_bytes = align_up(n_flat * 4, 16);
 
@@ -245,10 +254,22 @@ int build_plan(const uint32_t* flat, size_t n_flat, const uint32_t* off, const u
         size_t total_tiles = 0;
         for (size_t r = 0; r < B; ++r) total_tiles += (limits[r] + tile - 1) / tile;
         total_tiles *= Hkv;
-        // Work items (= workgroups) aimed for: enough to give every SIMD two resident waves.
-        const size_t slots = (size_t)g.n_cu * 8 / (size_t)(p.nw * p.ns);
-        size_t target = g.opt_target_items > 0 ? (size_t)g.opt_target_items : slots;
+        // Work items (= workgroups) aimed for: as many as are resident at once, which the
+        // 160 KiB of LDS per CU decides (at most 16 waves per CU are counted on).
+        const size_t lds_wg = (size_t)decode_lds_bytes((int)D, p.hpw, p.nw, p.ns, p.nbuf);
+        const size_t per_cu = std::max<size_t>(1, std::min<size_t>(160 * 1024 / lds_wg,
+                                                                   16 / (size_t)(p.nw * p.ns)));
+        const size_t slots = (size_t)g.n_cu * per_cu;
+        (void)slots;
+        // About 8 tiles per item, but no fewer than 4 and no more than 16 items per CU
+        // (measured optimum on MI355X for 35 MB .. 1.2 GB of KV per call).
+        size_t target = std::min<size_t>(std::max<size_t>(total_tiles / 8, (size_t)g.n_cu * 4),
+                                         (size_t)g.n_cu * 16);
+        if (g.opt_target_items > 0) target = (size_t)g.opt_target_items;
         size_t chunk = std::max<size_t>(1, (total_tiles + target - 1) / target);
+        // Short items cannot use a second buffer; one buffer lets twice the workgroups
+        // share a CU and hide each other's memory latency.
+        if (g.opt_buffers == 0) p.nbuf = (chunk >= 4 * (size_t)p.ns) ? 2 : 1;
         for (size_t r = 0; r < B; ++r) {  // the merge pass handles at most kMaxSplits partials
             const size_t tiles_r = (limits[r] + tile - 1) / tile;
             chunk = std::max(chunk, (tiles_r + kMaxSplits - 1) / kMaxSplits);
@@ -272,13 +293,9 @@ int build_plan(const uint32_t* flat, size_t n_flat, const uint32_t* off, const u
                     it.pt_base = off[r];
                     it.tok_begin = (uint32_t)std::min<size_t>(s * per * tile, limits[r]);
                     it.tok_end = (uint32_t)std::min<size_t>((s + 1) * per * tile, limits[r]);
-                    for (size_t w = 0; w < 4; ++w) {
-                        const size_t t0 = it.tok_begin + w * tile;
-                        it.first_pages[w] = t0 < it.tok_end ? flat[off[r] + t0 / P] : 0;
-                    }
                     it.part_first = first_part;
                     it.split = (uint32_t)s | ((uint32_t)ns_eff << 16);
-                    it.pad = 0;
+                    std::memset(it.pad, 0, sizeof(it.pad));
                     items.push_back(it);
                 }
             }
@@ -347,21 +364,21 @@ int ensure_partials(size_t n_part, size_t G, size_t D, size_t nw) {
     return 1;
 }
 
-bool launch_fast(size_t D, int hpw, int nw, int ns, const DecodeArgs& a) {
+bool launch_fast(size_t D, int hpw, int nw, int ns, int nbuf, const DecodeArgs& a) {
     const bool pv16 = g.opt_pv_fp16 != 0;
     if (D == 64) {
         switch (hpw) {
-            case 8: return launch_decode_fast_64_8(nw, ns, pv16, a, g.stream);
-            case 4: return launch_decode_fast_64_4(nw, ns, pv16, a, g.stream);
-            case 2: return launch_decode_fast_64_2(nw, ns, pv16, a, g.stream);
-            default: return launch_decode_fast_64_1(nw, ns, pv16, a, g.stream);
+            case 8: return launch_decode_fast_64_8(nw, ns, nbuf, pv16, a, g.stream);
+            case 4: return launch_decode_fast_64_4(nw, ns, nbuf, pv16, a, g.stream);
+            case 2: return launch_decode_fast_64_2(nw, ns, nbuf, pv16, a, g.stream);
+            default: return launch_decode_fast_64_1(nw, ns, nbuf, pv16, a, g.stream);
         }
     }
     switch (hpw) {
-        case 8: return launch_decode_fast_128_8(nw, ns, pv16, a, g.stream);
-        case 4: return launch_decode_fast_128_4(nw, ns, pv16, a, g.stream);
-        case 2: return launch_decode_fast_128_2(nw, ns, pv16, a, g.stream);
-        default: return launch_decode_fast_128_1(nw, ns, pv16, a, g.stream);
+        case 8: return launch_decode_fast_128_8(nw, ns, nbuf, pv16, a, g.stream);
+        case 4: return launch_decode_fast_128_4(nw, ns, nbuf, pv16, a, g.stream);
+        case 2: return launch_decode_fast_128_2(nw, ns, nbuf, pv16, a, g.stream);
+        default: return launch_decode_fast_128_1(nw, ns, nbuf, pv16, a, g.stream);
     }
 }
 
@@ -542,7 +559,7 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
         a.page_size = (uint32_t)page_size_tokens;
         a.n_items = p.n_items;
         a.scale_log2e = scale_log2e;
-        if (!launch_fast(head_dim, p.hpw, p.nw, p.ns, a)) return fail("decode: kernel variant not built");
+        if (!launch_fast(head_dim, p.hpw, p.nw, p.ns, p.nbuf, a)) return fail("decode: kernel variant not built");
         ++g.last_launches;
     } else {
         GenericArgs a;
@@ -817,13 +834,18 @@ int mlc_hip_set_option(const char* name, long value) {
     if (!std::strcmp(name, "decode_target_items")) { g.opt_target_items = value; return 1; }
     if (!std::strcmp(name, "decode_force_generic")) { g.opt_force_generic = value; return 1; }
     if (!std::strcmp(name, "decode_pv_fp16")) { g.opt_pv_fp16 = value ? 1 : 0; return 1; }
+    if (!std::strcmp(name, "decode_buffers")) {
+        if (value != 0 && value != 1 && value != 2) return 0;
+        g.opt_buffers = value;
+        return 1;
+    }
     if (!std::strcmp(name, "decode_tile_rows")) {
-        if (value != 1 && value != 2 && value != 4) return 0;
+        if (value != 1 && value != 2) return 0;
         g.opt_tile_rows = value;
         return 1;
     }
     if (!std::strcmp(name, "decode_heads_per_wave")) {
-        if (value != 1 && value != 2 && value != 4 && value != 8) return 0;
+        if (value != 0 && value != 1 && value != 2 && value != 4 && value != 8) return 0;
         g.opt_hpw_max = value;
         return 1;
     }

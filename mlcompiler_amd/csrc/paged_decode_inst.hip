@@ -12,28 +12,36 @@
 namespace mlc_hip {
 
 namespace {
+template <int NW, int NS, int NBUF>
+bool launch_buf(bool pv16, const DecodeArgs& a, hipStream_t stream) {
+    if constexpr (decode_lds_bytes(MLC_D, MLC_HPW, NW, NS, NBUF) <= kMaxStaticLds) {
+        const dim3 grid(a.n_items), block(64 * NW * NS);
+        if (pv16)
+            hipLaunchKernelGGL((paged_decode_fast_kernel<MLC_D, MLC_HPW, NW, NS, NBUF, true>), grid, block, 0, stream, a);
+        else
+            hipLaunchKernelGGL((paged_decode_fast_kernel<MLC_D, MLC_HPW, NW, NS, NBUF, false>), grid, block, 0, stream, a);
+        return true;
+    } else {
+        return false;
+    }
+}
+
 template <int NW, int NS>
-void launch_one(bool pv16, const DecodeArgs& a, hipStream_t stream) {
-    const dim3 grid(a.n_items), block(64 * NW * NS);
-    if (pv16)
-        hipLaunchKernelGGL((paged_decode_fast_kernel<MLC_D, MLC_HPW, NW, NS, true>), grid, block, 0, stream, a);
-    else
-        hipLaunchKernelGGL((paged_decode_fast_kernel<MLC_D, MLC_HPW, NW, NS, false>), grid, block, 0, stream, a);
+bool launch_one(int nbuf, bool pv16, const DecodeArgs& a, hipStream_t stream) {
+    return nbuf == 1 ? launch_buf<NW, NS, 1>(pv16, a, stream) : launch_buf<NW, NS, 2>(pv16, a, stream);
 }
 }  // namespace
 
 // nw = waves over the GQA group, ns = tile rows; returns false for an unbuilt combination.
-bool MLC_CAT(MLC_D, MLC_HPW)(int nw, int ns, bool pv16, const DecodeArgs& a, hipStream_t stream) {
+bool MLC_CAT(MLC_D, MLC_HPW)(int nw, int ns, int nbuf, bool pv16, const DecodeArgs& a, hipStream_t stream) {
     const int key = nw * 10 + ns;
     switch (key) {
-        case 11: launch_one<1, 1>(pv16, a, stream); return true;
-        case 12: launch_one<1, 2>(pv16, a, stream); return true;
-        case 14: launch_one<1, 4>(pv16, a, stream); return true;
-        case 21: launch_one<2, 1>(pv16, a, stream); return true;
-        case 22: launch_one<2, 2>(pv16, a, stream); return true;
-        case 24: launch_one<2, 4>(pv16, a, stream); return true;
-        case 41: launch_one<4, 1>(pv16, a, stream); return true;
-        case 42: launch_one<4, 2>(pv16, a, stream); return true;
+        case 11: return launch_one<1, 1>(nbuf, pv16, a, stream);
+        case 12: return launch_one<1, 2>(nbuf, pv16, a, stream);
+        case 21: return launch_one<2, 1>(nbuf, pv16, a, stream);
+        case 22: return launch_one<2, 2>(nbuf, pv16, a, stream);
+        case 41: return launch_one<4, 1>(nbuf, pv16, a, stream);
+        case 42: return launch_one<4, 2>(nbuf, pv16, a, stream);
         default: return false;
     }
 }

@@ -51,8 +51,7 @@ struct DecodeWorkItem {
     uint32_t tok_end;     // one past the last visible kv position of this item
     uint32_t part_first;  // first partial slot of this (request, kv head), or kNoPartial
     uint32_t split;       // this item's split index | number of splits << 16
-    uint32_t first_pages[4];  // page id of the first tile of each tile row (saves a dependent load)
-    uint32_t pad;
+    uint32_t pad[5];
 };
 static_assert(sizeof(DecodeWorkItem) == 48, "work items are uploaded as raw bytes");
 static constexpr uint32_t kNoPartial = 0xFFFFFFFFu;
@@ -124,9 +123,32 @@ static constexpr float kNegBig = -1.0e30f;
 // A tile may exceed the running reference by 2^kLazyTau before accumulators are rescaled.
 static constexpr float kLazyTau = 8.0f;
 
-template <int D, int HPW, int NW, int NS, bool PV16>
+// Static LDS of one workgroup of the tiled kernel (staging buffers, reused by the epilogue).
+static constexpr int kMaxStaticLds = 65536;
+constexpr int decode_lds_bytes(int D, int HPW, int NW, int NS, int NBUF) {
+    const int rpi = 64 / (D / 8);
+    const int stage = NS * 2 * (8 * rpi * D * 2);  // one staging buffer: [NS][K, V] tiles
+    const int epi = NW * NS * rpi * HPW * D * 4;   // the epilogue's sums must fit one buffer
+    return NBUF * (epi > stage ? epi : stage) + (NBUF == 1 ? 512 : 0);
+}
+
+// 16-byte global -> LDS copy that bypasses the register file: lane i's 16 bytes land at
+// lds_base + 16*i (lds_base is wave-uniform), whatever global address lane i reads.
+__device__ __forceinline__ void g2lds16(const uint4* g, void* lds_base) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                     (__attribute__((address_space(3))) void*)lds_base, 16, 0, 0);
+}
+
+// s_waitcnt vmcnt(N) with the other counters left alone (gfx9 encoding).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
+}
+
+template <int D, int HPW, int NW, int NS, int NBUF, bool PV16>
 __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const DecodeArgs a) {
     static_assert(D == 64 || D == 128, "fast path covers head_dim 64 and 128");
+    static_assert(NW == 1 || NW == 2 || NW == 4, "waves per GQA group");
     constexpr int CPR = D / 8;         // 16-byte chunks per row
     constexpr int RPI = 64 / CPR;      // rows fetched by one wave-wide load
     constexpr int TT = 8 * RPI;        // tokens per tile
@@ -134,57 +156,50 @@ __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const D
     constexpr int HPK = D / 64;        // epilogue registers per head: idx = k*64+lane -> h = k/HPK
     constexpr int G = HPW * NW;        // query heads per KV head
     constexpr int NWAVES = NW * NS;
-
-    __shared__ float s_acc_all[NWAVES][RPI * HPW * D];
-    __shared__ float s_ml[NWAVES][HPW][2];
+    constexpr int TILE_BYTES = TT * D * 2;  // one tensor, one KV head: 8 KiB for both head sizes
+    constexpr int LPW = 16 / NW;            // tile-load instructions per wave and step (8 K + 8 V per tile)
+    // LDS: [2 buffers][NS tile rows][K, V][TILE_BYTES] staging, reused by the epilogue as
+    // [NWAVES][RPI*HPW*D] floats + [NWAVES][HPW][2] floats.
+    // one buffer: [NS tile rows][K, V], at least as large as the epilogue's [NWAVES][RPI*HPW*D] floats
+    constexpr int STAGE_BYTES = (decode_lds_bytes(D, HPW, NW, NS, NBUF) - (NBUF == 1 ? 512 : 0)) / NBUF;
+    static_assert(NBUF * STAGE_BYTES <= kMaxStaticLds, "workgroup LDS budget");
+    // Two separate arrays (not one indexed by the step parity): the compiler then knows that
+    // reads of the buffer being consumed do not alias the global -> LDS loads in flight into
+    // the other one, and does not wait for those loads before every LDS read.
+    __shared__ __attribute__((aligned(16))) unsigned char stage0[STAGE_BYTES];
+    // With one buffer (NBUF == 1) the second array only holds the epilogue's (m, l) pairs;
+    // latency is then hidden by the other workgroups of the CU instead of by prefetching.
+    __shared__ __attribute__((aligned(16))) unsigned char stage1[NBUF == 2 ? STAGE_BYTES : 512];
 
     const uint32_t item_idx = blockIdx.x;
     if (item_idx >= a.n_items) return;
-    const DecodeWorkItem it = a.items[item_idx];
-    const int wave = threadIdx.x / 64;
+    // The item is read once, into scalar registers: any vector load issued after the tile
+    // loads would have to wait for them (loads return in order).
+    struct {
+        uint32_t req, kv_head, pt_base, tok_begin, tok_end, part_first, split;
+    } it;
+    {
+        const DecodeWorkItem* gi = a.items + item_idx;
+        it.req = __builtin_amdgcn_readfirstlane(gi->req);
+        it.kv_head = __builtin_amdgcn_readfirstlane(gi->kv_head);
+        it.pt_base = __builtin_amdgcn_readfirstlane(gi->pt_base);
+        it.tok_begin = __builtin_amdgcn_readfirstlane(gi->tok_begin);
+        it.tok_end = __builtin_amdgcn_readfirstlane(gi->tok_end);
+        it.part_first = __builtin_amdgcn_readfirstlane(gi->part_first);
+        it.split = __builtin_amdgcn_readfirstlane(gi->split);
+    }
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);  // wave-uniform, in an SGPR
     const int lane = threadIdx.x % 64;
     const int hg = wave % NW;   // head group of this wave
     const int sub = wave / NW;  // tile row of this wave
-    float* s_acc = s_acc_all[wave];
     const int c = lane % CPR;
     const int r = lane / CPR;
     const int c7 = c & 7;
     const int gsw = c7 ^ ((c7 & 4) ? 3 : 0);  // row-group swizzle g(c)
     const uint32_t head0 = it.kv_head * G + hg * HPW;
 
-    const uint32_t row_u4 = a.kv_heads * CPR;  // 16-byte chunks per token row (all KV heads)
-    const uint32_t lane_u4 = it.kv_head * CPR + c;
-
-    // The 8 rows this lane reads in a tile; rows past the visible end are clamped onto the
-    // last visible row (in bounds, masked out of the softmax below).
-    auto load_tile = [&](const uint4* pages, uint32_t page_id, uint32_t tile_start,
-                         uint4 (&reg)[8]) {
-        const uint32_t slot0 = tile_start % a.page_size;
-        const uint32_t last = it.tok_end - 1u - tile_start;  // last visible row of the tile
-        const uint4* base = pages + ((size_t)page_id * a.page_size + slot0) * row_u4 + lane_u4;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            uint32_t t = (uint32_t)((j ^ gsw) * RPI + r);
-            t = t < last ? t : last;
-            reg[j] = base[(size_t)t * row_u4];
-        }
-    };
-    auto page_of = [&](uint32_t tile_start) {
-        return a.pt_flat[it.pt_base + tile_start / a.page_size];
-    };
-
-    constexpr uint32_t STEP = TT * NS;  // this wave's tiles are STEP tokens apart
-    const uint32_t my_begin = it.tok_begin + (uint32_t)sub * TT;
-    uint4 kreg[8], vreg[8];
-    if (my_begin < it.tok_end) {
-        const uint32_t pg = it.first_pages[sub];
-        load_tile(a.k_pages, pg, my_begin, kreg);
-        load_tile(a.v_pages, pg, my_begin, vreg);
-    }
-    uint32_t next_page = 0;
-    if (my_begin + STEP < it.tok_end) next_page = page_of(my_begin + STEP);
-
-    // q for this wave's heads, dims c*8 .. c*8+7, pre-scaled.
+    // q for this wave's heads, dims c*8 .. c*8+7 (issued before the tile loads, so that waiting
+    // for it does not wait for them).
     float qv[HPW][8];
     {
         const float* qbase = a.q + ((size_t)it.req * a.num_heads + head0) * D + c * 8;
@@ -192,12 +207,65 @@ __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const D
         for (int h = 0; h < HPW; ++h) {
             const float4 lo = *reinterpret_cast<const float4*>(qbase + h * D);
             const float4 hi = *reinterpret_cast<const float4*>(qbase + h * D + 4);
-            qv[h][0] = lo.x * a.scale_log2e; qv[h][1] = lo.y * a.scale_log2e;
-            qv[h][2] = lo.z * a.scale_log2e; qv[h][3] = lo.w * a.scale_log2e;
-            qv[h][4] = hi.x * a.scale_log2e; qv[h][5] = hi.y * a.scale_log2e;
-            qv[h][6] = hi.z * a.scale_log2e; qv[h][7] = hi.w * a.scale_log2e;
+            qv[h][0] = lo.x; qv[h][1] = lo.y; qv[h][2] = lo.z; qv[h][3] = lo.w;
+            qv[h][4] = hi.x; qv[h][5] = hi.y; qv[h][6] = hi.z; qv[h][7] = hi.w;
         }
     }
+
+    const uint32_t row_u4 = a.kv_heads * CPR;  // 16-byte chunks per token row (all KV heads)
+    const uint32_t lane_u4 = it.kv_head * CPR + c;
+    const uint32_t n_tiles = (it.tok_end - it.tok_begin + TT - 1) / TT;
+    const uint32_t n_steps = (n_tiles + NS - 1) / NS;
+
+    // This wave's share of the global -> LDS loads of tile `t` of the item (row `sub` of
+    // buffer `buf`).  Load instruction j of a tensor brings row group j ^ g(c) to lane (r, c),
+    // at LDS offset j*1024 + lane*16; rows past the visible end are clamped onto the last
+    // visible row (in bounds, masked out of the softmax).
+    auto issue_tile = [&](uint32_t t, unsigned char* stage, uint32_t page_id) {
+        const uint32_t tile_start = it.tok_begin + t * TT;
+        const uint32_t slot0 = tile_start % a.page_size;
+        const uint32_t last = it.tok_end - 1u - tile_start;
+        const size_t row0 = ((size_t)page_id * a.page_size + slot0) * row_u4 + lane_u4;
+        unsigned char* slot = stage + (size_t)(sub * 2) * TILE_BYTES;
+        constexpr int PARTS = (NW == 1) ? 2 : 1;
+        constexpr int JN = (NW == 4) ? 4 : 8;
+#pragma unroll
+        for (int p = 0; p < PARTS; ++p) {
+            const int tensor = (NW == 1) ? p : (NW == 2 ? hg : hg / 2);
+            const int j0 = (NW == 4) ? (hg % 2) * 4 : 0;
+            const uint4* base = (tensor ? a.v_pages : a.k_pages) + row0;
+            unsigned char* dst = slot + tensor * TILE_BYTES;
+#pragma unroll
+            for (int jj = 0; jj < JN; ++jj) {
+                const int j = j0 + jj;
+                uint32_t tr = (uint32_t)((j ^ gsw) * RPI + r);
+                tr = tr < last ? tr : last;
+                g2lds16(base + (size_t)tr * row_u4, dst + j * 1024);
+            }
+        }
+    };
+    // Page ids of this wave's tiles (tile sub + i*NS in lane i), fetched 64 steps at a time
+    // and before the tile loads for the same reason as q.
+    uint32_t page_vec = 0;
+    auto fetch_pages = [&](uint32_t step0) {
+        const uint32_t t = (step0 + lane) * NS + sub;
+        page_vec = 0;
+        if (t < n_tiles) page_vec = a.pt_flat[it.pt_base + (it.tok_begin + t * TT) / a.page_size];
+    };
+    auto page_of_step = [&](uint32_t step) {
+        return (uint32_t)__builtin_amdgcn_readlane((int)page_vec, (int)(step & 63u));
+    };
+    fetch_pages(0);
+    const uint32_t pg0 = page_of_step(0), pg1 = page_of_step(1);  // waits for the fetch here
+
+    const bool have1 = NBUF == 2 && (uint32_t)(NS + sub) < n_tiles;
+    if ((uint32_t)sub < n_tiles) issue_tile(sub, stage0, pg0);
+    if (have1) issue_tile(NS + sub, stage1, pg1);
+
+#pragma unroll
+    for (int h = 0; h < HPW; ++h)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) qv[h][i] *= a.scale_log2e;
 
     float acc[HPW][8];
     float m_ref[HPW], l_sum[HPW];
@@ -209,35 +277,53 @@ __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const D
         for (int i = 0; i < 8; ++i) acc[h][i] = 0.f;
     }
 
-    for (uint32_t tile_start = my_begin; tile_start < it.tok_end; tile_start += STEP) {
-        const uint32_t next = tile_start + STEP;
-        const bool has_next = next < it.tok_end;
-        const uint32_t page_n = next_page;
-        if (next + STEP < it.tok_end) next_page = page_of(next + STEP);
+    // One step of the pipeline: consume `cur`, refill `nxt` (which the previous step consumed).
+    auto do_step = [&](uint32_t step, unsigned char* cur, unsigned char* nxt) {
+        const uint32_t t = step * NS + sub;
+        if (NBUF == 1 && step >= 1) {
+            __syncthreads();  // everyone left the previous step: the buffer can be refilled
+            if ((step & 63u) == 0) fetch_pages(step);
+            if (t < n_tiles) issue_tile(t, cur, page_of_step(step));
+        }
+        // own loads of this step have landed (at step 0 the loads of step 1 may stay in flight)
+        if (step == 0 && have1) wait_vmcnt<LPW>(); else wait_vmcnt<0>();
+        __syncthreads();  // everyone's loads of this step landed; everyone left the previous step
+        if (NBUF == 2 && step >= 1 && step + 1 < n_steps) {
+            if (((step + 1) & 63u) == 0) fetch_pages(step + 1);  // nothing else is in flight here
+            const uint32_t t2 = (step + 1) * NS + sub;
+            if (t2 < n_tiles) issue_tile(t2, nxt, page_of_step(step + 1));
+        }
+        if (t >= n_tiles) return;
+        const uint32_t tile_start = it.tok_begin + t * TT;
+        const uint4* kl = reinterpret_cast<const uint4*>(cur + (size_t)(sub * 2) * TILE_BYTES) + lane;
+        const uint4* vl = kl + TILE_BYTES / 16;
 
-        // ---- QK: per head, partial dots over this lane's 8 dims for the 8 row groups,
-        // then a reduce-scatter over the 8 c-lanes (lane keeps row group g(c)).
-        float sc[HPW];
+        // ---- QK: partial dots over this lane's 8 dims for the 8 row groups, then per head a
+        // reduce-scatter over the 8 c-lanes (lane keeps row group g(c)).
+        float part[HPW][8];
 #pragma unroll
-        for (int h = 0; h < HPW; ++h) {
-            float part[8];
+        for (int j = 0; j < 8; ++j) {
+            const uint4 kq = kl[j * 64];
+            const half8_t kh = __builtin_bit_cast(half8_t, kq);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const half8_t kh = __builtin_bit_cast(half8_t, kreg[j]);
+            for (int h = 0; h < HPW; ++h) {
                 float s = qv[h][0] * (float)kh[0];
 #pragma unroll
                 for (int i = 1; i < 8; ++i) s = fmaf(qv[h][i], (float)kh[i], s);
-                part[j] = s;
+                part[h][j] = s;
             }
+        }
+        float sc[HPW];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) part[j] += dpp_f<kDppHalfMirror>(part[j + 4]);
+        for (int h = 0; h < HPW; ++h) {
 #pragma unroll
-            for (int j = 0; j < 2; ++j) part[j] += dpp_f<kDppQuadXor2>(part[j + 2]);
-            float s = part[0] + dpp_f<kDppQuadXor1>(part[1]);
+            for (int j = 0; j < 4; ++j) part[h][j] += dpp_f<kDppHalfMirror>(part[h][j + 4]);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) part[h][j] += dpp_f<kDppQuadXor2>(part[h][j + 2]);
+            float s = part[h][0] + dpp_f<kDppQuadXor1>(part[h][1]);
             if (CPR == 16) s += dpp_f<kDppRowRor8>(s);
             sc[h] = s;
         }
-        if (has_next) load_tile(a.k_pages, page_n, next, kreg);
 
         // ---- mask, tile maximum over the r-set, lazy reference update
         const uint32_t my_tok = tile_start + (uint32_t)(gsw * RPI + r);
@@ -270,10 +356,12 @@ __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const D
         if constexpr (PV16) {
             // ---- weights rounded to fp16 (the sum l uses the rounded values, so the result
             // is an exactly normalised average with weights perturbed by <= 2^-11), packed
-            // two heads to a register.
-            uint32_t pp[(HPW + 1) / 2];
+            // two heads to a register and gathered over the 8 c-lanes: register j of the
+            // gather holds the weights of the token whose V row sits in V register j.
+            constexpr int H2 = (HPW + 1) / 2;
+            uint32_t g8[H2][8];
 #pragma unroll
-            for (int h2 = 0; h2 < (HPW + 1) / 2; ++h2) {
+            for (int h2 = 0; h2 < H2; ++h2) {
                 const _Float16 p0 = (_Float16)fast_exp2(sc[2 * h2] - m_ref[2 * h2]);
                 l_sum[2 * h2] += (float)p0;
                 _Float16 p1 = (_Float16)0.f;
@@ -282,85 +370,89 @@ __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const D
                     l_sum[2 * h2 + 1] += (float)p1;
                 }
                 half2_t pk = {p0, p1};
-                pp[h2] = __builtin_bit_cast(uint32_t, pk);
+                const uint32_t pp = __builtin_bit_cast(uint32_t, pk);
+                g8[h2][0] = pp;
+                g8[h2][1] = dpp_u<kDppQuadXor1>(pp);
+                g8[h2][2] = dpp_u<kDppQuadXor2>(pp);
+                g8[h2][3] = dpp_u<kDppQuadXor3>(pp);
+                g8[h2][4] = dpp_u<kDppHalfMirror>(pp);
+                g8[h2][5] = dpp_u<kDppQuadXor1>(g8[h2][4]);
+                g8[h2][6] = dpp_u<kDppQuadXor2>(g8[h2][4]);
+                g8[h2][7] = dpp_u<kDppQuadXor3>(g8[h2][4]);
             }
-            // ---- PV with v_dot2_f32_f16: register j of this lane holds the V row whose
-            // weight lives in the lane at swizzle distance j.  V rows are paired (j, j+1)
-            // per dim, the weights of the same two rows are paired per head.
-            uint32_t vp[4][8];  // [row pair][dim] = (v[2k][i], v[2k+1][i])
+            // ---- PV with v_dot2_f32_f16 on row pairs (2k, 2k+1)
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-                const uint32_t* va = reinterpret_cast<const uint32_t*>(&vreg[2 * k]);
-                const uint32_t* vb = reinterpret_cast<const uint32_t*>(&vreg[2 * k + 1]);
+                const uint4 va4 = vl[(2 * k) * 64];
+                const uint4 vb4 = vl[(2 * k + 1) * 64];
+                const uint32_t* va = reinterpret_cast<const uint32_t*>(&va4);
+                const uint32_t* vb = reinterpret_cast<const uint32_t*>(&vb4);
+                uint32_t vp[8];  // (v[2k][i], v[2k+1][i])
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
-                    // dims 2w (low halves) and 2w+1 (high halves) of both rows
-                    vp[k][2 * w] = __builtin_amdgcn_perm(vb[w], va[w], 0x05040100u);
-                    vp[k][2 * w + 1] = __builtin_amdgcn_perm(vb[w], va[w], 0x07060302u);
+                    vp[2 * w] = __builtin_amdgcn_perm(vb[w], va[w], 0x05040100u);
+                    vp[2 * w + 1] = __builtin_amdgcn_perm(vb[w], va[w], 0x07060302u);
                 }
-            }
-            if (has_next) load_tile(a.v_pages, page_n, next, vreg);  // vreg is dead once packed
 #pragma unroll
-            for (int h2 = 0; h2 < (HPW + 1) / 2; ++h2) {
-                uint32_t g8[8];
-                g8[0] = pp[h2];
-                g8[1] = dpp_u<kDppQuadXor1>(pp[h2]);
-                g8[2] = dpp_u<kDppQuadXor2>(pp[h2]);
-                g8[3] = dpp_u<kDppQuadXor3>(pp[h2]);
-                g8[4] = dpp_u<kDppHalfMirror>(pp[h2]);
-                g8[5] = dpp_u<kDppQuadXor1>(g8[4]);
-                g8[6] = dpp_u<kDppQuadXor2>(g8[4]);
-                g8[7] = dpp_u<kDppQuadXor3>(g8[4]);
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    // (p[h][row 2k], p[h][row 2k+1]) for the two heads packed in g8
-                    const uint32_t w0 = __builtin_amdgcn_perm(g8[2 * k + 1], g8[2 * k], 0x05040100u);
+                for (int h2 = 0; h2 < H2; ++h2) {
+                    const uint32_t w0 =
+                        __builtin_amdgcn_perm(g8[h2][2 * k + 1], g8[h2][2 * k], 0x05040100u);
                     const half2_t pw0 = __builtin_bit_cast(half2_t, w0);
 #pragma unroll
                     for (int i = 0; i < 8; ++i)
                         acc[2 * h2][i] = __builtin_amdgcn_fdot2(
-                            __builtin_bit_cast(half2_t, vp[k][i]), pw0, acc[2 * h2][i], false);
+                            __builtin_bit_cast(half2_t, vp[i]), pw0, acc[2 * h2][i], false);
                     if (2 * h2 + 1 < HPW) {
                         const uint32_t w1 =
-                            __builtin_amdgcn_perm(g8[2 * k + 1], g8[2 * k], 0x07060302u);
+                            __builtin_amdgcn_perm(g8[h2][2 * k + 1], g8[h2][2 * k], 0x07060302u);
                         const half2_t pw1 = __builtin_bit_cast(half2_t, w1);
 #pragma unroll
                         for (int i = 0; i < 8; ++i)
                             acc[2 * h2 + 1][i] = __builtin_amdgcn_fdot2(
-                                __builtin_bit_cast(half2_t, vp[k][i]), pw1, acc[2 * h2 + 1][i],
-                                false);
+                                __builtin_bit_cast(half2_t, vp[i]), pw1, acc[2 * h2 + 1][i], false);
                     }
                 }
             }
         } else {
             // ---- exact fp32 weights: gather them over the 8 lanes, fp16 V widened in the FMA
-            float p[HPW];
+            float pj[HPW][8];
 #pragma unroll
             for (int h = 0; h < HPW; ++h) {
-                p[h] = fast_exp2(sc[h] - m_ref[h]);
-                l_sum[h] += p[h];
+                const float p = fast_exp2(sc[h] - m_ref[h]);
+                l_sum[h] += p;
+                pj[h][0] = p;
+                pj[h][1] = dpp_f<kDppQuadXor1>(p);
+                pj[h][2] = dpp_f<kDppQuadXor2>(p);
+                pj[h][3] = dpp_f<kDppQuadXor3>(p);
+                pj[h][4] = dpp_f<kDppHalfMirror>(p);
+                pj[h][5] = dpp_f<kDppQuadXor1>(pj[h][4]);
+                pj[h][6] = dpp_f<kDppQuadXor2>(pj[h][4]);
+                pj[h][7] = dpp_f<kDppQuadXor3>(pj[h][4]);
             }
 #pragma unroll
-            for (int h = 0; h < HPW; ++h) {
-                float pj[8];
-                pj[0] = p[h];
-                pj[1] = dpp_f<kDppQuadXor1>(p[h]);
-                pj[2] = dpp_f<kDppQuadXor2>(p[h]);
-                pj[3] = dpp_f<kDppQuadXor3>(p[h]);
-                pj[4] = dpp_f<kDppHalfMirror>(p[h]);
-                pj[5] = dpp_f<kDppQuadXor1>(pj[4]);
-                pj[6] = dpp_f<kDppQuadXor2>(pj[4]);
-                pj[7] = dpp_f<kDppQuadXor3>(pj[4]);
+            for (int j = 0; j < 8; ++j) {
+                const uint4 vq = vl[j * 64];
+                const half8_t vh = __builtin_bit_cast(half8_t, vq);
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const half8_t vh = __builtin_bit_cast(half8_t, vreg[j]);
+                for (int h = 0; h < HPW; ++h)
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) acc[h][i] = fmaf(pj[j], (float)vh[i], acc[h][i]);
-                }
+                    for (int i = 0; i < 8; ++i) acc[h][i] = fmaf(pj[h][j], (float)vh[i], acc[h][i]);
             }
-            if (has_next) load_tile(a.v_pages, page_n, next, vreg);
         }
+    };
+    if constexpr (NBUF == 2) {
+        for (uint32_t step = 0; step < n_steps; step += 2) {
+            do_step(step, stage0, stage1);
+            if (step + 1 < n_steps) do_step(step + 1, stage1, stage0);
+        }
+    } else {
+        for (uint32_t step = 0; step < n_steps; ++step) do_step(step, stage0, stage0);
     }
+    __syncthreads();  // staging memory is reused below
+
+    static_assert(NWAVES * RPI * HPW * D * 4 <= STAGE_BYTES, "epilogue sums fit the first buffer");
+    float* s_acc = reinterpret_cast<float*>(stage0) + (size_t)wave * (RPI * HPW * D);
+    float* s_ml = reinterpret_cast<float*>(stage1);  // [NWAVES][HPW][2]
 
     // ---- epilogue 1: bring the RPI r-sets of this wave onto one reference, sum over r
     // through this wave's LDS region.
@@ -407,8 +499,8 @@ __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const D
                 mh = (lane == hh) ? m_all[hh] : mh;
                 lh = (lane == hh) ? l_all[hh] : lh;
             }
-            s_ml[wave][lane][0] = mh;
-            s_ml[wave][lane][1] = lh;
+            s_ml[(wave * HPW + lane) * 2] = mh;
+            s_ml[(wave * HPW + lane) * 2 + 1] = lh;
         }
         __syncthreads();
         if (sub != 0) return;
@@ -416,13 +508,13 @@ __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const D
         for (int h = 0; h < HPW; ++h) {
             float m = kNegBig;
 #pragma unroll
-            for (int s = 0; s < NS; ++s) m = max_nn(m, s_ml[s * NW + hg][h][0]);
+            for (int s = 0; s < NS; ++s) m = max_nn(m, s_ml[((s * NW + hg) * HPW + h) * 2]);
             float l = 0.f;
             float w[NS];
 #pragma unroll
             for (int s = 0; s < NS; ++s) {
-                w[s] = fast_exp2(s_ml[s * NW + hg][h][0] - m);
-                l += w[s] * s_ml[s * NW + hg][h][1];
+                w[s] = fast_exp2(s_ml[((s * NW + hg) * HPW + h) * 2] - m);
+                l += w[s] * s_ml[((s * NW + hg) * HPW + h) * 2 + 1];
             }
             m_all[h] = m;
             l_all[h] = l;
@@ -431,7 +523,8 @@ __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const D
                 const int k = h * HPK + kk;
                 float sum = 0.f;
 #pragma unroll
-                for (int s = 0; s < NS; ++s) sum += w[s] * s_acc_all[s * NW + hg][k * 64 + lane];
+                for (int s = 0; s < NS; ++s)
+                    sum += w[s] * reinterpret_cast<const float*>(stage0)[(size_t)(s * NW + hg) * (RPI * HPW * D) + k * 64 + lane];
                 o_un[k] = sum;
             }
         }
