@@ -772,9 +772,9 @@ int mlc_hip_paged_attn_prefill(const void* q_f16, const void* k_pages, const voi
         !check_pool_bounds(v_pages, page_tables_flat, page_table_offsets, seq_lens, batch,
                            page_size_tokens, row_bytes, "prefill V"))
         return 0;
-    if (!prefill_shape_supported(head_dim, page_size_tokens) || !aligned16(q_f16) ||
+    if (!prefill_shape_supported(head_dim, page_size_tokens, num_heads, kv_heads) || !aligned16(q_f16) ||
         !aligned16(k_pages) || !aligned16(v_pages) || !aligned16(o))
-        return fail("prefill: unsupported shape (head_dim must be 128 or 64, page size a multiple of 32, 16-byte aligned buffers)");
+        return fail("prefill: unsupported shape (head_dim 64 or 128, page size a multiple of 32, heads/kv_heads in {1,2,4,8}, 16-byte aligned buffers)");
 
     MetaSlot& s = g.ring[g.ring_next];
     g.ring_next = (g.ring_next + 1) % 8;
