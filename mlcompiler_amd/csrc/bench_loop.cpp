@@ -76,4 +76,29 @@ int mlc_bench_decode_step_loop(const void* q, void* const* k_pools, void* const*
     return 1;
 }
 
+// Chunked prefill: `steps` calls of the MFMA kernel on the same inputs.
+int mlc_bench_prefill_loop(const void* q_f16, const void* k_pages, const void* v_pages, void* o,
+                           const uint32_t* page_tables_flat, size_t n_flat,
+                           const uint32_t* page_table_offsets, const uint32_t* seq_lens,
+                           const uint32_t* q_start, size_t batch, size_t chunk, size_t num_heads,
+                           size_t kv_heads, size_t head_dim, size_t page_size_tokens, size_t steps,
+                           float* event_ms, double* wall_s) {
+    if (!mlc_hip_begin()) return 0;
+    const auto t0 = std::chrono::steady_clock::now();
+    if (!mlc_hip_timer_start()) return 0;
+    for (size_t i = 0; i < steps; ++i) {
+        if (!mlc_hip_paged_attn_prefill(q_f16, k_pages, v_pages, o, page_tables_flat, n_flat,
+                                        page_table_offsets, seq_lens, q_start, batch, chunk,
+                                        num_heads, kv_heads, head_dim, page_size_tokens, 0))
+            return 0;
+    }
+    const float ms = mlc_hip_timer_stop();
+    if (ms < 0.f) return 0;
+    if (!mlc_hip_flush()) return 0;
+    const auto t1 = std::chrono::steady_clock::now();
+    if (event_ms) *event_ms = ms;
+    if (wall_s) *wall_s = std::chrono::duration<double>(t1 - t0).count();
+    return 1;
+}
+
 }  // extern "C"
