@@ -28,6 +28,117 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
+
+
+def bench_copy(args) -> int:
+    """Plain copy kernel of known size: calibrates FETCH_SIZE / WRITE_SIZE and gives the
+    practical streaming ceiling at the decode workload's size."""
+    import ctypes as C
+
+    from mlcompiler_amd import HipExecutor
+    from mlcompiler_amd.build import BENCH_LIB_PATH
+    exe = HipExecutor.Instance()
+    exe.requireAvailable()
+    bl = C.CDLL(BENCH_LIB_PATH)
+    nbytes = args.copy_mib << 20
+    pairs = [(exe.allocateScratchBuffer(nbytes), exe.allocateScratchBuffer(nbytes)) for _ in range(8)]
+    for s_, d_ in pairs:
+        exe.zeroBuffer(s_, nbytes)
+    ms = C.c_float()
+    total_ms = 0.0
+    for rep in range(2):   # first pass warms up
+        total_ms = 0.0
+        for s_, d_ in pairs:  # rotate buffers so the data does not sit in the Infinity Cache
+            assert bl.mlc_bench_copy_loop(C.c_void_p(s_), C.c_void_p(d_), C.c_size_t(nbytes),
+                                          C.c_size_t(max(args.steps // 8, 1)), C.byref(ms))
+            total_ms += ms.value
+    n = max(args.steps // 8, 1) * 8
+    us = total_ms / n * 1e3
+    print(json.dumps({"metric": "plain copy kernel", "bytes_read_per_launch": nbytes,
+                      "bytes_written_per_launch": nbytes, "us_per_launch": round(us, 3),
+                      "read_plus_write_GBs": round(2 * nbytes / us / 1e3, 1), "launches": n}))
+    return 0
+
+
+def bench_prefill(args) -> int:
+    """Chunked prefill (benchmark configuration 5): B=8, 256-row fp16 query chunk after 3840
+    cached tokens, 32q/8kv heads, head_dim 128.  Reports TFLOP/s on the exact causal FLOPs."""
+    import ctypes as C
+
+    from mlcompiler_amd import HipExecutor
+    from mlcompiler_amd.build import BENCH_LIB_PATH
+    from test_paged_prefill_gpu import make_prefill, oracle
+    exe = HipExecutor.Instance()
+    exe.requireAvailable()
+    B, Cc, H, Hkv, D, P, ctx = 8, 256, 32, 8, 128, 64, 3840
+    w = make_prefill(B, Cc, H, Hkv, D, P, [ctx] * B, seed=55)
+    bufs = [exe.allocateScratchBuffer(w[n].nbytes) for n in ("q", "k", "v")]
+    for b, n in zip(bufs, ("q", "k", "v")):
+        assert exe.uploadToBuffer(b, w[n])
+    ob = exe.allocateScratchBuffer(B * Cc * H * D * 4)
+    bl = C.CDLL(BENCH_LIB_PATH)
+    u32p = C.POINTER(C.c_uint32)
+    meta = [np.ascontiguousarray(w[k], np.uint32) for k in ("flat", "off", "seq", "q_start")]
+
+    def loop(steps):
+        ms, wall_s = C.c_float(), C.c_double()
+        ok = bl.mlc_bench_prefill_loop(
+            C.c_void_p(bufs[0]), C.c_void_p(bufs[1]), C.c_void_p(bufs[2]), C.c_void_p(ob),
+            meta[0].ctypes.data_as(u32p), C.c_size_t(meta[0].size), meta[1].ctypes.data_as(u32p),
+            meta[2].ctypes.data_as(u32p), meta[3].ctypes.data_as(u32p), C.c_size_t(B), C.c_size_t(Cc),
+            C.c_size_t(H), C.c_size_t(Hkv), C.c_size_t(D), C.c_size_t(P), C.c_size_t(steps),
+            C.byref(ms), C.byref(wall_s))
+        if not ok:
+            raise RuntimeError("prefill loop failed: " + exe.lastError())
+        return ms.value, wall_s.value
+
+    steps = min(args.steps, 200)
+    loop(max(1, min(args.warmup, 10)))
+    ev_ms, wall = loop(steps)
+    flops = 4 * D * H * B * sum(ctx + i + 1 for i in range(Cc))  # exact causal count
+    tflops = flops / (wall / steps) / 1e12
+    ach = flops / (ev_ms / steps * 1e-3) / 1e12
+    kv_bytes = B * (ctx + Cc) * 4 * Hkv * D
+    result = {
+        "metric": "chunked-prefill paged attention TFLOP/s (exact causal FLOPs), config 5",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": steps,
+        "warmup": min(args.warmup, 10), "ms_per_step": round(wall / steps * 1e3, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 (fp16 q/K/V, MFMA with fp32 accumulate, fp32 output)", "data": "synthetic",
+        "config": {"workload": f"cfg5_chunked_prefill: batch {B}, {Cc}-row chunk after {ctx} cached "
+                               f"tokens, {H}q/{Hkv}kv heads, head_dim {D}, {P}-token pages",
+                   "flop_per_step": flops, "kv_bytes_per_step": kv_bytes},
+        "roofline": {"bound": "mfma", "achieved": round(ach, 2), "peak": MFMA_F16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(ach / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
+                     "us_per_launch": round(ev_ms / steps * 1e3, 2)},
+    }
+    if not args.no_cpu:
+        from oracle import paged_oracle as po
+        sub = dict(w)
+        sub.update(B=1)
+        for k_ in ("q",):
+            sub[k_] = w["q"].reshape(B, -1)[0]
+        sub["flat"] = w["flat"][w["off"][0]:w["off"][1]]
+        sub["off"] = np.array([0, sub["flat"].size], np.uint32)
+        sub["seq"], sub["q_start"] = w["seq"][:1], w["q_start"][:1]
+        rows = 8   # bounded sample: the first 8 chunk rows of request 0, all heads, one thread
+        sub["C"] = rows
+        sub["q"] = np.ascontiguousarray(w["q"].reshape(B, Cc, H * D)[0, :rows]).ravel()
+        t0 = time.perf_counter()
+        want = oracle(sub, n_threads=1)
+        dt = time.perf_counter() - t0
+        f_s = 4 * D * H * sum(ctx + i + 1 for i in range(rows))
+        got = np.empty((B, Cc, H, D), np.float32)
+        exe.downloadFromBuffer(ob, got)
+        rep = po.per_head_report(got[0, :rows], want[0], D)
+        result["cpu_baseline"] = {"value": round(f_s / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1,
+                                  "kind": "port",
+                                  "sample": f"{rows} of {Cc} chunk rows of request 0 (all heads), {dt:.2f} s"}
+        result["parity_vs_cpu_baseline"] = {"min_cosine": round(rep["min_cosine"], 7),
+                                            "max_abs": float(f"{rep['max_abs']:.3e}")}
+    print(json.dumps(result))
+    return 0
 
 
 def build_workload(name: str):
@@ -98,7 +209,8 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=100)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4"])
+    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "copy"])
+    ap.add_argument("--copy-mib", type=int, default=32, help="size of the calibration copy")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU baseline work")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--target-items", type=int, default=0)
@@ -107,6 +219,11 @@ def main() -> int:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); "
               "use --gpus 1", file=sys.stderr)
         return 2
+
+    if args.workload == "cfg5":
+        return bench_prefill(args)
+    if args.workload == "copy":
+        return bench_copy(args)
 
     from mlcompiler_amd import HipExecutor
     exe = HipExecutor.Instance()

@@ -3,7 +3,8 @@
   libmlc_hip.so       HIP kernels + the C ABI declared in include/mlc_hip.h
   libhip_executor.so  the C++ HipExecutor class (mirror of the reference's
                       MetalExecutor paged-path methods) on top of that ABI
-  libmlc_bench.so     native benchmark loop that calls the ABI (no kernels)
+  libmlc_bench.so     native benchmark loops that call the ABI, plus a plain copy kernel
+                      used to calibrate the HBM traffic counters
 """
 from __future__ import annotations
 
@@ -58,7 +59,7 @@ def build_all(verbose: bool = False) -> None:
     _run([cc, "--offload-arch=gfx950", "-shared", "-fPIC", *[j[1] for j in jobs], "-o", LIB_PATH])
     _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", os.path.join(CSRC, "hip_executor.cpp"),
           "-o", EXECUTOR_LIB_PATH, "-L" + CSRC, "-lmlc_hip", "-Wl,-rpath,$ORIGIN"])
-    _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", os.path.join(CSRC, "bench_loop.cpp"),
+    _run([cc, *HIPCC_FLAGS, "-shared", "-x", "hip", os.path.join(CSRC, "bench_loop.cpp"),
           "-o", BENCH_LIB_PATH, "-L" + CSRC, "-lmlc_hip", "-Wl,-rpath,$ORIGIN"])
     if verbose:
         print("built", LIB_PATH, EXECUTOR_LIB_PATH, BENCH_LIB_PATH)

@@ -6,7 +6,17 @@
 #include <cstddef>
 #include <cstdint>
 
+#include <hip/hip_runtime.h>
+
 #include "../../include/mlc_hip.h"
+
+// Plain streaming copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE counters are
+// scaled by, and the practical HBM ceiling quoted beside the decode kernel.
+__global__ __launch_bounds__(256) void mlc_bench_copy_kernel(const uint4* __restrict__ src,
+                                                             uint4* __restrict__ dst, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256)
+        dst[i] = src[i];
+}
 
 extern "C" {
 
@@ -98,6 +108,23 @@ int mlc_bench_prefill_loop(const void* q_f16, const void* k_pages, const void* v
     const auto t1 = std::chrono::steady_clock::now();
     if (event_ms) *event_ms = ms;
     if (wall_s) *wall_s = std::chrono::duration<double>(t1 - t0).count();
+    return 1;
+}
+
+// `steps` launches of the copy kernel over `bytes` bytes (src and dst are device buffers of
+// that size), on the library's stream; reports the HIP-event time in milliseconds.
+int mlc_bench_copy_loop(const void* src, void* dst, size_t bytes, size_t steps, float* event_ms) {
+    hipStream_t stream = static_cast<hipStream_t>(mlc_hip_stream());
+    if (!stream || !src || !dst) return 0;
+    const size_t n = bytes / 16;
+    const unsigned grid = (unsigned)((n + 255) / 256 < 65536 * 4 ? (n + 255) / 256 : 65536 * 4);
+    if (!mlc_hip_timer_start()) return 0;
+    for (size_t i = 0; i < steps; ++i)
+        hipLaunchKernelGGL(mlc_bench_copy_kernel, dim3(grid), dim3(256), 0, stream,
+                           static_cast<const uint4*>(src), static_cast<uint4*>(dst), n);
+    const float ms = mlc_hip_timer_stop();
+    if (ms < 0.f) return 0;
+    if (event_ms) *event_ms = ms;
     return 1;
 }
 
