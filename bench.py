@@ -71,6 +71,8 @@ def bench_prefill(args) -> int:
     from test_paged_prefill_gpu import make_prefill, oracle
     exe = HipExecutor.Instance()
     exe.requireAvailable()
+    if args.prefill_stages and not exe.setOption("prefill_stages", args.prefill_stages):
+        raise SystemExit("bench.py: --prefill-stages must be 2, 4, 6 or 8")
     B, Cc, H, Hkv, D, P, ctx = 8, 256, 32, 8, 128, 64, 3840
     w = make_prefill(B, Cc, H, Hkv, D, P, [ctx] * B, seed=55)
     bufs = [exe.allocateScratchBuffer(w[n].nbytes) for n in ("q", "k", "v")]
@@ -214,6 +216,7 @@ def main() -> int:
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU baseline work")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--target-items", type=int, default=0)
+    ap.add_argument("--prefill-stages", type=int, default=0, help="cfg5: LDS pipeline depth (0 = automatic)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); "

@@ -167,6 +167,7 @@ int mlc_hip_last_decode_work_items(void);
  *   "decode_pv_fp16"        1 = softmax weights rounded to fp16 for the P.V product
  *                           (v_dot2_f32_f16, fp32 accumulate), 0 = fp32 weights
  *   "decode_force_generic"  1 = always use the shape-agnostic kernel
+ *   "prefill_stages"        2, 4, 6 or 8 K/V tiles staged in LDS by the prefill kernel (0 = automatic)
  * Returns 0 for an unknown name or value. */
 int mlc_hip_set_option(const char* name, long value);
 

@@ -96,6 +96,7 @@ struct Ctx {
     long opt_hpw_max = 0;                                      // query heads per wave, at most (0 = automatic)
     long opt_buffers = 0;                                      // LDS staging buffers per workgroup (1, 2; 0 = automatic)
     long opt_tile_rows = 1;                                    // wave rows that share an item's tiles
+    long opt_prefill_stages = 0;                               // LDS pipeline depth of the prefill kernel (0 = automatic)
     long opt_pv_fp16 = 1;                                      // softmax weights rounded to fp16 for P.V
     int last_launches = 0;
     int last_items = 0;
@@ -804,7 +805,8 @@ int mlc_hip_paged_attn_prefill(const void* q_f16, const void* k_pages, const voi
     a.kv_heads = (uint32_t)kv_heads;
     a.page_size = (uint32_t)page_size_tokens;
     a.scale_log2e = (1.0f / std::sqrt(static_cast<float>(head_dim))) * 1.44269504088896340736f;
-    launch_prefill(a, head_dim, g.stream);
+    a.row_blocks = 0;  // set by the launcher
+    launch_prefill(a, head_dim, (int)g.opt_prefill_stages, g.stream);
     if (!slot_mark(s)) return 0;
     return finish(sync);
 }
@@ -834,6 +836,11 @@ int mlc_hip_set_option(const char* name, long value) {
     if (!std::strcmp(name, "decode_target_items")) { g.opt_target_items = value; return 1; }
     if (!std::strcmp(name, "decode_force_generic")) { g.opt_force_generic = value; return 1; }
     if (!std::strcmp(name, "decode_pv_fp16")) { g.opt_pv_fp16 = value ? 1 : 0; return 1; }
+    if (!std::strcmp(name, "prefill_stages")) {
+        if (value != 0 && value != 2 && value != 4 && value != 6 && value != 8) return 0;
+        g.opt_prefill_stages = value;
+        return 1;
+    }
     if (!std::strcmp(name, "decode_buffers")) {
         if (value != 0 && value != 1 && value != 2) return 0;
         g.opt_buffers = value;
