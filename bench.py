@@ -358,7 +358,7 @@ def main() -> int:
             "traffic": traffic,
             "us_per_launch": round(ev_us, 3),
             "note": "HIP events around the timed region on the library stream / steps: one step = "
-                    "decode kernel (+ split-K merge kernel when requests are split)",
+                    "decode kernel (split requests are merged inside it by the last workgroup to arrive)",
         },
     }
     if not args.no_cpu:

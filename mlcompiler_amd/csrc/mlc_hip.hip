@@ -224,9 +224,10 @@ int build_plan(const uint32_t* flat, size_t n_flat, const uint32_t* off, const u
     const size_t G = H / Hkv;
     if (p.fast) {
         // query heads per wave (power of two dividing G), waves per workgroup = G / that
-        // Measured on MI355X: a wave issues one VALU instruction every ~5 cycles and a SIMD
-        // needs two or more waves in flight to use its ALUs, so wide GQA groups are spread
-        // over four waves (2 heads each); narrower groups keep 4 heads per wave.
+        // Chosen by sweep on MI355X: wide GQA groups (8 query heads per KV head) run fastest
+        // spread over four waves of 2 heads each (more waves to hide the latency of short
+        // items); narrower groups keep 4 heads per wave, which shares the per-tile softmax
+        // and packing work over more heads.
         const long hpw_cap = g.opt_hpw_max > 0 ? g.opt_hpw_max : (G >= 8 ? 2 : 4);
         int hpw = 8;
         while (hpw > 1 && (hpw > hpw_cap || (G % (size_t)hpw) != 0)) hpw >>= 1;
@@ -296,7 +297,11 @@ int build_plan(const uint32_t* flat, size_t n_flat, const uint32_t* off, const u
                     it.tok_end = (uint32_t)std::min<size_t>((s + 1) * per * tile, limits[r]);
                     it.part_first = first_part;
                     it.split = (uint32_t)s | ((uint32_t)ns_eff << 16);
-                    std::memset(it.pad, 0, sizeof(it.pad));
+                    for (size_t i = 0; i < 4; ++i) {
+                        const size_t tok = (size_t)it.tok_begin + i * tile;
+                        it.first_pages[i] = tok < it.tok_end ? flat[off[r] + tok / P] : 0u;
+                    }
+                    it.pad = 0;
                     items.push_back(it);
                 }
             }

@@ -51,7 +51,9 @@ struct DecodeWorkItem {
     uint32_t tok_end;     // one past the last visible kv position of this item
     uint32_t part_first;  // first partial slot of this (request, kv head), or kNoPartial
     uint32_t split;       // this item's split index | number of splits << 16
-    uint32_t pad[5];
+    uint32_t first_pages[4];  // page ids of the item's first four tiles: the first tile loads
+                              // then depend on the item alone, not on a page-table fetch
+    uint32_t pad;
 };
 static_assert(sizeof(DecodeWorkItem) == 48, "work items are uploaded as raw bytes");
 static constexpr uint32_t kNoPartial = 0xFFFFFFFFu;
@@ -176,7 +178,7 @@ __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const D
     // The item is read once, into scalar registers: any vector load issued after the tile
     // loads would have to wait for them (loads return in order).
     struct {
-        uint32_t req, kv_head, pt_base, tok_begin, tok_end, part_first, split;
+        uint32_t req, kv_head, pt_base, tok_begin, tok_end, part_first, split, pg[4];
     } it;
     {
         const DecodeWorkItem* gi = a.items + item_idx;
@@ -187,6 +189,8 @@ __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const D
         it.tok_end = __builtin_amdgcn_readfirstlane(gi->tok_end);
         it.part_first = __builtin_amdgcn_readfirstlane(gi->part_first);
         it.split = __builtin_amdgcn_readfirstlane(gi->split);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) it.pg[i] = __builtin_amdgcn_readfirstlane(gi->first_pages[i]);
     }
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);  // wave-uniform, in an SGPR
     const int lane = threadIdx.x % 64;
@@ -197,6 +201,15 @@ __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const D
     const int c7 = c & 7;
     const int gsw = c7 ^ ((c7 & 4) ? 3 : 0);  // row-group swizzle g(c)
     const uint32_t head0 = it.kv_head * G + hg * HPW;
+
+    // An item without visible tokens (only a request of length 0 makes one; it is never
+    // split) writes its zeros and leaves before anything is loaded.
+    if (it.tok_end == it.tok_begin) {
+        float* orow = a.o + ((size_t)it.req * a.num_heads + head0) * D;
+        if (wave < NW)
+            for (int i = lane; i < HPW * D; i += 64) orow[i] = 0.f;
+        return;
+    }
 
     // q for this wave's heads, dims c*8 .. c*8+7 (issued before the tile loads, so that waiting
     // for it does not wait for them).
@@ -244,22 +257,32 @@ __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const D
             }
         }
     };
-    // Page ids of this wave's tiles (tile sub + i*NS in lane i), fetched 64 steps at a time
-    // and before the tile loads for the same reason as q.
+    // Page ids: the first four tiles' come with the item, later ones are fetched 64 steps at a
+    // time (tile sub + i*NS in lane i) -- the first batch after this wave's first tile loads
+    // were issued, later batches when nothing else is in flight.
     uint32_t page_vec = 0;
     auto fetch_pages = [&](uint32_t step0) {
         const uint32_t t = (step0 + lane) * NS + sub;
         page_vec = 0;
         if (t < n_tiles) page_vec = a.pt_flat[it.pt_base + (it.tok_begin + t * TT) / a.page_size];
     };
+    // (selected without indexing: a runtime index would move the item to scratch memory)
+    const uint32_t pg0 = (NS == 2 && sub) ? it.pg[1] : it.pg[0];
+    const uint32_t pg1 = (NS == 2) ? (sub ? it.pg[3] : it.pg[2]) : it.pg[1];
     auto page_of_step = [&](uint32_t step) {
+        if (step == 0) return pg0;
+        if (step == 1) return pg1;
         return (uint32_t)__builtin_amdgcn_readlane((int)page_vec, (int)(step & 63u));
     };
-    fetch_pages(0);
-    const uint32_t pg0 = page_of_step(0), pg1 = page_of_step(1);  // waits for the fetch here
+    static_assert(2 * NS <= 4, "the item carries the page ids of the first two steps");
 
+    // Order of the first loads: q, page ids (long items only), tile 0, tile 1.  The wait that
+    // precedes the first use of q or of tile 0 then leaves exactly tile 1 in flight; tile 0 is
+    // issued unconditionally (NS == 1) because a conditional load here would turn that wait
+    // into a wait for everything.
     const bool have1 = NBUF == 2 && (uint32_t)(NS + sub) < n_tiles;
-    if ((uint32_t)sub < n_tiles) issue_tile(sub, stage0, pg0);
+    if (n_tiles > 2u * NS) fetch_pages(0);
+    if (NS == 1 || (uint32_t)sub < n_tiles) issue_tile(sub, stage0, pg0);
     if (have1) issue_tile(NS + sub, stage1, pg1);
 
 #pragma unroll

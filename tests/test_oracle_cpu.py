@@ -386,28 +386,9 @@ def test_requests_get_disjoint_pages():
     assert not (tables[0] & tables[1]) and not (tables[0] & tables[2]) and not (tables[1] & tables[2])
 
 
-@needs_ref
-def test_allocator_transcript_matches_reference_build():
-    """Replays a random script through the reference's PagePool/RequestKVState (compiled from
-    compiler/runtime/paged_kv.cpp) and through the oracle, and compares every reply."""
-    rng = np.random.default_rng(99)
-    script = ["pool 24", "req 4"]
-    for _ in range(300):
-        r = rng.random()
-        if r < 0.55:
-            script.append("extend")
-        elif r < 0.65:
-            script.append(f"reserve {int(rng.integers(0, 40))}")
-        elif r < 0.8:
-            script.append(f"locate {int(rng.integers(0, 50))}")
-        elif r < 0.9:
-            script.append("total")
-        elif r < 0.95:
-            script.append("release_all")
-        else:
-            script.append("stats")
-    ref_out = subprocess.run([po.REF_ALLOC_DRIVER], input="\n".join(script) + "\n", text=True,
-                             capture_output=True, check=True).stdout.split("\n")
+def replay_allocator_script(script):
+    """Runs a PagePool / RequestKVState command script through the oracle and returns its
+    replies in the text form of oracle/ref_alloc_driver.cpp."""
     pool, st, mine = None, None, []
     for line in script:
         cmd, *arg = line.split()
@@ -434,4 +415,30 @@ def test_allocator_transcript_matches_reference_build():
             mine.append("ok")
         elif cmd == "stats":
             mine.append(f"{pool.pages_in_use()} {pool.pages_free()}")
+    return mine
+
+
+@needs_ref
+def test_allocator_transcript_matches_reference_build():
+    """Replays a random script through the reference's PagePool/RequestKVState (compiled from
+    compiler/runtime/paged_kv.cpp) and through the oracle, and compares every reply."""
+    rng = np.random.default_rng(99)
+    script = ["pool 24", "req 4"]
+    for _ in range(300):
+        r = rng.random()
+        if r < 0.55:
+            script.append("extend")
+        elif r < 0.65:
+            script.append(f"reserve {int(rng.integers(0, 40))}")
+        elif r < 0.8:
+            script.append(f"locate {int(rng.integers(0, 50))}")
+        elif r < 0.9:
+            script.append("total")
+        elif r < 0.95:
+            script.append("release_all")
+        else:
+            script.append("stats")
+    ref_out = subprocess.run([po.REF_ALLOC_DRIVER], input="\n".join(script) + "\n", text=True,
+                             capture_output=True, check=True).stdout.split("\n")
+    mine = replay_allocator_script(script)
     assert mine == ref_out[:len(mine)]
