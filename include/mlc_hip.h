@@ -126,6 +126,43 @@ int mlc_hip_gather_kv_pages(const void* page_storage,
                             size_t page_size_tokens, size_t n_kv_heads, size_t head_dim,
                             size_t num_tokens, void* dst, size_t dtype_bytes);
 
+/* The step before the KV write.  MetalExecutor::encodeQkvSplitRopeCast
+ * (metal_runtime.hpp:540-547, metal_runtime.mm:7915-8025; kernels
+ * strided_copy_f32 :447-455, batched_rope :287-314, cast_f32_to_f16 :457-464):
+ *   q[r][:]  = rope(qkv[r][0 : q_rows])                    fp32 [batch][q_rows]
+ *   k[r][:]  = rope(qkv[r][q_rows : q_rows+k_rows])        fp32 [batch][k_rows]
+ *   v[r][:]  =      qkv[r][q_rows+k_rows : ... + v_rows]   fp32 [batch][v_rows]
+ *   k_f16 = half(k), v_f16 = half(v)   (round to nearest even, as MSL half())
+ * rope rotates pairs (2p, 2p+1), p < rotary_dim/2, of every head with
+ * cos_buf/sin_buf [batch][rotary_dim/2] (fp32, device): x0*c - x1*s, x0*s + x1*c,
+ * each product and sum rounded on its own as in the CPU
+ * applyRotaryEmbedding (compiler/runtime/quantization.cpp:772-793).
+ * rotary_dim == 0 skips it.  sync = 0 needs an open pass (the reference form),
+ * sync = 1 waits.  One launch instead of the reference's seven dispatches. */
+int mlc_hip_qkv_split_rope_cast(const void* qkv, void* q, void* k, void* v,
+                                void* k_f16, void* v_f16,
+                                const void* cos_buf, const void* sin_buf,
+                                size_t batch, size_t num_heads, size_t kv_heads, size_t head_dim,
+                                size_t qkv_rows, size_t q_rows, size_t k_rows, size_t v_rows,
+                                size_t rotary_dim, int sync);
+
+/* The same step fused with the two scatter_kv_paged_batched_f16 calls that
+ * follow it in the walker (compiler/runtime/batched_walker.cpp:287-331): the
+ * fp16 K and V rows go straight to page page_ids[r], slot slots_in_page[r] of
+ * k_pages / v_pages (layout and index formula of metal_runtime.mm:405-424), so
+ * the fp16 staging buffers and two launches disappear.  k_f32 / v_f32 may be
+ * NULL when the caller does not need the fp32 copies.  No single counterpart
+ * in the reference; results are bit-identical to
+ * mlc_hip_qkv_split_rope_cast followed by two batched scatters. */
+int mlc_hip_qkv_split_rope_scatter(const void* qkv, void* q, void* k_pages, void* v_pages,
+                                   void* k_f32, void* v_f32,
+                                   const void* cos_buf, const void* sin_buf,
+                                   const uint32_t* page_ids, const uint32_t* slots_in_page,
+                                   size_t page_size_tokens,
+                                   size_t batch, size_t num_heads, size_t kv_heads, size_t head_dim,
+                                   size_t qkv_rows, size_t q_rows, size_t k_rows, size_t v_rows,
+                                   size_t rotary_dim, int sync);
+
 /* Chunked prefill over paged KV (MFMA path).  No counterpart in the reference,
  * which prefills by looping the decode path once per prompt token
  * (compiler/runtime/batched_executor.cpp:454-466); semantics are the decode

@@ -34,6 +34,8 @@ SIGNATURES = {
                                                        C.c_int]),
     "mlc_hip_scatter_kv_paged": (C.c_int, [_vp, _u32p, _sz, _sz, _sz, _sz, _sz, _sz, _vp, _sz]),
     "mlc_hip_gather_kv_pages": (C.c_int, [_vp, _u32p, _sz, _sz, _sz, _sz, _sz, _vp, _sz]),
+    "mlc_hip_qkv_split_rope_cast": (C.c_int, [_vp] * 8 + [_sz] * 9 + [C.c_int]),
+    "mlc_hip_qkv_split_rope_scatter": (C.c_int, [_vp] * 8 + [_u32p, _u32p] + [_sz] * 10 + [C.c_int]),
     "mlc_hip_paged_attn_prefill": (C.c_int, [_vp, _vp, _vp, _vp, _u32p, _sz, _u32p, _u32p, _u32p,
                                              _sz, _sz, _sz, _sz, _sz, _sz, C.c_int]),
     "mlc_hip_stream": (_vp, []),

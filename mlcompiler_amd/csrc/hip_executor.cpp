@@ -109,6 +109,34 @@ bool HipExecutor::gatherKVPages(void* page_storage_buffer, const std::vector<uin
                                    num_tokens, dst_buffer, dtype_bytes) != 0;
 }
 
+bool HipExecutor::encodeQkvSplitRopeCast(void* qkv_buf, void* q_buf, void* k_buf, void* v_buf,
+                                         void* k_f16_buf, void* v_f16_buf, void* cos_buf,
+                                         void* sin_buf, size_t batch, size_t num_heads,
+                                         size_t kv_heads, size_t head_dim, size_t qkv_rows,
+                                         size_t q_rows, size_t k_rows, size_t v_rows,
+                                         size_t rotary_dim) const {
+    return mlc_hip_qkv_split_rope_cast(qkv_buf, q_buf, k_buf, v_buf, k_f16_buf, v_f16_buf, cos_buf,
+                                       sin_buf, batch, num_heads, kv_heads, head_dim, qkv_rows,
+                                       q_rows, k_rows, v_rows, rotary_dim, /*sync=*/0) != 0;
+}
+
+bool HipExecutor::encodeQkvSplitRopeScatter(void* qkv_buf, void* q_buf, void* k_pages_buffer,
+                                            void* v_pages_buffer, void* k_f32_buf, void* v_f32_buf,
+                                            void* cos_buf, void* sin_buf,
+                                            const std::vector<uint32_t>& page_ids,
+                                            const std::vector<uint32_t>& slots_in_page,
+                                            size_t page_size_tokens, size_t batch, size_t num_heads,
+                                            size_t kv_heads, size_t head_dim, size_t qkv_rows,
+                                            size_t q_rows, size_t k_rows, size_t v_rows,
+                                            size_t rotary_dim) const {
+    if (page_ids.size() < batch || slots_in_page.size() < batch) return false;
+    return mlc_hip_qkv_split_rope_scatter(qkv_buf, q_buf, k_pages_buffer, v_pages_buffer, k_f32_buf,
+                                          v_f32_buf, cos_buf, sin_buf, page_ids.data(),
+                                          slots_in_page.data(), page_size_tokens, batch, num_heads,
+                                          kv_heads, head_dim, qkv_rows, q_rows, k_rows, v_rows,
+                                          rotary_dim, /*sync=*/0) != 0;
+}
+
 bool HipExecutor::runPagedPrefillAttention(void* q_f16_buffer, void* k_pages_buffer,
                                            void* v_pages_buffer, void* o_buffer,
                                            const std::vector<uint32_t>& page_tables_flat,

@@ -71,6 +71,24 @@ public:
                                size_t page_size_tokens, size_t n_kv_heads, size_t head_dim,
                                size_t batch, const void* src_buffer) const;
 
+    // metal_runtime.hpp:540-547 (needs an open pass, like every encode* method)
+    bool encodeQkvSplitRopeCast(void* qkv_buf, void* q_buf, void* k_buf, void* v_buf,
+                                void* k_f16_buf, void* v_f16_buf, void* cos_buf, void* sin_buf,
+                                size_t batch, size_t num_heads, size_t kv_heads, size_t head_dim,
+                                size_t qkv_rows, size_t q_rows, size_t k_rows, size_t v_rows,
+                                size_t rotary_dim) const;
+
+    // The same step fused with the two batched KV scatters that follow it in the walker
+    // (batched_walker.cpp:287-331); k_f32_buf / v_f32_buf may be null.  No reference method.
+    bool encodeQkvSplitRopeScatter(void* qkv_buf, void* q_buf, void* k_pages_buffer,
+                                   void* v_pages_buffer, void* k_f32_buf, void* v_f32_buf,
+                                   void* cos_buf, void* sin_buf,
+                                   const std::vector<uint32_t>& page_ids,
+                                   const std::vector<uint32_t>& slots_in_page,
+                                   size_t page_size_tokens, size_t batch, size_t num_heads,
+                                   size_t kv_heads, size_t head_dim, size_t qkv_rows, size_t q_rows,
+                                   size_t k_rows, size_t v_rows, size_t rotary_dim) const;
+
     // Chunked prefill over paged KV: no reference method (the reference loops its
     // decode path per prompt token, batched_executor.cpp:454-466).
     bool runPagedPrefillAttention(void* q_f16_buffer, void* k_pages_buffer, void* v_pages_buffer,

@@ -157,6 +157,30 @@ class HipExecutor:
             page_storage_buffer, _ptr(pt_arg), pt.size, page_size_tokens, n_kv_heads, head_dim,
             num_tokens, dst_buffer, dtype_bytes))
 
+    # -- the step before the KV write (metal_runtime.hpp:540-547, metal_runtime.mm:7915-8025)
+    def encodeQkvSplitRopeCast(self, qkv_buf, q_buf, k_buf, v_buf, k_f16_buf, v_f16_buf, cos_buf,
+                               sin_buf, batch, num_heads, kv_heads, head_dim, qkv_rows, q_rows,
+                               k_rows, v_rows, rotary_dim, sync: bool = False) -> bool:
+        return bool(self._lib.mlc_hip_qkv_split_rope_cast(
+            qkv_buf, q_buf, k_buf, v_buf, k_f16_buf, v_f16_buf, cos_buf, sin_buf, batch, num_heads,
+            kv_heads, head_dim, qkv_rows, q_rows, k_rows, v_rows, rotary_dim, int(bool(sync))))
+
+    # the same step fused with the two batched scatters that follow it in the walker
+    # (batched_walker.cpp:287-331); no single reference method
+    def encodeQkvSplitRopeScatter(self, qkv_buf, q_buf, k_pages_buffer, v_pages_buffer, cos_buf,
+                                  sin_buf, page_ids, slots_in_page, page_size_tokens, batch,
+                                  num_heads, kv_heads, head_dim, qkv_rows, q_rows, k_rows, v_rows,
+                                  rotary_dim, k_f32_buf=None, v_f32_buf=None,
+                                  sync: bool = False) -> bool:
+        ids = _u32(page_ids)
+        sl = _u32(slots_in_page)
+        if ids.size != batch or sl.size != batch:
+            return False
+        return bool(self._lib.mlc_hip_qkv_split_rope_scatter(
+            qkv_buf, q_buf, k_pages_buffer, v_pages_buffer, k_f32_buf, v_f32_buf, cos_buf, sin_buf,
+            _ptr(ids), _ptr(sl), page_size_tokens, batch, num_heads, kv_heads, head_dim, qkv_rows,
+            q_rows, k_rows, v_rows, rotary_dim, int(bool(sync))))
+
     # -- chunked prefill (no reference method; see include/mlc_hip.h)
     def runPagedPrefillAttention(self, q_f16_buffer, k_pages_buffer, v_pages_buffer, o_buffer,
                                  page_tables_flat, page_table_offsets, seq_lens, q_start, batch,

@@ -188,6 +188,66 @@ int oracle_gather_kv_pages(const void* page_storage,
     return 1;
 }
 
+/* ------------------------------------------------- qkv split + RoPE + cast */
+
+size_t oracle_rotary_coefficients(size_t position, size_t rotary_dim, float freq_base,
+                                  float freq_scale, float* cos_out, float* sin_out) {
+    /* quantization.cpp:801-822 */
+    if (rotary_dim < 2) return 0;
+    if (freq_base <= 0.0f) freq_base = 10000.0f;
+    if (freq_scale == 0.0f) freq_scale = 1.0f;
+    size_t pairs = rotary_dim / 2;
+    float pos = (float)position;
+    for (size_t i = 0; i < pairs; ++i) {
+        float exponent = (float)(2 * i) / (float)rotary_dim;
+        float inv_freq = powf(freq_base, -exponent);
+        float angle = pos * inv_freq * freq_scale;
+        cos_out[i] = cosf(angle);
+        sin_out[i] = sinf(angle);
+    }
+    return pairs;
+}
+
+int oracle_qkv_split_rope_cast(const float* qkv, float* q, float* k, float* v,
+                               uint16_t* k_f16, uint16_t* v_f16,
+                               const float* cos_table, const float* sin_table,
+                               size_t batch, size_t num_heads, size_t kv_heads, size_t head_dim,
+                               size_t qkv_rows, size_t q_rows, size_t k_rows, size_t v_rows,
+                               size_t rotary_dim) {
+    if (!qkv || !q || !k || !v || !k_f16 || !v_f16) return 0;
+    if (batch == 0 || num_heads == 0 || kv_heads == 0 || head_dim == 0) return 0;
+    if (q_rows + k_rows + v_rows > qkv_rows) return 0;
+    if (q_rows != num_heads * head_dim || k_rows != kv_heads * head_dim) return 0;
+    if (rotary_dim > head_dim || (rotary_dim & 1)) return 0;
+    if (rotary_dim > 0 && (!cos_table || !sin_table)) return 0;
+    /* split: metal_runtime.mm:447-455 with offsets 0, q_rows, q_rows + k_rows (:7962-7964) */
+    for (size_t r = 0; r < batch; ++r) {
+        memcpy(q + r * q_rows, qkv + r * qkv_rows, q_rows * sizeof(float));
+        memcpy(k + r * k_rows, qkv + r * qkv_rows + q_rows, k_rows * sizeof(float));
+        memcpy(v + r * v_rows, qkv + r * qkv_rows + q_rows + k_rows, v_rows * sizeof(float));
+    }
+    /* rope on q (num_heads) and k (kv_heads): metal_runtime.mm:287-314, :7989-7990 */
+    const size_t pairs = rotary_dim / 2;
+    for (int which = 0; which < 2 && pairs; ++which) {
+        float* data = which ? k : q;
+        const size_t nh = which ? kv_heads : num_heads;
+        for (size_t r = 0; r < batch; ++r)
+            for (size_t h = 0; h < nh; ++h)
+                for (size_t p = 0; p < pairs; ++p) {
+                    float* x = data + (r * nh + h) * head_dim + 2 * p;
+                    const float c = cos_table[r * pairs + p], s = sin_table[r * pairs + p];
+                    const float x0 = x[0], x1 = x[1];
+                    const float a0 = x0 * c, a1 = x1 * s, b0 = x0 * s, b1 = x1 * c;
+                    x[0] = a0 - a1;
+                    x[1] = b0 + b1;
+                }
+    }
+    /* casts: metal_runtime.mm:457-464, :8009-8010 */
+    oracle_float_to_fp16_rne_n(k, k_f16, batch * k_rows);
+    oracle_float_to_fp16_rne_n(v, v_f16, batch * v_rows);
+    return 1;
+}
+
 /* ------------------------------------------------------------- attention */
 
 static int attention_args_ok(const void* q, const void* k, const void* v, const void* o,

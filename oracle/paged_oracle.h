@@ -92,6 +92,33 @@ int oracle_gather_kv_pages(const void* page_storage,
                            size_t head_dim, size_t num_tokens,
                            void* dst, size_t dtype_bytes);
 
+/* The step before the KV write: split one fused qkv row per request into q, k, v
+ * (strided_copy_f32, compiler/runtime/metal_runtime.mm:447-455), rotate q and k
+ * in place (batched_rope :287-314; same arithmetic as the CPU
+ * applyRotaryEmbedding, compiler/runtime/quantization.cpp:772-793: pair
+ * (2p, 2p+1) -> (x0*c - x1*s, x0*s + x1*c), every product and sum rounded to
+ * fp32 on its own), and cast k and v to fp16 with round-to-nearest-even
+ * (cast_f32_to_f16 :457-464, `half(x)`), in the order of
+ * MetalExecutor::encodeQkvSplitRopeCast (:7915-8025).
+ *   qkv [batch][qkv_rows]; q [batch][q_rows]; k [batch][k_rows]; v [batch][v_rows];
+ *   cos, sin [batch][rotary_dim/2]; k_f16, v_f16 like k, v.
+ * rotary_dim == 0 skips the rotation (cos/sin may be NULL).  Returns 0 when a
+ * buffer is missing or the row counts do not fit (q_rows + k_rows + v_rows >
+ * qkv_rows, q_rows != num_heads*head_dim, k_rows != kv_heads*head_dim,
+ * rotary_dim > head_dim or odd). */
+int oracle_qkv_split_rope_cast(const float* qkv, float* q, float* k, float* v,
+                               uint16_t* k_f16, uint16_t* v_f16,
+                               const float* cos_table, const float* sin_table,
+                               size_t batch, size_t num_heads, size_t kv_heads, size_t head_dim,
+                               size_t qkv_rows, size_t q_rows, size_t k_rows, size_t v_rows,
+                               size_t rotary_dim);
+
+/* compiler/runtime/quantization.cpp:795-823: cos/sin of position * base^(-2i/rotary_dim) * scale
+ * for i < rotary_dim/2, all in fp32 (powf, cosf, sinf).  base <= 0 -> 10000, scale == 0 -> 1.
+ * Returns the number of pairs written. */
+size_t oracle_rotary_coefficients(size_t position, size_t rotary_dim, float freq_base,
+                                  float freq_scale, float* cos_out, float* sin_out);
+
 /* The executor-CPU attention, compiler/runtime/attention_cpu.cpp:437-470
  * (per head: left-to-right dot over every cached row :99-105, softmax that
  * subtracts the max, exponentiates and divides each weight by the sum :21-33,

@@ -59,6 +59,11 @@ def lib() -> C.CDLL:
         L.oracle_scatter_kv_paged.restype = C.c_int
         L.oracle_scatter_kv_paged.argtypes = [C.c_void_p, _u32p, _sz, _sz, _sz, _sz, _sz, _sz,
                                               C.c_void_p, _sz]
+        L.oracle_qkv_split_rope_cast.restype = C.c_int
+        L.oracle_qkv_split_rope_cast.argtypes = [_f32p, _f32p, _f32p, _f32p, _u16p, _u16p, C.c_void_p,
+                                                 C.c_void_p] + [_sz] * 9
+        L.oracle_rotary_coefficients.restype = _sz
+        L.oracle_rotary_coefficients.argtypes = [_sz, _sz, C.c_float, C.c_float, _f32p, _f32p]
         L.oracle_gather_kv_pages.restype = C.c_int
         L.oracle_gather_kv_pages.argtypes = [C.c_void_p, _u32p, _sz, _sz, _sz, _sz, _sz,
                                              C.c_void_p, _sz]
@@ -170,6 +175,39 @@ def gather_kv_pages(page_storage: np.ndarray, page_table, page_size_tokens: int,
     return bool(lib().oracle_gather_kv_pages(
         ps.ctypes.data, _p(pt, _u32p), pt.size, page_size_tokens, n_kv_heads, head_dim,
         num_tokens, dst.ctypes.data, dtype_bytes))
+
+
+# ------------------------------------------------- qkv split + RoPE + cast
+
+def rotary_coefficients(position: int, rotary_dim: int, freq_base: float = 10000.0,
+                        freq_scale: float = 1.0):
+    """(cos, sin), each rotary_dim // 2 floats (quantization.cpp:795-823)."""
+    pairs = rotary_dim // 2
+    cos = np.zeros(max(pairs, 1), np.float32)
+    sin = np.zeros(max(pairs, 1), np.float32)
+    n = lib().oracle_rotary_coefficients(position, rotary_dim, freq_base, freq_scale,
+                                         _p(cos, _f32p), _p(sin, _f32p))
+    return cos[:n], sin[:n]
+
+
+def qkv_split_rope_cast(qkv, cos, sin, batch, num_heads, kv_heads, head_dim, qkv_rows, q_rows, k_rows,
+                        v_rows, rotary_dim):
+    """Returns (q, k, v, k_f16, v_f16) or None on the argument errors."""
+    qkv = _c(qkv, np.float32)
+    q = np.zeros((batch, q_rows), np.float32)
+    k = np.zeros((batch, k_rows), np.float32)
+    v = np.zeros((batch, v_rows), np.float32)
+    k16 = np.zeros((batch, k_rows), np.uint16)
+    v16 = np.zeros((batch, v_rows), np.uint16)
+    cosp = sinp = None
+    if cos is not None:
+        cos = _c(cos, np.float32)
+        sin = _c(sin, np.float32)
+        cosp, sinp = cos.ctypes.data, sin.ctypes.data
+    ok = lib().oracle_qkv_split_rope_cast(_p(qkv, _f32p), _p(q, _f32p), _p(k, _f32p), _p(v, _f32p),
+                                          _p(k16, _u16p), _p(v16, _u16p), cosp, sinp, batch, num_heads,
+                                          kv_heads, head_dim, qkv_rows, q_rows, k_rows, v_rows, rotary_dim)
+    return (q, k, v, k16, v16) if ok else None
 
 
 # ------------------------------------------------------------ attention
@@ -361,6 +399,10 @@ def ref_lib():
         R.ref_fp16_to_float_n.argtypes = [_u16p, _f32p, _sz]
         R.ref_float_to_fp16_n.restype = None
         R.ref_float_to_fp16_n.argtypes = [_f32p, _u16p, _sz]
+        R.ref_apply_rotary.restype = None
+        R.ref_apply_rotary.argtypes = [_f32p, _f32p, _f32p, _sz, _sz, _sz]
+        R.ref_rotary_coefficients.restype = _sz
+        R.ref_rotary_coefficients.argtypes = [_sz, _sz, C.c_float, C.c_float, _f32p, _f32p]
         R.ref_run_attention_cpu.restype = C.c_int
         R.ref_run_attention_cpu.argtypes = [_f32p, _u16p, _u16p, _sz, _sz, _sz, _sz, _sz, _f32p,
                                             _f32p, _f32p]
@@ -380,6 +422,22 @@ def ref_float_to_fp16(v) -> np.ndarray:
     out = np.empty(v.size, np.uint16)
     ref_lib().ref_float_to_fp16_n(_p(v, _f32p), _p(out, _u16p), v.size)
     return out
+
+
+def ref_apply_rotary(vec, cos, sin, head_dim, rotary_dim) -> np.ndarray:
+    """The reference's applyRotaryEmbedding on one head vector (returns a rotated copy)."""
+    x = np.array(vec, np.float32).ravel().copy()
+    cos, sin = _c(cos, np.float32), _c(sin, np.float32)
+    ref_lib().ref_apply_rotary(_p(x, _f32p), _p(cos, _f32p), _p(sin, _f32p), cos.size, head_dim, rotary_dim)
+    return x
+
+
+def ref_rotary_coefficients(position, rotary_dim, freq_base, freq_scale):
+    pairs = max(rotary_dim // 2, 1)
+    cos, sin = np.zeros(pairs, np.float32), np.zeros(pairs, np.float32)
+    n = ref_lib().ref_rotary_coefficients(position, rotary_dim, freq_base, freq_scale,
+                                          _p(cos, _f32p), _p(sin, _f32p))
+    return cos[:n], sin[:n]
 
 
 def ref_run_attention_cpu(q, k_cache, v_cache, heads, kv_heads, head_dim, ctx_len, position,

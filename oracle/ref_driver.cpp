@@ -5,6 +5,8 @@
 // reference is copied here: this file only includes its headers and calls
 //   mlc::runtime::RunAttentionCPU         compiler/runtime/attention_cpu.cpp:272-478
 //   mlc::runtime::fp16ToFloat/floatToFp16 compiler/runtime/float_convert.hpp:14-76
+//   mlc::runtime::applyRotaryEmbedding / computeRotaryCoefficients
+//                                         compiler/runtime/quantization.cpp:772-823
 // the way the reference's own test does (tests/test_runtime.cpp:1659-1690):
 // an ExecutionGraph with one Attention node, state tensors {Hkv, ctx, D}
 // tagged role=kv_cache so ExecutionContext stores them as F16
@@ -22,6 +24,7 @@
 #include "runtime/execution_graph.hpp"
 #include "runtime/float_convert.hpp"
 #include "runtime/operator_backend.hpp"
+#include "runtime/quantization.hpp"
 #include "runtime/session.hpp"
 
 namespace {
@@ -122,6 +125,23 @@ int ref_run_attention_cpu(const float* q, const uint16_t* k_cache, const uint16_
     } catch (...) {
         return 0;
     }
+}
+
+// applyRotaryEmbedding on one head vector (in place); n_pairs entries of cos/sin.
+void ref_apply_rotary(float* data, const float* cos, const float* sin, size_t n_pairs,
+                      size_t head_dim, size_t rotary_dim) {
+    std::vector<float> c(cos, cos + n_pairs), s(sin, sin + n_pairs);
+    mlc::runtime::applyRotaryEmbedding(data, c, s, head_dim, rotary_dim);
+}
+
+// computeRotaryCoefficients; cos/sin must hold rotary_dim / 2 floats.  Returns the pair count.
+size_t ref_rotary_coefficients(size_t position, size_t rotary_dim, float freq_base, float freq_scale,
+                               float* cos, float* sin) {
+    std::vector<float> c, s;
+    mlc::runtime::computeRotaryCoefficients(position, rotary_dim, freq_base, freq_scale, c, s);
+    std::memcpy(cos, c.data(), c.size() * sizeof(float));
+    std::memcpy(sin, s.data(), s.size() * sizeof(float));
+    return c.size();
 }
 
 }  // extern "C"

@@ -442,3 +442,92 @@ def test_allocator_transcript_matches_reference_build():
                              capture_output=True, check=True).stdout.split("\n")
     mine = replay_allocator_script(script)
     assert mine == ref_out[:len(mine)]
+
+
+# ------------------------------------------------- qkv split + RoPE + cast
+
+ROPE_VEC = [1.7640524, 0.4001572, 0.9787380, 2.2408931, 1.8675580, -0.9772779, 0.95008844, -0.1513572]
+ROPE_COS = [0.96366274, 0.3834415, 0.79172504, 0.5288949]
+ROPE_SIN = [0.56804454, 0.92559665, 0.07103606, 0.0871293]
+ROPE_EXPECTED = [1.4726444, 1.3876770, -1.6988745, 1.7651681, 1.5480144, -0.6410714, 0.5156846, 0.00272848]
+
+
+def test_rope_known_answer_of_the_reference_test():
+    """tests/test_runtime.cpp:799-818 (RotaryEmbeddingTest.CpuMatchesExpectedRotation), 1e-5."""
+    qkv = np.array(ROPE_VEC * 3, np.float32)
+    q, k, v, k16, v16 = po.qkv_split_rope_cast(qkv, ROPE_COS, ROPE_SIN, 1, 1, 1, 8, 24, 8, 8, 8, 8)
+    assert np.max(np.abs(q[0] - np.array(ROPE_EXPECTED, np.float32))) <= 1e-5
+    assert np.max(np.abs(k[0] - np.array(ROPE_EXPECTED, np.float32))) <= 1e-5
+    assert np.array_equal(v[0], np.array(ROPE_VEC, np.float32))          # v is never rotated
+    assert np.array_equal(k16[0], po.float_to_fp16_rne(k[0]))
+    assert np.array_equal(v16[0], po.float_to_fp16_rne(v[0]))
+
+
+def test_rope_split_closed_forms():
+    rng = np.random.default_rng(5)
+    B, H, Hkv, D, rot = 3, 4, 2, 16, 8
+    q_rows, k_rows, v_rows = H * D, Hkv * D, Hkv * D
+    qkv_rows = q_rows + k_rows + v_rows + 6           # padding after v is ignored
+    qkv = rng.standard_normal((B, qkv_rows)).astype(np.float32)
+    ang = rng.uniform(-3, 3, (B, rot // 2))
+    cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    q, k, v, k16, v16 = po.qkv_split_rope_cast(qkv, cos, sin, B, H, Hkv, D, qkv_rows, q_rows, k_rows,
+                                               v_rows, rot)
+    # split offsets (metal_runtime.mm:7962-7964) and untouched dims >= rotary_dim
+    assert np.array_equal(v, qkv[:, q_rows + k_rows:q_rows + k_rows + v_rows])
+    q_in = qkv[:, :q_rows].reshape(B, H, D)
+    assert np.array_equal(q.reshape(B, H, D)[:, :, rot:], q_in[:, :, rot:])
+    # rotation in float64 as the independent leg: pair norms are preserved, formula matches
+    x0, x1 = q_in[:, :, 0:rot:2].astype(np.float64), q_in[:, :, 1:rot:2].astype(np.float64)
+    c, s = cos[:, None, :].astype(np.float64), sin[:, None, :].astype(np.float64)
+    want0, want1 = x0 * c - x1 * s, x0 * s + x1 * c
+    got = q.reshape(B, H, D)
+    assert np.max(np.abs(got[:, :, 0:rot:2] - want0)) < 1e-6
+    assert np.max(np.abs(got[:, :, 1:rot:2] - want1)) < 1e-6
+    # a transposed or sign-flipped rotation would fail this: rotating by -angle undoes it
+    back = po.qkv_split_rope_cast(np.concatenate([q, k, v], axis=1), cos, -sin, B, H, Hkv, D,
+                                  q_rows + k_rows + v_rows, q_rows, k_rows, v_rows, rot)
+    assert np.max(np.abs(back[0] - qkv[:, :q_rows])) < 1e-6
+    # rotary_dim 0: pure split + cast, tables may be absent
+    q0, k0, v0, k160, _ = po.qkv_split_rope_cast(qkv, None, None, B, H, Hkv, D, qkv_rows, q_rows, k_rows,
+                                                 v_rows, 0)
+    assert np.array_equal(q0, qkv[:, :q_rows]) and np.array_equal(k0, qkv[:, q_rows:q_rows + k_rows])
+    assert np.array_equal(k160, qkv[:, q_rows:q_rows + k_rows].astype(np.float16).view(np.uint16))
+    # argument errors
+    assert po.qkv_split_rope_cast(qkv, cos, sin, B, H, Hkv, D, q_rows, q_rows, k_rows, v_rows, rot) is None
+    assert po.qkv_split_rope_cast(qkv, cos, sin, B, H, Hkv, D, qkv_rows, q_rows, k_rows, v_rows, D + 2) is None
+    assert po.qkv_split_rope_cast(qkv, None, None, B, H, Hkv, D, qkv_rows, q_rows, k_rows, v_rows, rot) is None
+
+
+def test_rotary_coefficients_closed_forms():
+    cos, sin = po.rotary_coefficients(0, 64)
+    assert np.all(cos == 1.0) and np.all(sin == 0.0)                   # position 0: identity
+    cos, sin = po.rotary_coefficients(3, 8, 10000.0, 1.0)
+    want = 3.0 * 10000.0 ** (-np.arange(4) * 2 / 8)
+    assert np.max(np.abs(cos - np.cos(want))) < 1e-6 and np.max(np.abs(sin - np.sin(want))) < 1e-6
+    # base <= 0 and scale == 0 fall back to 10000 and 1 (quantization.cpp:806-811)
+    a, b = po.rotary_coefficients(7, 16, 0.0, 0.0), po.rotary_coefficients(7, 16, 10000.0, 1.0)
+    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+    assert po.rotary_coefficients(5, 1)[0].size == 0
+
+
+@needs_ref
+def test_rope_bit_exact_with_reference_build():
+    """applyRotaryEmbedding / computeRotaryCoefficients compiled from
+    compiler/runtime/quantization.cpp:772-823."""
+    rng = np.random.default_rng(8)
+    for D, rot, pos in [(64, 64, 1234), (128, 128, 8191), (64, 32, 17), (16, 8, 3)]:
+        cos, sin = po.rotary_coefficients(pos, rot, 10000.0, 1.0)
+        rc, rs = po.ref_rotary_coefficients(pos, rot, 10000.0, 1.0)
+        assert np.array_equal(cos.view(np.uint32), rc.view(np.uint32))
+        assert np.array_equal(sin.view(np.uint32), rs.view(np.uint32))
+        H, Hkv = 4, 2
+        qkv = rng.standard_normal((H + 2 * Hkv) * D).astype(np.float32)
+        q, k, v, _, _ = po.qkv_split_rope_cast(qkv, cos, sin, 1, H, Hkv, D, qkv.size, H * D, Hkv * D,
+                                               Hkv * D, rot)
+        for h in range(H):
+            want = po.ref_apply_rotary(qkv[h * D:(h + 1) * D], cos, sin, D, rot)
+            assert np.array_equal(q[0, h * D:(h + 1) * D].view(np.uint32), want.view(np.uint32))
+        for h in range(Hkv):
+            want = po.ref_apply_rotary(qkv[(H + h) * D:(H + h + 1) * D], cos, sin, D, rot)
+            assert np.array_equal(k[0, h * D:(h + 1) * D].view(np.uint32), want.view(np.uint32))
