@@ -55,15 +55,29 @@ static constexpr int kPfKeys = 32;   // keys per tile
 static constexpr int kPfRows = 32;   // chunk rows per wave
 static constexpr int kPfWaves = 8;   // waves per workgroup
 
-__device__ __forceinline__ void pf_g2lds16(const void* g, void* lds_base) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
-                                     (__attribute__((address_space(3))) void*)lds_base, 16, 0, 0);
+// 16-byte global -> LDS load that bypasses the register file: lane i's 16 bytes land at LDS
+// byte address lds_base + 16*i (lds_base wave-uniform).  Issued as inline assembly on
+// purpose: the compiler tracks the builtin form of this load and, at the head of the tile
+// loop, waits for ALL outstanding loads before the first LDS read (it cannot prove which of
+// them target the stage being read), which would stall the pipeline once per round.  Here the
+// ordering is explicit instead: pf_wait_vmcnt + pf_barrier below.
+__device__ __forceinline__ void pf_g2lds16(const void* g, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(lds_base), "v"(g)
+                 : "memory", "m0");
 }
 
-// s_waitcnt vmcnt(N), other counters untouched (gfx9 encoding).
+// Byte address of an LDS object, as the M0 base of pf_g2lds16 wants it.
+__device__ __forceinline__ uint32_t pf_lds_addr(const void* p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
+}
+
+// s_waitcnt vmcnt(N), other counters untouched.  Also a compiler barrier for memory accesses:
+// the LDS reads that follow it depend on loads the compiler does not know about.
 template <int N>
 __device__ __forceinline__ void pf_wait_vmcnt() {
-    __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
 // Workgroup barrier that orders LDS traffic only: __syncthreads() would also wait for every
@@ -150,17 +164,23 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_prefill_mfma_kernel(const
     }
 
     const uint32_t row_elems = a.kv_heads * D;  // halves per token row (all KV heads)
-    const bool loader = tid < CHUNKS;           // wave-uniform: CHUNKS is a multiple of 64
+    // Every thread issues its two loads on every tile, unconditionally: a load under a branch
+    // would make the compiler's count of "loads issued since" uncertain and turn the partial
+    // waits below into waits for everything.  With head_dim 64 a tile has only 256 chunks per
+    // tensor, so the upper four waves repeat the lower four's loads (same bytes to the same LDS
+    // addresses).
+    const int ltid = tid % CHUNKS;          // chunk position served by this thread
+    const int lwave = wave % (CHUNKS / 64);
 
     // ---- tile loader: thread tid fetches K chunk position tid and V chunk position tid.
     // K position p (row = p / CPR, slot = p % CPR) is filled with global chunk
     // slot ^ (row % CPR) of key `row`: rows are 2*D bytes apart in LDS, the XOR spreads the 32
     // rows an MFMA operand read touches over the banks.  V position p is chunk p / 32 of key
     // p % 32.  Rows past the last key of the workgroup are clamped (in bounds, masked later).
-    const uint32_t k_row = (uint32_t)tid / CPR;
-    const uint32_t k_col = ((((uint32_t)tid % CPR) ^ (k_row % CPR)) * 8u) + kvh * D;
-    const uint32_t v_row = (uint32_t)tid % kPfKeys;
-    const uint32_t v_col = ((uint32_t)tid / kPfKeys) * 8u + kvh * D;
+    const uint32_t k_row = (uint32_t)ltid / CPR;
+    const uint32_t k_col = ((((uint32_t)ltid % CPR) ^ (k_row % CPR)) * 8u) + kvh * D;
+    const uint32_t v_row = (uint32_t)ltid % kPfKeys;
+    const uint32_t v_col = ((uint32_t)ltid / kPfKeys) * 8u + kvh * D;
     // Page ids are kept 64 at a time in one register (lane j: page 64*group + j) and picked
     // with readlane: a vector load issued between the tile loads would have to wait for all
     // of them, since loads return in order.  The register is refilled when the loader enters
@@ -180,14 +200,13 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_prefill_mfma_kernel(const
         const uint32_t page_id = __builtin_amdgcn_readlane(page_vec, page % 64u);
         const size_t tok0 = (size_t)page_id * a.page_size + key0 % a.page_size;
         const uint32_t last = wg_limit - 1u - key0;  // last valid row of the tile
-        if (loader) {
-            const uint32_t kr = k_row < last ? k_row : last;
-            const uint32_t vr = v_row < last ? v_row : last;
-            const _Float16* kbase = a.k_pages + tok0 * row_elems;
-            const _Float16* vbase = a.v_pages + tok0 * row_elems;
-            pf_g2lds16(kbase + (kr * row_elems + k_col), st + wave * 1024);
-            pf_g2lds16(vbase + (vr * row_elems + v_col), st + K_TILE + wave * 1024);
-        }
+        const uint32_t kr = k_row < last ? k_row : last;
+        const uint32_t vr = v_row < last ? v_row : last;
+        const _Float16* kbase = a.k_pages + tok0 * row_elems;
+        const _Float16* vbase = a.v_pages + tok0 * row_elems;
+        const uint32_t dst = __builtin_amdgcn_readfirstlane(pf_lds_addr(st) + lwave * 1024);
+        pf_g2lds16(kbase + (kr * row_elems + k_col), dst);
+        pf_g2lds16(vbase + (vr * row_elems + v_col), dst + K_TILE);
     };
     // ---- V transposer: the thread's own 16 bytes (key v_row, dims 8*(tid/32)..+8) go to
     // V^T[dim][pos(key)], keys of each 16-key group ordered 0-3, 8-11, 4-7, 12-15 (the order in
@@ -195,10 +214,10 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_prefill_mfma_kernel(const
     const uint32_t vt_off = [&] {
         const uint32_t x = v_row & 15u;
         const uint32_t pos = (v_row & 16u) | (x & 3u) | ((x & 8u) >> 1) | ((x & 4u) << 1);
-        return ((uint32_t)tid / kPfKeys) * 8u * VS + pos * 2u;
+        return ((uint32_t)ltid / kPfKeys) * 8u * VS + pos * 2u;
     }();
     auto transpose_v = [&](const unsigned char* st, unsigned char* vt) {
-        if (loader) {
+        if (tid < CHUNKS) {
             const pf_half8 h8 = *reinterpret_cast<const pf_half8*>(st + K_TILE + tid * 16);
 #pragma unroll
             for (int e = 0; e < 8; ++e)
@@ -215,17 +234,30 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_prefill_mfma_kernel(const
 
     auto compute_tile = [&](uint32_t tile, const unsigned char* kbuf, const unsigned char* vbuf) {
         const uint32_t key0 = tile * kPfKeys;
-        // ---- S^T = K . Q^T
+        // ---- S^T = K . Q^T.  All operand reads of a phase are issued before its first MFMA,
+        // and the V^T reads before the softmax, so LDS latency is paid once per phase and
+        // mostly behind other work instead of once per MFMA.
+        pf_half8 kf[KSTEPS];
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+            const int chunk = ks * 2 + half;
+            kf[ks] = *reinterpret_cast<const pf_half8*>(
+                kbuf + (size_t)l32 * (D * 2) + ((chunk ^ (l32 % CPR)) * 16));
+        }
         pf_float16 s;
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[i] = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-            const int chunk = ks * 2 + half;
-            const pf_half8 kf = *reinterpret_cast<const pf_half8*>(
-                kbuf + (size_t)l32 * (D * 2) + ((chunk ^ (l32 % CPR)) * 16));
-            s = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[ks], s, 0, 0, 0);
-        }
+        for (int ks = 0; ks < KSTEPS; ++ks)
+            s = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[ks], qf[ks], s, 0, 0, 0);
+        pf_half8 vf[MB][2];
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+                vf[mb][t] = *reinterpret_cast<const pf_half8*>(
+                    vbuf + (size_t)(mb * 32 + l32) * VS + (t * 16 + half * 8) * 2);
+        __builtin_amdgcn_sched_barrier(0);  // keep the V^T reads ahead of the softmax
         // ---- mask + online softmax on the raw scores (the scale is folded into the exp2
         // argument); register i holds key (i/4)*8 + half*4 + i%4 of the tile.  The running
         // reference is only raised when a tile exceeds it by more than 2^8, so the O^T
@@ -263,14 +295,10 @@ __global__ __launch_bounds__(64 * kPfWaves) void paged_prefill_mfma_kernel(const
         l_run += rs;  // this lane's keys only; the two halves are added at the end
         // ---- O^T += V^T . P^T
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
+        for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                const pf_half8 vf = *reinterpret_cast<const pf_half8*>(
-                    vbuf + (size_t)(mb * 32 + l32) * VS + (t * 16 + half * 8) * 2);
-                oacc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pfrag[t], oacc[mb], 0, 0, 0);
-            }
-        }
+            for (int t = 0; t < 2; ++t)
+                oacc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[mb][t], pfrag[t], oacc[mb], 0, 0, 0);
     };
 
     // Tile t lives in stage t % NST and V^T buffer t % 2.  Step S (t % NST == S): start the

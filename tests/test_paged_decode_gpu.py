@@ -241,3 +241,37 @@ def test_bad_arguments_are_rejected(exe):
         assert not run(flat=np.array([0, 999], np.uint32))
     finally:
         dev.free()
+
+
+@pytest.mark.timeout(600)
+def test_baseline_config4_full_size(exe):
+    """Llama-3-8B shape at its full size (batch 64, 16384-page pool, 1.16 GB of KV per call).
+    The oracle is too slow for all of it, so: (1) four sampled requests are checked against the
+    oracle on the same pool, (2) a second run with a different split-K plan must agree with the
+    first (the merge is associative up to rounding), (3) every output row is a convex
+    combination of V rows: finite and bounded by the largest |V| value."""
+    from dataclasses import replace
+    case = baseline_config(4)
+    print(f"[case] {case.name} full size: {case.kv_bytes / 1e9:.2f} GB of KV", flush=True)
+    dev = DeviceCase(exe, case)
+    try:
+        got = dev.run(sync=True)
+        items_auto = exe.lastDecodeWorkItems()
+        assert exe.setOption("decode_target_items", 1536)
+        again = dev.run(sync=True)
+        assert exe.lastDecodeWorkItems() != items_auto
+    finally:
+        exe.setOption("decode_target_items", 0)
+        dev.free()
+    assert np.all(np.isfinite(got))
+    assert np.max(np.abs(got - again)) < 3e-4
+    vmax = float(np.max(np.abs(case.v_pages.view(np.float16)[::257].astype(np.float32)))) + 8.0
+    assert np.max(np.abs(got)) <= vmax
+    for r in (0, 17, 40, 63):
+        lo, hi = int(case.page_table_offsets[r]), int(case.page_table_offsets[r + 1])
+        sub = replace(case, batch=1, seq_lens=case.seq_lens[r:r + 1], q_positions=case.q_positions[r:r + 1],
+                      page_tables_flat=case.page_tables_flat[lo:hi],
+                      page_table_offsets=np.array([0, hi - lo], np.uint32), q=case.q[r:r + 1])
+        want = oracle_decode(sub)
+        assert want is not None
+        assert_parity(got[r:r + 1], want, case.head_dim, f"cfg4 request {r}")
