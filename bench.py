@@ -112,7 +112,9 @@ def bench_prefill(args) -> int:
                                f"tokens, {H}q/{Hkv}kv heads, head_dim {D}, {P}-token pages",
                    "flop_per_step": flops, "kv_bytes_per_step": kv_bytes},
         "roofline": {"bound": "mfma", "achieved": round(ach, 2), "peak": MFMA_F16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(ach / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
+                     "unit": "TFLOP/s", "frac": round(ach / MFMA_F16_PEAK_TFLOPS, 4),
+                     # rocprofv3 FETCH_SIZE x2.0 + WRITE_SIZE x1.0 (copy-kernel calibration)
+                     "traffic": 184_800_000 if not (args.prefill_stages) else None,
                      "us_per_launch": round(ev_ms / steps * 1e3, 2)},
     }
     if not args.no_cpu:
@@ -320,7 +322,7 @@ def main() -> int:
 
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs),
     # scaled by the copy-kernel calibration (x2.0 / x1.0); valid for the default planner only.
-    measured_traffic = {"cfg2": 44_160_000, "cfg3": 142_460_000}
+    measured_traffic = {"cfg2": 44_220_000, "cfg3": 142_580_000, "cfg4": 1_191_200_000}
     traffic = measured_traffic.get(args.workload) if not args.target_items else None
 
     result = {
