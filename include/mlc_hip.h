@@ -163,6 +163,37 @@ int mlc_hip_qkv_split_rope_scatter(const void* qkv, void* q, void* k_pages, void
                                    size_t qkv_rows, size_t q_rows, size_t k_rows, size_t v_rows,
                                    size_t rotary_dim, int sync);
 
+/* ---- the other per-layer operators of the batched decode step ---------------
+ * (compiler/runtime/batched_walker.cpp:246-405).  sync = 0 needs an open pass
+ * like every encode* method of the reference; sync = 1 also waits.
+ *
+ * MetalExecutor::encodeRmsNormBatched (metal_runtime.hpp:474-479,
+ * metal_runtime.mm:6887-6926; kernel rms_norm_kernel_v2_batched :166-208):
+ * out[r][i] = in[r][i] * (1 / sqrt(mean(in[r]^2) + epsilon)) * weight[i] for
+ * `batch` rows of `length` floats.  weight is a HOST vector borrowed for the
+ * call (the reference copies it into its "norm_w" buffer per call); entries
+ * past n_weight count as 1. */
+int mlc_hip_rms_norm_batched(const void* in, const float* weight, size_t n_weight, float epsilon,
+                             size_t batch, size_t length, void* out, int sync);
+
+/* MetalExecutor::encodeAddBatched (metal_runtime.hpp:501-502,
+ * metal_runtime.mm:7014-7042; kernel add_vectors :44-52): out = a + b. */
+int mlc_hip_add_batched(const void* a, const void* b, void* out, size_t total_elements, int sync);
+
+/* MetalExecutor::encodeSiluMulBatched (metal_runtime.hpp:505-506,
+ * metal_runtime.mm:7044-7072; kernel feedforward_silu_mul :32-42):
+ * out = gate / (1 + exp(-gate)) * up. */
+int mlc_hip_silu_mul_batched(const void* gate, const void* up, void* out, size_t total_elements,
+                             int sync);
+
+/* MetalExecutor::encodeGateUpSplitSiluMul (metal_runtime.hpp:549-552,
+ * metal_runtime.mm:8029-8091): gate = gate_up[:, 0:ffn_inner],
+ * up = gate_up[:, ffn_inner:2*ffn_inner] (rows of ffn_gate_up_rows floats),
+ * out = silu(gate) * up; one launch instead of three dispatches. */
+int mlc_hip_gate_up_split_silu_mul(const void* gate_up, void* gate, void* up, void* out,
+                                   size_t batch, size_t ffn_inner, size_t ffn_gate_up_rows,
+                                   int sync);
+
 /* Chunked prefill over paged KV (MFMA path).  No counterpart in the reference,
  * which prefills by looping the decode path once per prompt token
  * (compiler/runtime/batched_executor.cpp:454-466); semantics are the decode

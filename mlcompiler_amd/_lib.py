@@ -36,6 +36,10 @@ SIGNATURES = {
     "mlc_hip_gather_kv_pages": (C.c_int, [_vp, _u32p, _sz, _sz, _sz, _sz, _sz, _vp, _sz]),
     "mlc_hip_qkv_split_rope_cast": (C.c_int, [_vp] * 8 + [_sz] * 9 + [C.c_int]),
     "mlc_hip_qkv_split_rope_scatter": (C.c_int, [_vp] * 8 + [_u32p, _u32p] + [_sz] * 10 + [C.c_int]),
+    "mlc_hip_rms_norm_batched": (C.c_int, [_vp, _vp, _sz, C.c_float, _sz, _sz, _vp, C.c_int]),
+    "mlc_hip_add_batched": (C.c_int, [_vp, _vp, _vp, _sz, C.c_int]),
+    "mlc_hip_silu_mul_batched": (C.c_int, [_vp, _vp, _vp, _sz, C.c_int]),
+    "mlc_hip_gate_up_split_silu_mul": (C.c_int, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, C.c_int]),
     "mlc_hip_paged_attn_prefill": (C.c_int, [_vp, _vp, _vp, _vp, _u32p, _sz, _u32p, _u32p, _u32p,
                                              _sz, _sz, _sz, _sz, _sz, _sz, C.c_int]),
     "mlc_hip_stream": (_vp, []),

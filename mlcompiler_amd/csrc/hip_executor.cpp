@@ -137,6 +137,29 @@ bool HipExecutor::encodeQkvSplitRopeScatter(void* qkv_buf, void* q_buf, void* k_
                                           rotary_dim, /*sync=*/0) != 0;
 }
 
+bool HipExecutor::encodeRmsNormBatched(void* in_buf, const std::vector<float>& weight, float epsilon,
+                                       size_t batch, size_t length, void* out_buf) const {
+    return mlc_hip_rms_norm_batched(in_buf, weight.data(), weight.size(), epsilon, batch, length,
+                                    out_buf, /*sync=*/0) != 0;
+}
+
+bool HipExecutor::encodeAddBatched(void* a_buf, void* b_buf, void* out_buf,
+                                   size_t total_elements) const {
+    return mlc_hip_add_batched(a_buf, b_buf, out_buf, total_elements, /*sync=*/0) != 0;
+}
+
+bool HipExecutor::encodeSiluMulBatched(void* gate_buf, void* up_buf, void* out_buf,
+                                       size_t total_elements) const {
+    return mlc_hip_silu_mul_batched(gate_buf, up_buf, out_buf, total_elements, /*sync=*/0) != 0;
+}
+
+bool HipExecutor::encodeGateUpSplitSiluMul(void* gate_up_buf, void* gate_buf, void* up_buf,
+                                           void* out_buf, size_t batch, size_t ffn_inner,
+                                           size_t ffn_gate_up_rows) const {
+    return mlc_hip_gate_up_split_silu_mul(gate_up_buf, gate_buf, up_buf, out_buf, batch, ffn_inner,
+                                          ffn_gate_up_rows, /*sync=*/0) != 0;
+}
+
 bool HipExecutor::runPagedPrefillAttention(void* q_f16_buffer, void* k_pages_buffer,
                                            void* v_pages_buffer, void* o_buffer,
                                            const std::vector<uint32_t>& page_tables_flat,

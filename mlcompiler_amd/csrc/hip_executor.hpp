@@ -89,6 +89,15 @@ public:
                                    size_t kv_heads, size_t head_dim, size_t qkv_rows, size_t q_rows,
                                    size_t k_rows, size_t v_rows, size_t rotary_dim) const;
 
+    // metal_runtime.hpp:474-479, 501-506, 549-552: the walker's small per-layer operators
+    bool encodeRmsNormBatched(void* in_buf, const std::vector<float>& weight, float epsilon,
+                              size_t batch, size_t length, void* out_buf) const;
+    bool encodeAddBatched(void* a_buf, void* b_buf, void* out_buf, size_t total_elements) const;
+    bool encodeSiluMulBatched(void* gate_buf, void* up_buf, void* out_buf,
+                              size_t total_elements) const;
+    bool encodeGateUpSplitSiluMul(void* gate_up_buf, void* gate_buf, void* up_buf, void* out_buf,
+                                  size_t batch, size_t ffn_inner, size_t ffn_gate_up_rows) const;
+
     // Chunked prefill over paged KV: no reference method (the reference loops its
     // decode path per prompt token, batched_executor.cpp:454-466).
     bool runPagedPrefillAttention(void* q_f16_buffer, void* k_pages_buffer, void* v_pages_buffer,

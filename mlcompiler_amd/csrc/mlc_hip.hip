@@ -21,6 +21,7 @@
 #include "paged_decode_kernels.h"
 #include "paged_prefill_kernels.h"
 #include "paged_rope_kernels.h"
+#include "walker_kernels.h"
 
 namespace mlc_hip {
 // Defined in paged_decode_inst.hip, one object per (head_dim, heads-per-wave).
@@ -870,6 +871,85 @@ int mlc_hip_qkv_split_rope_scatter(const void* qkv, void* q, void* k_pages, void
     a.rotary_dim = (uint32_t)rotary_dim; a.page_size = (uint32_t)page_size_tokens;
     launch_qkv_split_rope_cast<true>(a, g.stream);
     if (!slot_mark(s)) return 0;
+    return finish(sync);
+}
+
+// ---- the walker's small per-layer operators ----------------------------------------------
+
+int mlc_hip_rms_norm_batched(const void* in, const float* weight, size_t n_weight, float epsilon,
+                             size_t batch, size_t length, void* out, int sync) {
+    if (!init_once()) return fail("GPU unavailable");
+    if (!sync && !g.pass_open) return fail("encode: no open forward pass");
+    if (!in || !out || batch == 0 || length == 0) return fail("rms norm: null buffer or zero size");  // :6895
+    if (n_weight && !weight) return fail("rms norm: null weight");
+    if (batch * length > 0x7FFFFFFFull) return fail("rms norm: too many elements");
+    const size_t ki = known_bytes(in), ko = known_bytes(out);
+    if ((ki && batch * length * 4 > ki) || (ko && batch * length * 4 > ko))
+        return fail("rms norm: buffer too small");
+    // the weight vector is borrowed for the call: staged like the other metadata
+    MetaSlot& s = g.ring[g.ring_next];
+    g.ring_next = (g.ring_next + 1) % 8;
+    const size_t w_bytes = std::max<size_t>(align_up(n_weight * 4, 16), 16);
+    if (!slot_reserve(s, w_bytes)) return 0;
+    if (n_weight) std::memcpy(s.host, weight, n_weight * 4);
+    if (!slot_upload(s, w_bytes)) return 0;
+    hipLaunchKernelGGL(rms_norm_batched_kernel, dim3((unsigned)batch), dim3(256), 0, g.stream,
+                       static_cast<const float*>(in), static_cast<const float*>(s.dev),
+                       (uint32_t)n_weight, epsilon, (uint32_t)length, static_cast<float*>(out));
+    if (!slot_mark(s)) return 0;
+    return finish(sync);
+}
+
+namespace {
+const char* flat3_problem(const void* a, const void* b, const void* out, size_t n, const char* what) {
+    static thread_local std::string msg;
+    if (!a || !b || !out || n == 0) { msg = std::string(what) + ": null buffer or zero size"; return msg.c_str(); }
+    if (n > 0x7FFFFFFFull) { msg = std::string(what) + ": too many elements"; return msg.c_str(); }
+    for (const void* p : {a, b, out}) {
+        const size_t k = known_bytes(p);
+        if (k && n * 4 > k) { msg = std::string(what) + ": buffer too small"; return msg.c_str(); }
+    }
+    return nullptr;
+}
+}  // namespace
+
+int mlc_hip_add_batched(const void* a, const void* b, void* out, size_t total_elements, int sync) {
+    if (!init_once()) return fail("GPU unavailable");
+    if (!sync && !g.pass_open) return fail("encode: no open forward pass");
+    if (const char* why = flat3_problem(a, b, out, total_elements, "add")) return fail(why);  // :7018
+    hipLaunchKernelGGL(add_kernel, dim3((unsigned)((total_elements + 255) / 256)), dim3(256), 0, g.stream,
+                       static_cast<const float*>(a), static_cast<const float*>(b),
+                       static_cast<float*>(out), (uint32_t)total_elements);
+    return finish(sync);
+}
+
+int mlc_hip_silu_mul_batched(const void* gate, const void* up, void* out, size_t total_elements,
+                             int sync) {
+    if (!init_once()) return fail("GPU unavailable");
+    if (!sync && !g.pass_open) return fail("encode: no open forward pass");
+    if (const char* why = flat3_problem(gate, up, out, total_elements, "silu mul")) return fail(why);  // :7048
+    hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((total_elements + 255) / 256)), dim3(256), 0,
+                       g.stream, static_cast<const float*>(gate), static_cast<const float*>(up),
+                       static_cast<float*>(out), (uint32_t)total_elements);
+    return finish(sync);
+}
+
+int mlc_hip_gate_up_split_silu_mul(const void* gate_up, void* gate, void* up, void* out, size_t batch,
+                                   size_t ffn_inner, size_t ffn_gate_up_rows, int sync) {
+    if (!init_once()) return fail("GPU unavailable");
+    if (!sync && !g.pass_open) return fail("encode: no open forward pass");
+    if (!gate_up) return fail("gate/up split: null buffer");
+    if (batch == 0 || ffn_inner == 0) return fail("gate/up split: zero size");
+    if (const char* why = flat3_problem(gate, up, out, batch * ffn_inner, "gate/up split")) return fail(why);
+    if (2 * ffn_inner > ffn_gate_up_rows) return fail("gate/up split: 2 * ffn_inner > ffn_gate_up_rows");
+    if (batch * ffn_gate_up_rows > 0x7FFFFFFFull) return fail("gate/up split: too many elements");
+    const size_t kg = known_bytes(gate_up);
+    if (kg && batch * ffn_gate_up_rows * 4 > kg) return fail("gate/up split: gate_up buffer too small");
+    const size_t n = batch * ffn_inner;
+    hipLaunchKernelGGL(gate_up_split_silu_mul_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                       g.stream, static_cast<const float*>(gate_up), static_cast<float*>(gate),
+                       static_cast<float*>(up), static_cast<float*>(out), (uint32_t)batch,
+                       (uint32_t)ffn_inner, (uint32_t)ffn_gate_up_rows);
     return finish(sync);
 }
 

@@ -181,6 +181,29 @@ class HipExecutor:
             _ptr(ids), _ptr(sl), page_size_tokens, batch, num_heads, kv_heads, head_dim, qkv_rows,
             q_rows, k_rows, v_rows, rotary_dim, int(bool(sync))))
 
+    # -- the other per-layer operators of the batched decode step
+    def encodeRmsNormBatched(self, in_buf, weight, epsilon, batch, length, out_buf,
+                             sync: bool = False) -> bool:  # metal_runtime.hpp:474-479
+        w = np.ascontiguousarray(weight, np.float32)
+        return bool(self._lib.mlc_hip_rms_norm_batched(
+            in_buf, w.ctypes.data if w.size else None, w.size, float(epsilon), batch, length, out_buf,
+            int(bool(sync))))
+
+    def encodeAddBatched(self, a_buf, b_buf, out_buf, total_elements, sync: bool = False) -> bool:
+        return bool(self._lib.mlc_hip_add_batched(a_buf, b_buf, out_buf, total_elements,
+                                                  int(bool(sync))))  # metal_runtime.hpp:501-502
+
+    def encodeSiluMulBatched(self, gate_buf, up_buf, out_buf, total_elements,
+                             sync: bool = False) -> bool:  # metal_runtime.hpp:505-506
+        return bool(self._lib.mlc_hip_silu_mul_batched(gate_buf, up_buf, out_buf, total_elements,
+                                                       int(bool(sync))))
+
+    def encodeGateUpSplitSiluMul(self, gate_up_buf, gate_buf, up_buf, out_buf, batch, ffn_inner,
+                                 ffn_gate_up_rows, sync: bool = False) -> bool:  # :549-552
+        return bool(self._lib.mlc_hip_gate_up_split_silu_mul(
+            gate_up_buf, gate_buf, up_buf, out_buf, batch, ffn_inner, ffn_gate_up_rows,
+            int(bool(sync))))
+
     # -- chunked prefill (no reference method; see include/mlc_hip.h)
     def runPagedPrefillAttention(self, q_f16_buffer, k_pages_buffer, v_pages_buffer, o_buffer,
                                  page_tables_flat, page_table_offsets, seq_lens, q_start, batch,

@@ -248,6 +248,116 @@ int oracle_qkv_split_rope_cast(const float* qkv, float* q, float* k, float* v,
     return 1;
 }
 
+/* ------------------------------------------------ walker layer operators */
+
+int oracle_rms_norm_batched(const float* in, const float* weight, size_t n_weight, float epsilon,
+                            size_t batch, size_t length, float* out) {
+    if (!in || !out || batch == 0 || length == 0) return 0;
+    for (size_t r = 0; r < batch; ++r) {
+        const float* x = in + r * length;
+        float mean_sq = 0.0f; /* operator_backend.cpp:194-198 */
+        for (size_t i = 0; i < length; ++i) mean_sq += x[i] * x[i];
+        mean_sq = mean_sq / (float)length;
+        float inv = 1.0f / sqrtf(mean_sq + epsilon);
+        for (size_t i = 0; i < length; ++i) {
+            float gamma = (weight && i < n_weight) ? weight[i] : 1.0f;
+            out[r * length + i] = x[i] * inv * gamma;
+        }
+    }
+    return 1;
+}
+
+int oracle_add(const float* a, const float* b, float* out, size_t n) {
+    if (!a || !b || !out || n == 0) return 0;
+    for (size_t i = 0; i < n; ++i) out[i] = a[i] + b[i];
+    return 1;
+}
+
+int oracle_silu_mul(const float* gate, const float* up, float* out, size_t n) {
+    if (!gate || !up || !out || n == 0) return 0;
+    for (size_t i = 0; i < n; ++i) {
+        float g = gate[i];
+        float silu = g / (1.0f + expf(-g));
+        out[i] = silu * up[i];
+    }
+    return 1;
+}
+
+int oracle_gate_up_split_silu_mul(const float* gate_up, float* gate, float* up, float* out,
+                                  size_t batch, size_t ffn_inner, size_t gate_up_rows) {
+    if (!gate_up || !gate || !up || !out || batch == 0 || ffn_inner == 0) return 0;
+    if (2 * ffn_inner > gate_up_rows) return 0;
+    for (size_t r = 0; r < batch; ++r) {
+        memcpy(gate + r * ffn_inner, gate_up + r * gate_up_rows, ffn_inner * sizeof(float));
+        memcpy(up + r * ffn_inner, gate_up + r * gate_up_rows + ffn_inner, ffn_inner * sizeof(float));
+    }
+    return oracle_silu_mul(gate, up, out, batch * ffn_inner);
+}
+
+int oracle_matmul_q4_0_batched(const uint8_t* weights, const float* in, size_t batch, size_t rows,
+                               size_t cols, size_t row_stride, float* out, int n_threads) {
+    if (!weights || !in || !out || batch == 0 || rows == 0 || cols == 0) return 0;
+    if (cols < 64 || (rows % 4u) != 0) return 0; /* metal_runtime.mm:6942 */
+    const size_t nb = (cols + 31) / 32;
+    if (row_stride < nb * 18) return 0;
+    if (n_threads < 1) n_threads = 1;
+#pragma omp parallel for num_threads(n_threads) schedule(static)
+    for (long long r = 0; r < (long long)rows; ++r) {
+        const uint8_t* row = weights + (size_t)r * row_stride;
+        for (size_t b = 0; b < batch; ++b) {
+            const float* vec = in + b * cols;
+            float acc = 0.0f; /* quantization.cpp:247-267 */
+            for (size_t blk = 0; blk < nb; ++blk) {
+                const size_t base = blk * 32;
+                const uint8_t* p = row + blk * 18;
+                uint16_t dh;
+                memcpy(&dh, p, 2);
+                const float d = oracle_fp16_to_float(dh);
+                for (size_t j = 0; j < 16; ++j) {
+                    const uint8_t byte = p[2 + j];
+                    const int lo = (int)(byte & 0x0F) - 8;
+                    const int hi = (int)((byte >> 4) & 0x0F) - 8;
+                    if (base + j < cols) acc += d * (float)lo * vec[base + j];
+                    if (base + j + 16 < cols) acc += d * (float)hi * vec[base + j + 16];
+                }
+            }
+            out[b * rows + (size_t)r] = acc;
+        }
+    }
+    return 1;
+}
+
+void oracle_quantize_row_q4_0(const float* src, size_t cols, uint8_t* dst) {
+    const size_t blocks = (cols + 31) / 32;
+    size_t idx = 0;
+    for (size_t b = 0; b < blocks; ++b) {
+        const float* block = src + idx;
+        const size_t bs = cols - idx < 32 ? cols - idx : 32;
+        float max_abs = 0.0f, max_val = 0.0f; /* quantization.cpp:283-292 */
+        for (size_t i = 0; i < bs; ++i) {
+            float v = block[i], av = fabsf(v);
+            if (av > max_abs) {
+                max_abs = av;
+                max_val = v;
+            }
+        }
+        const float scale = max_val / -8.0f;
+        const float inv_scale = (scale != 0.0f) ? (1.0f / scale) : 0.0f;
+        const uint16_t fp = oracle_float_to_fp16_ref(scale);
+        uint8_t* o = dst + b * 18;
+        memcpy(o, &fp, 2);
+        for (size_t j = 0; j < 16; ++j) {
+            const float x0 = (j < bs) ? block[j] * inv_scale : 0.0f;
+            const float x1 = (j + 16 < bs) ? block[j + 16] * inv_scale : 0.0f;
+            int q0 = (int)(x0 + 8.5f), q1 = (int)(x1 + 8.5f);
+            q0 = q0 < 0 ? 0 : (q0 > 15 ? 15 : q0);
+            q1 = q1 < 0 ? 0 : (q1 > 15 ? 15 : q1);
+            o[2 + j] = (uint8_t)((q1 << 4) | q0);
+        }
+        idx += bs;
+    }
+}
+
 /* ------------------------------------------------------------- attention */
 
 static int attention_args_ok(const void* q, const void* k, const void* v, const void* o,

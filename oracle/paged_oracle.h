@@ -119,6 +119,43 @@ int oracle_qkv_split_rope_cast(const float* qkv, float* q, float* k, float* v,
 size_t oracle_rotary_coefficients(size_t position, size_t rotary_dim, float freq_base,
                                   float freq_scale, float* cos_out, float* sin_out);
 
+/* ---- the walker's other per-layer operators (compiler/runtime/batched_walker.cpp:246-405) ----
+ *
+ * RMSNorm over `batch` rows of `length` floats with one shared weight vector: the CPU rmsNorm
+ * of compiler/runtime/operator_backend.cpp:186-203 per row (sequential fp32 sum of squares,
+ * mean, inv = 1/sqrtf(mean + eps), out = in * inv * gamma; gamma = 1 past the end of weight),
+ * which the kernel rms_norm_kernel_v2_batched (metal_runtime.mm:166-208) follows up to the
+ * order of its sum.  Returns 0 when a buffer is missing or batch/length is 0
+ * (metal_runtime.mm:6895). */
+int oracle_rms_norm_batched(const float* in, const float* weight, size_t n_weight, float epsilon,
+                            size_t batch, size_t length, float* out);
+
+/* add_vectors (metal_runtime.mm:44-52) over a flat range: encodeAddBatched (:7014-7042). */
+int oracle_add(const float* a, const float* b, float* out, size_t n);
+
+/* feedforward_silu_mul (metal_runtime.mm:32-42): out = gate / (1 + expf(-gate)) * up. */
+int oracle_silu_mul(const float* gate, const float* up, float* out, size_t n);
+
+/* encodeGateUpSplitSiluMul (metal_runtime.mm:8029-8091): gate = gate_up[:, 0:inner],
+ * up = gate_up[:, inner:2*inner] (rows of gate_up_rows floats), out = silu(gate) * up. */
+int oracle_gate_up_split_silu_mul(const float* gate_up, float* gate, float* up, float* out,
+                                  size_t batch, size_t ffn_inner, size_t gate_up_rows);
+
+/* Q4_0 rows: 18-byte blocks of 32 weights (fp16 scale d, then 16 bytes; byte j holds weight j
+ * in its low nibble and weight j+16 in its high nibble, value = d * (nibble - 8)),
+ * compiler/runtime/quantization.cpp:70-74, 191-214.  out[b][r] = the CPU dotProductRowQ4_0
+ * (quantization.cpp:240-269: one fp32 accumulator, blocks in order, within a block the pairs
+ * (j, j+16) in order, each term d * q * x rounded as written) of weight row r (row_stride bytes
+ * apart) with input row b.  Same result layout and constraints as q4_0_matmul_v3_batched
+ * (metal_runtime.mm:710-785; host :6930-6990: cols >= 64, rows % 4 == 0). */
+int oracle_matmul_q4_0_batched(const uint8_t* weights, const float* in, size_t batch, size_t rows,
+                               size_t cols, size_t row_stride, float* out, int n_threads);
+
+/* quantizeRowQ4_0 (quantization.cpp:271-311), used to make test weights: scale = (value of
+ * largest magnitude) / -8, q = clamp((int)(x / scale + 8.5), 0, 15), scale stored through the
+ * reference's floatToFp16.  dst must hold ceil(cols/32)*18 bytes. */
+void oracle_quantize_row_q4_0(const float* src, size_t cols, uint8_t* dst);
+
 /* The executor-CPU attention, compiler/runtime/attention_cpu.cpp:437-470
  * (per head: left-to-right dot over every cached row :99-105, softmax that
  * subtracts the max, exponentiates and divides each weight by the sum :21-33,

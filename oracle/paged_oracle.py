@@ -64,6 +64,18 @@ def lib() -> C.CDLL:
                                                  C.c_void_p] + [_sz] * 9
         L.oracle_rotary_coefficients.restype = _sz
         L.oracle_rotary_coefficients.argtypes = [_sz, _sz, C.c_float, C.c_float, _f32p, _f32p]
+        L.oracle_rms_norm_batched.restype = C.c_int
+        L.oracle_rms_norm_batched.argtypes = [_f32p, C.c_void_p, _sz, C.c_float, _sz, _sz, _f32p]
+        L.oracle_add.restype = C.c_int
+        L.oracle_add.argtypes = [_f32p, _f32p, _f32p, _sz]
+        L.oracle_silu_mul.restype = C.c_int
+        L.oracle_silu_mul.argtypes = [_f32p, _f32p, _f32p, _sz]
+        L.oracle_gate_up_split_silu_mul.restype = C.c_int
+        L.oracle_gate_up_split_silu_mul.argtypes = [_f32p, _f32p, _f32p, _f32p, _sz, _sz, _sz]
+        L.oracle_matmul_q4_0_batched.restype = C.c_int
+        L.oracle_matmul_q4_0_batched.argtypes = [C.c_void_p, _f32p, _sz, _sz, _sz, _sz, _f32p, C.c_int]
+        L.oracle_quantize_row_q4_0.restype = None
+        L.oracle_quantize_row_q4_0.argtypes = [_f32p, _sz, C.c_void_p]
         L.oracle_gather_kv_pages.restype = C.c_int
         L.oracle_gather_kv_pages.argtypes = [C.c_void_p, _u32p, _sz, _sz, _sz, _sz, _sz,
                                              C.c_void_p, _sz]
@@ -208,6 +220,64 @@ def qkv_split_rope_cast(qkv, cos, sin, batch, num_heads, kv_heads, head_dim, qkv
                                           _p(k16, _u16p), _p(v16, _u16p), cosp, sinp, batch, num_heads,
                                           kv_heads, head_dim, qkv_rows, q_rows, k_rows, v_rows, rotary_dim)
     return (q, k, v, k16, v16) if ok else None
+
+
+# ------------------------------------------------ walker layer operators
+
+def rms_norm_batched(x, weight, epsilon, batch, length):
+    x = _c(x, np.float32)
+    w = None if weight is None else _c(weight, np.float32)
+    out = np.zeros((batch, length), np.float32)
+    ok = lib().oracle_rms_norm_batched(_p(x, _f32p), None if w is None else w.ctypes.data,
+                                       0 if w is None else w.size, epsilon, batch, length, _p(out, _f32p))
+    return out if ok else None
+
+
+def add(a, b):
+    a, b = _c(a, np.float32), _c(b, np.float32)
+    out = np.zeros(a.shape, np.float32)
+    return out if lib().oracle_add(_p(a, _f32p), _p(b, _f32p), _p(out, _f32p), a.size) else None
+
+
+def silu_mul(gate, up):
+    g, u = _c(gate, np.float32), _c(up, np.float32)
+    out = np.zeros(g.shape, np.float32)
+    return out if lib().oracle_silu_mul(_p(g, _f32p), _p(u, _f32p), _p(out, _f32p), g.size) else None
+
+
+def gate_up_split_silu_mul(gate_up, batch, ffn_inner, gate_up_rows):
+    """Returns (gate, up, out) or None."""
+    gu = _c(gate_up, np.float32)
+    gate = np.zeros((batch, ffn_inner), np.float32)
+    up = np.zeros((batch, ffn_inner), np.float32)
+    out = np.zeros((batch, ffn_inner), np.float32)
+    ok = lib().oracle_gate_up_split_silu_mul(_p(gu, _f32p), _p(gate, _f32p), _p(up, _f32p), _p(out, _f32p),
+                                             batch, ffn_inner, gate_up_rows)
+    return (gate, up, out) if ok else None
+
+
+def q4_0_row_bytes(cols: int) -> int:
+    return (cols + 31) // 32 * 18
+
+
+def quantize_q4_0(w) -> np.ndarray:
+    """Rows of floats -> Q4_0 rows (uint8 [rows][q4_0_row_bytes(cols)]), quantizeRowQ4_0."""
+    w = _c(w, np.float32)
+    rows, cols = w.shape
+    out = np.zeros((rows, q4_0_row_bytes(cols)), np.uint8)
+    L = lib()
+    for r in range(rows):
+        L.oracle_quantize_row_q4_0(_p(w[r], _f32p), cols, out[r].ctypes.data)
+    return out
+
+
+def matmul_q4_0_batched(weights, x, batch, rows, cols, row_stride=None, n_threads=8):
+    wq = _c(weights, np.uint8)
+    x = _c(x, np.float32)
+    out = np.zeros((batch, rows), np.float32)
+    ok = lib().oracle_matmul_q4_0_batched(wq.ctypes.data, _p(x, _f32p), batch, rows, cols,
+                                          row_stride or q4_0_row_bytes(cols), _p(out, _f32p), n_threads)
+    return out if ok else None
 
 
 # ------------------------------------------------------------ attention
@@ -403,6 +473,12 @@ def ref_lib():
         R.ref_apply_rotary.argtypes = [_f32p, _f32p, _f32p, _sz, _sz, _sz]
         R.ref_rotary_coefficients.restype = _sz
         R.ref_rotary_coefficients.argtypes = [_sz, _sz, C.c_float, C.c_float, _f32p, _f32p]
+        R.ref_quantize_row_q4_0.restype = _sz
+        R.ref_quantize_row_q4_0.argtypes = [_f32p, _sz, C.c_void_p, _sz]
+        R.ref_dot_q4_0.restype = C.c_float
+        R.ref_dot_q4_0.argtypes = [C.c_void_p, _sz, _f32p]
+        R.ref_dequantize_row_q4_0.restype = None
+        R.ref_dequantize_row_q4_0.argtypes = [C.c_void_p, _sz, _f32p]
         R.ref_run_attention_cpu.restype = C.c_int
         R.ref_run_attention_cpu.argtypes = [_f32p, _u16p, _u16p, _sz, _sz, _sz, _sz, _sz, _f32p,
                                             _f32p, _f32p]

@@ -7,6 +7,8 @@
 //   mlc::runtime::fp16ToFloat/floatToFp16 compiler/runtime/float_convert.hpp:14-76
 //   mlc::runtime::applyRotaryEmbedding / computeRotaryCoefficients
 //                                         compiler/runtime/quantization.cpp:772-823
+//   mlc::runtime::quantizeRowQ4_0 / dotProductRowQ4_0 / dequantizeRowQ4_0
+//                                         compiler/runtime/quantization.cpp:235-311
 // the way the reference's own test does (tests/test_runtime.cpp:1659-1690):
 // an ExecutionGraph with one Attention node, state tensors {Hkv, ctx, D}
 // tagged role=kv_cache so ExecutionContext stores them as F16
@@ -142,6 +144,21 @@ size_t ref_rotary_coefficients(size_t position, size_t rotary_dim, float freq_ba
     std::memcpy(cos, c.data(), c.size() * sizeof(float));
     std::memcpy(sin, s.data(), s.size() * sizeof(float));
     return c.size();
+}
+
+// quantizeRowQ4_0 / dotProductRowQ4_0 / dequantizeRowQ4_0 (compiler/runtime/quantization.cpp:235-311)
+size_t ref_quantize_row_q4_0(const float* src, size_t cols, uint8_t* dst, size_t dst_cap) {
+    std::vector<uint8_t> out;
+    mlc::runtime::quantizeRowQ4_0(src, cols, 1, out);
+    if (out.size() > dst_cap) return 0;
+    std::memcpy(dst, out.data(), out.size());
+    return out.size();
+}
+float ref_dot_q4_0(const uint8_t* row, size_t cols, const float* vec) {
+    return mlc::runtime::dotProductRowQ4_0(row, cols, 1, vec);
+}
+void ref_dequantize_row_q4_0(const uint8_t* row, size_t cols, float* dst) {
+    mlc::runtime::dequantizeRowQ4_0(row, cols, 1, dst);
 }
 
 }  // extern "C"

@@ -531,3 +531,94 @@ def test_rope_bit_exact_with_reference_build():
         for h in range(Hkv):
             want = po.ref_apply_rotary(qkv[(H + h) * D:(H + h + 1) * D], cos, sin, D, rot)
             assert np.array_equal(k[0, h * D:(h + 1) * D].view(np.uint32), want.view(np.uint32))
+
+
+# ------------------------------------------------ walker layer operators
+
+def test_rms_norm_closed_forms_and_reference_test_formula():
+    rng = np.random.default_rng(3)
+    B, L, eps = 4, 2048, 1e-5
+    x = rng.uniform(-1, 1, (B, L)).astype(np.float32)
+    w = rng.uniform(-1, 1, L).astype(np.float32)
+    got = po.rms_norm_batched(x, w, eps, B, L)
+    # tests/test_batched_elementwise.cpp:19-32 (double-precision sum), tolerance 1e-4 there
+    want = x / np.sqrt((x.astype(np.float64) ** 2).mean(axis=1, keepdims=True) + eps) * w
+    assert np.max(np.abs(got - want)) < 1e-5
+    # constant rows: out = c / sqrt(c^2 + eps) * w
+    c = np.full((2, 64), 3.0, np.float32)
+    got = po.rms_norm_batched(c, np.ones(64, np.float32), eps, 2, 64)
+    assert np.allclose(got, 3.0 / np.sqrt(9.0 + eps), rtol=1e-6)
+    # scale invariance (up to eps) and the missing-weight rule (gamma = 1 past the end)
+    a = po.rms_norm_batched(x * 4, w, 0.0, B, L)
+    b = po.rms_norm_batched(x, w, 0.0, B, L)
+    assert np.max(np.abs(a - b)) < 1e-5
+    short = po.rms_norm_batched(x, w[:10], eps, B, L)
+    full = po.rms_norm_batched(x, np.concatenate([w[:10], np.ones(L - 10, np.float32)]), eps, B, L)
+    assert np.array_equal(short, full)
+    assert po.rms_norm_batched(x, w, eps, 0, L) is None
+
+
+def test_add_silu_gate_up_closed_forms():
+    rng = np.random.default_rng(4)
+    a, b = rng.standard_normal(1000).astype(np.float32), rng.standard_normal(1000).astype(np.float32)
+    assert np.array_equal(po.add(a, b), a + b)
+    g = np.array([0.0, 1.0, -1.0, 20.0, -20.0, 100.0, -100.0], np.float32)
+    u = np.full(g.size, 2.0, np.float32)
+    got = po.silu_mul(g, u)
+    want = g.astype(np.float64) / (1 + np.exp(-g.astype(np.float64))) * 2
+    assert np.allclose(got, want, rtol=1e-6, atol=1e-30)
+    assert got[0] == 0.0 and got[5] == 200.0 and abs(got[6]) < 1e-30   # limits: 0, identity, 0
+    B, inner, rows = 3, 8, 20
+    gu = rng.standard_normal((B, rows)).astype(np.float32)
+    gate, up, out = po.gate_up_split_silu_mul(gu, B, inner, rows)
+    assert np.array_equal(gate, gu[:, :inner]) and np.array_equal(up, gu[:, inner:2 * inner])
+    assert np.array_equal(out, po.silu_mul(gate, up))
+    assert po.gate_up_split_silu_mul(gu, B, 11, rows) is None         # 2*inner > rows
+
+
+def test_q4_0_known_block_and_dequant_formula():
+    # one block by hand: d = 0.5, nibbles j -> weight j, j+16
+    blk = np.zeros(18, np.uint8)
+    blk[:2] = np.frombuffer(np.float16(0.5).tobytes(), np.uint8)
+    lo = np.arange(16) % 16
+    hi = (np.arange(16) * 3 + 1) % 16
+    blk[2:] = (hi << 4 | lo).astype(np.uint8)
+    w = np.concatenate([0.5 * (lo - 8), 0.5 * (hi - 8)]).astype(np.float32)
+    x = np.linspace(-1, 1, 64).astype(np.float32)
+    rows = np.tile(np.concatenate([blk, blk]), (4, 1))              # 4 rows x 64 cols
+    got = po.matmul_q4_0_batched(rows, x[None, :], 1, 4, 64)
+    want = float(np.dot(np.concatenate([w, w]).astype(np.float64), x.astype(np.float64)))
+    assert np.allclose(got, want, rtol=1e-6)
+    # constraints of the batched kernel (metal_runtime.mm:6942)
+    assert po.matmul_q4_0_batched(rows, x[None, :32], 1, 4, 32) is None
+    assert po.matmul_q4_0_batched(rows[:3], x[None, :], 1, 3, 64) is None
+
+
+def test_q4_0_quantize_round_trip_error_bound():
+    rng = np.random.default_rng(6)
+    w = rng.standard_normal((8, 128)).astype(np.float32)
+    q = po.quantize_q4_0(w)
+    eye = np.eye(128, dtype=np.float32)
+    deq = po.matmul_q4_0_batched(q, eye, 128, 8, 128).T            # row r of W = products with unit vectors
+    d = np.abs(w).reshape(8, 4, 32).max(axis=2) / 8
+    assert np.all(np.abs(deq - w).reshape(8, 4, 32) <= d[:, :, None] * 1.01 + 1e-6)
+
+
+@needs_ref
+def test_q4_0_bit_exact_with_reference_build():
+    """quantizeRowQ4_0 / dotProductRowQ4_0 compiled from compiler/runtime/quantization.cpp."""
+    R = po.ref_lib()
+    rng = np.random.default_rng(12)
+    for cols in (64, 96, 2048):
+        w = (rng.standard_normal((4, cols)) * rng.uniform(0.01, 3)).astype(np.float32)
+        q = po.quantize_q4_0(w)
+        for r in range(4):
+            buf = np.zeros(q.shape[1], np.uint8)
+            n = R.ref_quantize_row_q4_0(w[r].ctypes.data_as(po._f32p), cols, buf.ctypes.data, buf.size)
+            assert n == q.shape[1] and np.array_equal(buf, q[r])
+        x = rng.standard_normal((3, cols)).astype(np.float32)
+        got = po.matmul_q4_0_batched(q, x, 3, 4, cols)
+        for b in range(3):
+            for r in range(4):
+                want = R.ref_dot_q4_0(q[r].ctypes.data, cols, x[b].ctypes.data_as(po._f32p))
+                assert np.float32(want).view(np.uint32) == got[b, r].view(np.uint32)
