@@ -194,6 +194,23 @@ int mlc_hip_gate_up_split_silu_mul(const void* gate_up, void* gate, void* up, vo
                                    size_t batch, size_t ffn_inner, size_t ffn_gate_up_rows,
                                    int sync);
 
+/* MetalExecutor::encodeMatMulQ4_0Batched (metal_runtime.hpp:481-489,
+ * metal_runtime.mm:6928-6990; kernel q4_0_matmul_v3_batched :710-785):
+ * out[b][r] = sum_c W[r][c] * in[b][c] for `batch` requests; W is `rows` Q4_0
+ * rows of `cols` weights, row_stride bytes apart (18-byte blocks of 32:
+ * fp16 scale, 16 nibble bytes; compiler/runtime/quantization.cpp:70-74,
+ * 191-214).  `weights` is the HOST copy, uploaded the first time a
+ * weight_name is seen and kept on the device (getOrCacheWeight); in/out are
+ * device fp32 [batch][cols] / [batch][rows].  Same constraints as the
+ * reference (cols >= 64, rows % 4 == 0).  Shapes with rows % 64 == 0 and
+ * cols % 32 == 0 run on the matrix cores with split-fp16 operands (relative
+ * error about 2^-22 per product, fp32 accumulation); others on a scalar
+ * kernel.  Uses library-owned scratch buffers: calls are stream-ordered and
+ * must not overlap from several threads (single-threaded contract above). */
+int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, size_t weight_bytes,
+                                const void* in, size_t batch, size_t rows, size_t cols,
+                                size_t row_stride, uint32_t quant_version, void* out, int sync);
+
 /* Chunked prefill over paged KV (MFMA path).  No counterpart in the reference,
  * which prefills by looping the decode path once per prompt token
  * (compiler/runtime/batched_executor.cpp:454-466); semantics are the decode
@@ -235,6 +252,8 @@ int mlc_hip_last_decode_work_items(void);
  *   "decode_pv_fp16"        1 = softmax weights rounded to fp16 for the P.V product
  *                           (v_dot2_f32_f16, fp32 accumulate), 0 = fp32 weights
  *   "decode_force_generic"  1 = always use the shape-agnostic kernel
+ *   "q4_force_generic"      1 = Q4_0 matmul always on the scalar kernel
+ *   "q4_ksplit"             K slices of the Q4_0 MFMA matmul (0 = automatic)
  *   "prefill_stages"        2, 4, 6 or 8 K/V tiles staged in LDS by the prefill kernel (0 = automatic)
  * Returns 0 for an unknown name or value. */
 int mlc_hip_set_option(const char* name, long value);

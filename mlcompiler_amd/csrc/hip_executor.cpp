@@ -160,6 +160,15 @@ bool HipExecutor::encodeGateUpSplitSiluMul(void* gate_up_buf, void* gate_buf, vo
                                           ffn_gate_up_rows, /*sync=*/0) != 0;
 }
 
+bool HipExecutor::encodeMatMulQ4_0Batched(const std::string& weight_name,
+                                          const std::vector<uint8_t>& weights, void* in_buf,
+                                          size_t batch, size_t rows, size_t cols, size_t row_stride,
+                                          uint32_t quant_version, void* out_buf) const {
+    return mlc_hip_matmul_q4_0_batched(weight_name.c_str(), weights.data(), weights.size(), in_buf,
+                                       batch, rows, cols, row_stride, quant_version, out_buf,
+                                       /*sync=*/0) != 0;
+}
+
 bool HipExecutor::runPagedPrefillAttention(void* q_f16_buffer, void* k_pages_buffer,
                                            void* v_pages_buffer, void* o_buffer,
                                            const std::vector<uint32_t>& page_tables_flat,

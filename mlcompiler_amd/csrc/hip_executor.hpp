@@ -11,6 +11,7 @@
 
 #include <cstddef>
 #include <cstdint>
+#include <string>
 #include <vector>
 
 namespace mlc_amd {
@@ -97,6 +98,11 @@ public:
                               size_t total_elements) const;
     bool encodeGateUpSplitSiluMul(void* gate_up_buf, void* gate_buf, void* up_buf, void* out_buf,
                                   size_t batch, size_t ffn_inner, size_t ffn_gate_up_rows) const;
+
+    // metal_runtime.hpp:481-489
+    bool encodeMatMulQ4_0Batched(const std::string& weight_name, const std::vector<uint8_t>& weights,
+                                 void* in_buf, size_t batch, size_t rows, size_t cols,
+                                 size_t row_stride, uint32_t quant_version, void* out_buf) const;
 
     // Chunked prefill over paged KV: no reference method (the reference loops its
     // decode path per prompt token, batched_executor.cpp:454-466).

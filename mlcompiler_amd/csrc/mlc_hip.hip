@@ -22,6 +22,7 @@
 #include "paged_prefill_kernels.h"
 #include "paged_rope_kernels.h"
 #include "walker_kernels.h"
+#include "q4_matmul_kernels.h"
 
 namespace mlc_hip {
 // Defined in paged_decode_inst.hip, one object per (head_dim, heads-per-wave).
@@ -84,6 +85,17 @@ struct Ctx {
     bool pass_open = false;
     std::unordered_map<std::string, std::pair<void*, size_t>> cached;
     std::unordered_map<const void*, size_t> allocs;  // base pointer -> bytes (ours only)
+    // Quantised weights, uploaded once per name (getOrCacheWeight, metal_runtime.mm:2434-2437):
+    // the raw rows and, for shapes the MFMA path takes, the repacked nibbles and scales.
+    struct Q4Weight {
+        size_t bytes = 0, rows = 0, cols = 0, stride = 0;
+        void* raw = nullptr;
+        void* qs = nullptr;
+        void* d = nullptr;
+    };
+    std::unordered_map<std::string, Q4Weight> q4_weights;
+    long opt_q4_force_generic = 0;
+    long opt_q4_ksplit = 0;  // 0 = automatic
     MetaSlot ring[8];
     int ring_next = 0;
     MetaSlot plan_slots[4];
@@ -953,6 +965,122 @@ int mlc_hip_gate_up_split_silu_mul(const void* gate_up, void* gate, void* up, vo
     return finish(sync);
 }
 
+// ---- batched Q4_0 matmul -------------------------------------------------------------------
+
+namespace {
+
+bool q4_fast_shape(size_t rows, size_t cols, size_t row_stride) {
+    return rows % 64 == 0 && cols % 32 == 0 && row_stride >= cols / 32 * 18;
+}
+
+// Uploads the weight matrix on first use of its name (or when its size changed).
+Ctx::Q4Weight* q4_weight(const char* name, const uint8_t* host, size_t bytes, size_t rows, size_t cols,
+                         size_t stride) {
+    Ctx::Q4Weight& w = g.q4_weights[name];
+    if (w.raw && w.bytes == bytes && w.rows == rows && w.cols == cols && w.stride == stride) return &w;
+    (void)hipStreamSynchronize(g.stream);
+    for (void** p : {&w.raw, &w.qs, &w.d})
+        if (*p) { (void)hipFree(*p); *p = nullptr; }
+    w = Ctx::Q4Weight{};
+    void* raw = nullptr;
+    if (hipMalloc(&raw, bytes) != hipSuccess) { (void)hipGetLastError(); fail("q4 matmul: hipMalloc failed"); return nullptr; }
+    if (hipMemcpy(raw, host, bytes, hipMemcpyHostToDevice) != hipSuccess) { (void)hipFree(raw); fail("q4 matmul: upload failed"); return nullptr; }
+    w.raw = raw; w.bytes = bytes; w.rows = rows; w.cols = cols; w.stride = stride;
+    if (q4_fast_shape(rows, cols, stride)) {
+        const size_t nb = cols / 32, tiles = rows / 32;
+        std::vector<uint8_t> qs(tiles * nb * 64 * 8);
+        std::vector<uint16_t> d(tiles * nb * 32);
+        for (size_t t = 0; t < tiles; ++t)
+            for (size_t b = 0; b < nb; ++b)
+                for (size_t m = 0; m < 32; ++m) {
+                    const uint8_t* blk = host + (t * 32 + m) * stride + b * 18;
+                    std::memcpy(&d[(t * nb + b) * 32 + m], blk, 2);
+                    for (size_t h = 0; h < 2; ++h)
+                        std::memcpy(&qs[((t * nb + b) * 64 + h * 32 + m) * 8], blk + 2 + h * 8, 8);
+                }
+        if (hipMalloc(&w.qs, qs.size()) != hipSuccess || hipMalloc(&w.d, d.size() * 2) != hipSuccess ||
+            hipMemcpy(w.qs, qs.data(), qs.size(), hipMemcpyHostToDevice) != hipSuccess ||
+            hipMemcpy(w.d, d.data(), d.size() * 2, hipMemcpyHostToDevice) != hipSuccess) {
+            (void)hipGetLastError();
+            fail("q4 matmul: repacked upload failed");
+            return nullptr;
+        }
+    }
+    return &w;
+}
+
+}  // namespace
+
+int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, size_t weight_bytes,
+                                const void* in, size_t batch, size_t rows, size_t cols,
+                                size_t row_stride, uint32_t quant_version, void* out, int sync) {
+    (void)quant_version;  // one block format: quantization.cpp:228-246 ignores it as well
+    if (!init_once()) return fail("GPU unavailable");
+    if (!sync && !g.pass_open) return fail("encode: no open forward pass");
+    if (!in || !out || batch == 0 || rows == 0 || cols == 0) return fail("q4 matmul: null buffer or zero size");  // :6940
+    if (cols < 64 || (rows % 4u) != 0) return fail("q4 matmul: needs cols >= 64 and rows % 4 == 0");          // :6942
+    if (!weight_name || !weights) return fail("q4 matmul: null weights");
+    const size_t nb = (cols + 31) / 32;
+    if (row_stride < nb * 18 || weight_bytes < (rows - 1) * row_stride + nb * 18)
+        return fail("q4 matmul: weight bytes do not cover rows x row_stride");
+    if (batch * rows > 0x7FFFFFFFull || batch * cols > 0x7FFFFFFFull) return fail("q4 matmul: too many elements");
+    const size_t ki = known_bytes(in), ko = known_bytes(out);
+    if ((ki && batch * cols * 4 > ki) || (ko && batch * rows * 4 > ko)) return fail("q4 matmul: buffer too small");
+    Ctx::Q4Weight* w = q4_weight(weight_name, static_cast<const uint8_t*>(weights), weight_bytes, rows, cols, row_stride);
+    if (!w) return 0;
+
+    if (!w->qs || g.opt_q4_force_generic || (reinterpret_cast<uintptr_t>(out) & 15u)) {
+        const size_t waves = batch * rows;
+        hipLaunchKernelGGL(q4_0_matmul_generic_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, g.stream,
+                           static_cast<const uint8_t*>(w->raw), static_cast<const float*>(in),
+                           static_cast<float*>(out), (uint32_t)batch, (uint32_t)rows, (uint32_t)cols,
+                           (uint32_t)row_stride);
+        return finish(sync);
+    }
+
+    // MFMA path, one pass over at most 64 requests at a time
+    const size_t nblocks = cols / 32, pairs = rows / 64;
+    size_t ksplit = (size_t)g.opt_q4_ksplit;
+    if (ksplit == 0) {
+        // workgroups of 256 rows x one slice (8 waves): aim at one per CU, slices of at least 8 blocks
+        const size_t groups = (pairs + 3) / 4;
+        ksplit = std::max<size_t>(1, (256 + groups / 2) / groups);
+        ksplit = std::min(ksplit, std::max<size_t>(1, nblocks / 8));
+    }
+    ksplit = std::min(ksplit, nblocks);
+    const size_t per_slice = (nblocks + ksplit - 1) / ksplit;
+    ksplit = (nblocks + per_slice - 1) / per_slice;
+    for (size_t bo = 0; bo < batch; bo += 64) {
+        const size_t bn = std::min<size_t>(64, batch - bo);
+        const size_t bpad = (bn + 31) / 32 * 32;
+        _Float16* frag = static_cast<_Float16*>(mlc_hip_cached("q4_x_fragments", bpad * cols * 4));
+        float* inv = static_cast<float*>(mlc_hip_cached("q4_x_inv_scale", 64 * 4));
+        float* slices = ksplit > 1 ? static_cast<float*>(mlc_hip_cached("q4_k_slices", ksplit * bn * rows * 4)) : nullptr;
+        if (!frag || !inv || (ksplit > 1 && !slices)) return fail("q4 matmul: scratch allocation failed");
+        const float* xin = static_cast<const float*>(in) + bo * cols;
+        float* o = static_cast<float*>(out) + bo * rows;
+        hipLaunchKernelGGL(q4_split_activations_kernel, dim3((unsigned)bpad), dim3(256), 0, g.stream, xin, frag,
+                           inv, (uint32_t)bn, (uint32_t)cols);
+        Q4Args a;
+        a.qs = static_cast<const uint2*>(w->qs);
+        a.d = static_cast<const _Float16*>(w->d);
+        a.xfrag = frag;
+        a.inv_scale = inv;
+        a.out = ksplit > 1 ? slices : o;
+        a.batch = (uint32_t)bn; a.rows = (uint32_t)rows; a.nblocks = (uint32_t)nblocks;
+        a.blocks_per_slice = (uint32_t)per_slice; a.ksplit = (uint32_t)ksplit;
+        const dim3 grid((unsigned)((pairs + 3) / 4), (unsigned)ksplit);
+        if (bpad == 32) hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<1>), grid, dim3(512), 0, g.stream, a);
+        else hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<2>), grid, dim3(512), 0, g.stream, a);
+        if (ksplit > 1) {
+            const uint32_t n = (uint32_t)(bn * rows);
+            hipLaunchKernelGGL(q4_sum_slices_kernel, dim3((n + 255) / 256), dim3(256), 0, g.stream, slices, o, n,
+                               (uint32_t)ksplit);
+        }
+    }
+    return finish(sync);
+}
+
 int mlc_hip_paged_attn_prefill(const void* q_f16, const void* k_pages, const void* v_pages,
                                void* o, const uint32_t* page_tables_flat, size_t n_flat,
                                const uint32_t* page_table_offsets, const uint32_t* seq_lens,
@@ -1042,6 +1170,12 @@ int mlc_hip_set_option(const char* name, long value) {
     if (!std::strcmp(name, "decode_target_items")) { g.opt_target_items = value; return 1; }
     if (!std::strcmp(name, "decode_force_generic")) { g.opt_force_generic = value; return 1; }
     if (!std::strcmp(name, "decode_pv_fp16")) { g.opt_pv_fp16 = value ? 1 : 0; return 1; }
+    if (!std::strcmp(name, "q4_force_generic")) { g.opt_q4_force_generic = value ? 1 : 0; return 1; }
+    if (!std::strcmp(name, "q4_ksplit")) {
+        if (value < 0 || value > 64) return 0;
+        g.opt_q4_ksplit = value;
+        return 1;
+    }
     if (!std::strcmp(name, "prefill_stages")) {
         if (value != 0 && value != 2 && value != 4 && value != 6 && value != 8) return 0;
         g.opt_prefill_stages = value;

@@ -204,6 +204,14 @@ class HipExecutor:
             gate_up_buf, gate_buf, up_buf, out_buf, batch, ffn_inner, ffn_gate_up_rows,
             int(bool(sync))))
 
+    def encodeMatMulQ4_0Batched(self, weight_name, weights, in_buf, batch, rows, cols, row_stride,
+                                quant_version, out_buf, sync: bool = False) -> bool:
+        """metal_runtime.hpp:481-489; `weights` is the host byte array of the Q4_0 rows."""
+        w = np.ascontiguousarray(weights, np.uint8)
+        return bool(self._lib.mlc_hip_matmul_q4_0_batched(
+            weight_name.encode(), w.ctypes.data, w.size, in_buf, batch, rows, cols, row_stride,
+            quant_version, out_buf, int(bool(sync))))
+
     # -- chunked prefill (no reference method; see include/mlc_hip.h)
     def runPagedPrefillAttention(self, q_f16_buffer, k_pages_buffer, v_pages_buffer, o_buffer,
                                  page_tables_flat, page_table_offsets, seq_lens, q_start, batch,
