@@ -1042,10 +1042,17 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
     const size_t nblocks = cols / 32, pairs = rows / 64;
     size_t ksplit = (size_t)g.opt_q4_ksplit;
     if (ksplit == 0) {
-        // workgroups of 256 rows x one slice (8 waves): aim at one per CU, slices of at least 8 blocks
-        const size_t groups = (pairs + 3) / 4;
-        ksplit = std::max<size_t>(1, (256 + groups / 2) / groups);
-        ksplit = std::min(ksplit, std::max<size_t>(1, nblocks / 8));
+        // One workgroup (8 waves, 256 rows, one slice) per CU and round: the kernel is bound by
+        // its MFMAs, about 1 us per block and round; every slice also costs writing and
+        // re-reading one partial result (about 3 TB/s).
+        const size_t groups = (pairs + 3) / 4, cus = 256;
+        const double slice_us = (double)std::min<size_t>(batch, 64) * (double)rows * 8.0 / 3.0e6;
+        double best = 1e30;
+        for (size_t ks = 1; ks <= std::min<size_t>(32, std::max<size_t>(1, nblocks / 4)); ++ks) {
+            const double rounds = (double)((groups * ks + cus - 1) / cus);
+            const double cost = rounds * (double)((nblocks + ks - 1) / ks) + (ks > 1 ? slice_us * (double)ks : 0.0);
+            if (cost < best) { best = cost; ksplit = ks; }
+        }
     }
     ksplit = std::min(ksplit, nblocks);
     const size_t per_slice = (nblocks + ksplit - 1) / ksplit;

@@ -151,7 +151,7 @@ __device__ __forceinline__ q4_half2 q4_pair(uint32_t bytes, uint32_t sel) {
 static constexpr int kQ4ChunkBlocks = 8;  // Q4_0 blocks (of 32 columns) staged in LDS at a time
 
 // One workgroup: 256 weight rows x NBT batch tiles of 32 x one K slice, taken in chunks of 8
-// blocks.  8 waves: wave w works on the 64 rows (two 32-row tiles) number w % 4 and on the
+// blocks that are double buffered.  8 waves: wave w works on the 64 rows (two 32-row tiles) number w % 4 and on the
 // blocks of parity w / 4, so every SIMD holds two waves whose unpacking (VALU) and MFMAs
 // overlap; the two halves are added through LDS at the end.  Per chunk the waves copy the
 // chunk's activation fragments into LDS (global -> LDS loads, shared by all waves) and their
@@ -161,6 +161,7 @@ __global__ __launch_bounds__(512) void q4_0_matmul_mfma_kernel(const Q4Args a) {
     constexpr int CB = kQ4ChunkBlocks;
     constexpr int FRAGS = CB * NBT * 4;  // 1 KiB fragments per chunk: [block][batch tile][k step][hi, lo]
     __shared__ __attribute__((aligned(16))) unsigned char xs[FRAGS * 1024];
+    __shared__ __attribute__((aligned(16))) unsigned char xs1[FRAGS * 1024];
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const uint32_t lane = threadIdx.x % 64;
     const uint32_t l32 = lane % 32, half = lane / 32;
@@ -182,21 +183,23 @@ __global__ __launch_bounds__(512) void q4_0_matmul_mfma_kernel(const Q4Args a) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[r][t][i] = 0.f;
 
-    for (uint32_t cb = b0; cb < b1; cb += CB) {
-        const uint32_t nbk = min((uint32_t)CB, b1 - cb);
-        // ---- this wave's weights of the chunk (blocks 2*jj + khalf) -> registers
+    // A chunk's loads: this wave's weights (blocks 2*jj + khalf of the chunk) -> registers, and
+    // its share of the chunk's activation fragments -> LDS (fragment f by wave f % 8).
+    struct Weights {
         uint2 q[CB / 2][2];
         _Float16 d[CB / 2][2];
+    };
+    auto issue = [&](uint32_t cb, unsigned char* xbuf, Weights& w) __attribute__((always_inline)) {
+        const uint32_t nbk = min((uint32_t)CB, b1 - cb);
 #pragma unroll
         for (int jj = 0; jj < CB / 2; ++jj)
 #pragma unroll
             for (int r = 0; r < 2; ++r) {
                 const uint32_t blk = cb + min(2u * jj + khalf, nbk - 1u);  // past the end: a repeat, unused
                 const size_t tb = (size_t)(pair * 2 + r) * a.nblocks + blk;
-                q[jj][r] = a.qs[tb * 64 + lane];
-                d[jj][r] = a.d[tb * 32 + l32];
+                w.q[jj][r] = a.qs[tb * 64 + lane];
+                w.d[jj][r] = a.d[tb * 32 + l32];
             }
-        // ---- the chunk's activation fragments -> LDS, fragment f by wave f % 8
 #pragma unroll
         for (int i = 0; i < FRAGS / 8; ++i) {
             const uint32_t f = i * 8 + wave;
@@ -205,11 +208,12 @@ __global__ __launch_bounds__(512) void q4_0_matmul_mfma_kernel(const Q4Args a) {
             const _Float16* src =
                 a.xfrag + ((((size_t)t * ksteps + (cb + j) * 2 + ks) * 2 + p) * 64 + lane) * 8;
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                             (__attribute__((address_space(3))) void*)(xs + f * 1024), 16, 0, 0);
+                                             (__attribute__((address_space(3))) void*)(xbuf + f * 1024), 16, 0, 0);
         }
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
-        // ---- unpack + MFMA
+    };
+    // unpack + MFMA over the chunk's blocks of this wave
+    auto compute = [&](uint32_t cb, const unsigned char* xbuf, const Weights& w) __attribute__((always_inline)) {
+        const uint32_t nbk = min((uint32_t)CB, b1 - cb);
 #pragma unroll
         for (int jj = 0; jj < CB / 2; ++jj) {
             const uint32_t j = 2u * jj + khalf;
@@ -222,15 +226,15 @@ __global__ __launch_bounds__(512) void q4_0_matmul_mfma_kernel(const Q4Args a) {
 #pragma unroll
                     for (int p = 0; p < 2; ++p)
                         xf[t][ks][p] = *reinterpret_cast<const q4_half8*>(
-                            xs + (size_t)((((j * NBT + t) * 2 + ks) * 2 + p) * 1024) + lane * 16);
+                            xbuf + (size_t)((((j * NBT + t) * 2 + ks) * 2 + p) * 1024) + lane * 16);
 #pragma unroll
             for (int r = 0; r < 2; ++r) {
-                const q4_half2 d2 = {d[jj][r], d[jj][r]};
+                const q4_half2 d2 = {w.d[jj][r], w.d[jj][r]};
                 // k step 0: low nibbles of this lane's 8 bytes, k step 1: high nibbles
 #pragma unroll
                 for (int ks = 0; ks < 2; ++ks) {
-                    const uint32_t w0 = (ks ? (q[jj][r].x >> 4) : q[jj][r].x) & 0x0F0F0F0Fu;
-                    const uint32_t w1 = (ks ? (q[jj][r].y >> 4) : q[jj][r].y) & 0x0F0F0F0Fu;
+                    const uint32_t w0 = (ks ? (w.q[jj][r].x >> 4) : w.q[jj][r].x) & 0x0F0F0F0Fu;
+                    const uint32_t w1 = (ks ? (w.q[jj][r].y >> 4) : w.q[jj][r].y) & 0x0F0F0F0Fu;
                     q4_half2 n[4] = {q4_pair(w0, 0x04010400u), q4_pair(w0, 0x04030402u),
                                      q4_pair(w1, 0x04010400u), q4_pair(w1, 0x04030402u)};
                     q4_half8 whi, wlo;
@@ -250,8 +254,25 @@ __global__ __launch_bounds__(512) void q4_0_matmul_mfma_kernel(const Q4Args a) {
                 }
             }
         }
-        __syncthreads();  // everyone is done with xs before the next chunk (or the epilogue) reuses it
+    };
+    // Two staging buffers and two register sets: the loads of chunk c+1 are in flight while
+    // chunk c is multiplied.  One barrier per chunk: it says that everybody's loads of chunk c
+    // have landed and that everybody has left chunk c-1, whose buffer chunk c+1 overwrites.
+    Weights wa, wb;
+    issue(b0, xs, wa);
+    for (uint32_t cb = b0; cb < b1; cb += 2 * CB) {
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        if (cb + CB < b1) issue(cb + CB, xs1, wb);
+        compute(cb, xs, wa);
+        if (cb + CB >= b1) break;
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        if (cb + 2 * CB < b1) issue(cb + 2 * CB, xs, wa);
+        compute(cb + CB, xs1, wb);
     }
+    __syncthreads();  // everyone is done with the staging memory: the steps below reuse it
+
     // ---- the odd-block waves hand their sums to the even-block waves (staging memory is free:
     // the loop ended with a barrier)
     static_assert(4 * 2 * NBT * 16 * 64 * 4 <= FRAGS * 1024, "partial sums fit the staging buffer");
