@@ -145,6 +145,155 @@ def bench_prefill(args) -> int:
     return 0
 
 
+def bench_layer(args) -> int:
+    """One whole decoder layer per step (TinyLlama-1.1B shape, Q4_0 weights) around the paged
+    decode attention of configuration 2: the eleven operators of the reference's layer loop
+    (compiler/runtime/batched_walker.cpp:246-405) enqueued through the C ABI with no host wait
+    between them.  Reports the algorithmic bytes (Q4_0 weights + KV read) per second."""
+    import ctypes as C
+
+    import layer_case as lc
+    from mlcompiler_amd import HipExecutor
+    from mlcompiler_amd.build import BENCH_LIB_PATH
+    exe = HipExecutor.Instance()
+    exe.requireAvailable()
+    if args.q4_ksplit:
+        exe.setOption("q4_ksplit", args.q4_ksplit)
+    if args.no_fuse:
+        exe.setOption("fuse_row_ops", 0)
+    case, n_layers = build_workload("cfg2")
+    c = case
+    B = c.batch
+    w = lc.make_layer_weights(7)
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((B, lc.HID)).astype(np.float32)
+    qpos = c.q_positions.astype(np.uint32)
+    cos, sin = lc.rotary_tables(qpos)
+    # the step's new K/V row of request r goes to the slot of its newest position
+    page_ids = np.array([c.page_tables_flat[c.page_table_offsets[r] + qpos[r] // c.page_size]
+                         for r in range(B)], np.uint32)
+    slots = (qpos % c.page_size).astype(np.uint32)
+
+    keep = []
+
+    def up(a):
+        a = np.ascontiguousarray(a)
+        b = exe.allocateScratchBuffer(a.nbytes)
+        assert b and exe.uploadToBuffer(b, a), "out of device memory"
+        keep.append(a)
+        return b
+
+    def dev(n_floats):
+        b = exe.allocateScratchBuffer(n_floats * 4)
+        assert b
+        return b
+
+    k_bufs = [up(c.k_pages) for _ in range(n_layers)]
+    v_bufs = [up(c.v_pages) for _ in range(n_layers)]
+    u32p, f32p = C.POINTER(C.c_uint32), C.POINTER(C.c_float)
+
+    class Layer(C.Structure):
+        _fields_ = ([(n, C.c_void_p) for n in
+                     ("x", "norm", "qkv", "q", "attn", "o", "resid", "gate_up", "gate", "up", "mix",
+                      "down", "out", "cos", "sin")]
+                    + [("attn_norm_w", f32p), ("ffn_norm_w", f32p)]
+                    + [(n, t) for wn in ("w_qkv", "w_o", "w_gate_up", "w_down")
+                       for n, t in ((wn, C.c_void_p), (wn + "_bytes", C.c_size_t))]
+                    + [(n, C.c_size_t) for n in ("hidden", "ffn_inner", "num_heads", "kv_heads",
+                                                 "head_dim", "page_size_tokens", "batch")]
+                    + [("page_ids", u32p), ("slots", u32p), ("page_tables_flat", u32p),
+                       ("n_flat", C.c_size_t), ("page_table_offsets", u32p), ("seq_lens", u32p),
+                       ("q_positions", u32p)])
+
+    meta = {n: np.ascontiguousarray(a, np.uint32) for n, a in
+            (("page_ids", page_ids), ("slots", slots), ("page_tables_flat", c.page_tables_flat),
+             ("page_table_offsets", c.page_table_offsets), ("seq_lens", c.seq_lens),
+             ("q_positions", qpos))}
+    L = Layer()
+    L.x, L.cos, L.sin = up(x), up(cos), up(sin)
+    for n, cols in (("norm", lc.HID), ("qkv", lc.QKV_ROWS), ("q", lc.Q_ROWS), ("attn", lc.HID),
+                    ("o", lc.HID), ("resid", lc.HID), ("gate_up", 2 * lc.FFN), ("gate", lc.FFN),
+                    ("up", lc.FFN), ("mix", lc.FFN), ("down", lc.HID), ("out", lc.HID)):
+        setattr(L, n, dev(B * cols))
+    L.attn_norm_w = w["g_attn"].ctypes.data_as(f32p)
+    L.ffn_norm_w = w["g_ffn"].ctypes.data_as(f32p)
+    for field, key in (("w_qkv", "w_qkv"), ("w_o", "w_o"), ("w_gate_up", "w_gu"), ("w_down", "w_down")):
+        setattr(L, field, w[key].ctypes.data)
+        setattr(L, field + "_bytes", w[key].nbytes)
+    L.hidden, L.ffn_inner, L.num_heads, L.kv_heads = lc.HID, lc.FFN, lc.H, lc.HKV
+    L.head_dim, L.page_size_tokens, L.batch = lc.D, c.page_size, B
+    for n, a in meta.items():
+        setattr(L, n, a.ctypes.data_as(u32p))
+    L.n_flat = meta["page_tables_flat"].size
+
+    bl = C.CDLL(BENCH_LIB_PATH)
+    kp = (C.c_void_p * n_layers)(*k_bufs)
+    vp = (C.c_void_p * n_layers)(*v_bufs)
+
+    def loop(steps):
+        ms, wall_s = C.c_float(), C.c_double()
+        if not bl.mlc_bench_layer_loop(C.byref(L), kp, vp, C.c_size_t(n_layers), C.c_size_t(steps),
+                                       C.byref(ms), C.byref(wall_s)):
+            raise RuntimeError("layer loop failed: " + exe.lastError())
+        return ms.value, wall_s.value
+
+    loop(max(args.warmup, n_layers))     # also uploads and repacks the weights (first use of a name)
+    ev_ms, wall = loop(args.steps)
+    out = np.empty((B, lc.HID), np.float32)
+    exe.downloadFromBuffer(L.out, out)
+
+    w_bytes = lc.weight_bytes(w)
+    alg_bytes = w_bytes + c.kv_bytes
+    us = wall / args.steps * 1e6
+    ev_us = ev_ms / args.steps * 1e3
+    value = alg_bytes / (wall / args.steps) / 1e9
+    ach = alg_bytes / (ev_us * 1e-6) / 1e9
+    result = {
+        "metric": "decoder layer (Q4_0 weights + KV read) GB/s & us/layer, TinyLlama shape B=32",
+        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": max(args.warmup, n_layers), "ms_per_step": round(us / 1e3, 6),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32 (Q4_0 weights, fp16 K/V storage; matmuls on split-fp16 MFMA with fp32 accumulate)",
+        "data": "synthetic",
+        "config": {
+            "workload": f"decoder layer, TinyLlama-1.1B shape (hidden {lc.HID}, {lc.H}q/{lc.HKV}kv heads, "
+                        f"head_dim {lc.D}, ffn {lc.FFN}), batch {B}, contexts of {c.name} "
+                        f"(sum {int(c.seq_lens.sum())}), 11 operators per step, {n_layers} K/V pools rotated",
+            "weight_bytes_per_step": w_bytes, "kv_bytes_per_step": c.kv_bytes,
+            "us_per_layer": round(us, 2),
+            "tokens_per_s_at_22_layers": round(B / (22 * us * 1e-6), 1),
+        },
+        "roofline": {"bound": "hbm", "achieved": round(ach, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None,
+                     "us_per_launch": round(ev_us, 2),
+                     "note": "whole layer (all its kernels) between HIP events / steps; per-kernel "
+                             "durations are in the rocprofv3 summary of this workload"},
+    }
+    if not args.no_cpu:
+        from oracle import paged_oracle as po
+        nb = 8   # bounded sample: the first 8 requests of the batch, one thread
+        off = c.page_table_offsets
+        flat = c.page_tables_flat[:off[nb]]
+        t0 = time.perf_counter()
+        ref = lc.oracle_chain(w, x[:nb], cos[:nb], sin[:nb], c.k_pages, c.v_pages, page_ids[:nb],
+                              slots[:nb], flat, off[:nb + 1], c.seq_lens[:nb], qpos[:nb], n_threads=1)
+        dt = time.perf_counter() - t0
+        # the CPU reads the weights once per request: bytes that count are per request
+        b_s = (w_bytes + int(c.seq_lens[:nb].sum()) * 4 * lc.HKV * lc.D / nb) * nb
+        result["cpu_baseline"] = {"value": round(b_s / dt / 1e9, 4), "unit": "GB/s", "cores": 1,
+                                  "kind": "port",
+                                  "sample": f"{nb} of {B} requests through the same 11 operators, "
+                                            f"{dt:.2f} s ({dt / nb * 1e3:.1f} ms per token-layer)",
+                                  "us_per_layer_at_full_batch": round(dt / nb * B * 1e6, 1)}
+        got = out[:nb]
+        rel = float(np.max(np.abs(got - ref["out"])) / np.max(np.abs(ref["out"])))
+        result["parity_vs_cpu_baseline"] = {"cosine": round(po.cosine(got.ravel(), ref["out"].ravel()), 8),
+                                            "max_abs_over_max": float(f"{rel:.3e}"),
+                                            "requests_checked": nb}
+    print(json.dumps(result))
+    return 0
+
+
 def build_workload(name: str):
     from paged_cases import baseline_config
     idx = {"cfg1": 1, "cfg2": 2, "cfg3": 3, "cfg4": 4}[name]
@@ -213,12 +362,14 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=100)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "copy"])
+    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "layer", "copy"])
     ap.add_argument("--copy-mib", type=int, default=32, help="size of the calibration copy")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU baseline work")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--target-items", type=int, default=0)
     ap.add_argument("--prefill-stages", type=int, default=0, help="cfg5: LDS pipeline depth (0 = automatic)")
+    ap.add_argument("--q4-ksplit", type=int, default=0, help="layer: K slices of the Q4_0 matmuls (0 = automatic)")
+    ap.add_argument("--no-fuse", action="store_true", help="layer: launch every operator on its own")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); "
@@ -229,6 +380,8 @@ def main() -> int:
         return bench_prefill(args)
     if args.workload == "copy":
         return bench_copy(args)
+    if args.workload == "layer":
+        return bench_layer(args)
 
     from mlcompiler_amd import HipExecutor
     exe = HipExecutor.Instance()

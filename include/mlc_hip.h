@@ -242,6 +242,8 @@ float mlc_hip_timer_stop(void);
  * number of split-K work items it planned (for benchmarks and tests). */
 int mlc_hip_last_decode_launches(void);
 int mlc_hip_last_decode_work_items(void);
+/* Number of fused row-operator launches so far (for tests of "fuse_row_ops"). */
+long mlc_hip_row_program_launches(void);
 
 /* Tunables (0 selects the automatic choice where noted):
  *   "decode_target_items"   split-K work items aimed for per launch (0 = automatic)
@@ -254,6 +256,12 @@ int mlc_hip_last_decode_work_items(void);
  *   "decode_force_generic"  1 = always use the shape-agnostic kernel
  *   "q4_force_generic"      1 = Q4_0 matmul always on the scalar kernel
  *   "q4_ksplit"             K slices of the Q4_0 MFMA matmul (0 = automatic)
+ *   "fuse_row_ops"          1 (default) = row-local operators encoded back to back in a pass
+ *                           (sum of matmul K slices, add, RMSNorm, gate/up SiLU, the fp16 split
+ *                           of the next matmul's input) are collected and launched as one
+ *                           kernel when something else is encoded, the pass is flushed or a
+ *                           call has sync = 1; every output buffer is still written.
+ *                           0 = each operator is launched when it is encoded
  *   "prefill_stages"        2, 4, 6 or 8 K/V tiles staged in LDS by the prefill kernel (0 = automatic)
  * Returns 0 for an unknown name or value. */
 int mlc_hip_set_option(const char* name, long value);

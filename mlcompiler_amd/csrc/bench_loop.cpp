@@ -128,4 +128,69 @@ int mlc_bench_copy_loop(const void* src, void* dst, size_t bytes, size_t steps, 
     return 1;
 }
 
+// One whole decoder layer per step, in the order of the reference's layer loop
+// (compiler/runtime/batched_walker.cpp:246-405): RMSNorm, qkv matmul, split + RoPE + KV write,
+// paged attention, out-projection, add, RMSNorm, gate/up matmul, SiLU gate, down-projection,
+// add.  Layer i uses K/V pool i % n_layers (the weights are the same for every layer: they
+// are re-read from HBM all the same, 12 MB do not stay in cache next to the KV traffic).
+struct MlcBenchLayer {
+    const void* x;            // [batch][hidden] fp32 input of the layer
+    void* norm; void* qkv; void* q; void* attn; void* o; void* resid; void* gate_up;
+    void* gate; void* up; void* mix; void* down; void* out;
+    const void* cos; const void* sin;
+    const float* attn_norm_w; const float* ffn_norm_w;
+    const void* w_qkv; size_t w_qkv_bytes;
+    const void* w_o; size_t w_o_bytes;
+    const void* w_gate_up; size_t w_gate_up_bytes;
+    const void* w_down; size_t w_down_bytes;
+    size_t hidden, ffn_inner, num_heads, kv_heads, head_dim, page_size_tokens, batch;
+    const uint32_t* page_ids; const uint32_t* slots;
+    const uint32_t* page_tables_flat; size_t n_flat;
+    const uint32_t* page_table_offsets; const uint32_t* seq_lens; const uint32_t* q_positions;
+};
+
+int mlc_bench_layer_loop(const MlcBenchLayer* L, void* const* k_pools, void* const* v_pools,
+                         size_t n_layers, size_t steps, float* event_ms, double* wall_s) {
+    const size_t B = L->batch, HID = L->hidden, FFN = L->ffn_inner;
+    const size_t q_rows = L->num_heads * L->head_dim, kv_rows = L->kv_heads * L->head_dim;
+    const size_t qkv_rows = q_rows + 2 * kv_rows;
+    const size_t s_hid = HID / 32 * 18, s_ffn = FFN / 32 * 18;
+    if (!mlc_hip_begin()) return 0;
+    const auto t0 = std::chrono::steady_clock::now();
+    if (!mlc_hip_timer_start()) return 0;
+    for (size_t i = 0; i < steps; ++i) {
+        const size_t l = i % n_layers;
+        int ok = mlc_hip_rms_norm_batched(L->x, L->attn_norm_w, HID, 1e-5f, B, HID, L->norm, 0);
+        ok = ok && mlc_hip_matmul_q4_0_batched("bench.attn_qkv", L->w_qkv, L->w_qkv_bytes, L->norm, B,
+                                               qkv_rows, HID, s_hid, 1, L->qkv, 0);
+        ok = ok && mlc_hip_qkv_split_rope_scatter(L->qkv, L->q, k_pools[l], v_pools[l], nullptr, nullptr,
+                                                  L->cos, L->sin, L->page_ids, L->slots,
+                                                  L->page_size_tokens, B, L->num_heads, L->kv_heads,
+                                                  L->head_dim, qkv_rows, q_rows, kv_rows, kv_rows,
+                                                  L->head_dim, 0);
+        ok = ok && mlc_hip_paged_attn_decode(L->q, k_pools[l], v_pools[l], L->attn, L->page_tables_flat,
+                                             L->n_flat, L->page_table_offsets, L->seq_lens,
+                                             L->q_positions, B, L->num_heads, L->kv_heads, L->head_dim,
+                                             L->page_size_tokens, 1, 0);
+        ok = ok && mlc_hip_matmul_q4_0_batched("bench.attn_output", L->w_o, L->w_o_bytes, L->attn, B, HID,
+                                               HID, s_hid, 1, L->o, 0);
+        ok = ok && mlc_hip_add_batched(L->x, L->o, L->resid, B * HID, 0);
+        ok = ok && mlc_hip_rms_norm_batched(L->resid, L->ffn_norm_w, HID, 1e-5f, B, HID, L->norm, 0);
+        ok = ok && mlc_hip_matmul_q4_0_batched("bench.ffn_gate_up", L->w_gate_up, L->w_gate_up_bytes,
+                                               L->norm, B, 2 * FFN, HID, s_hid, 1, L->gate_up, 0);
+        ok = ok && mlc_hip_gate_up_split_silu_mul(L->gate_up, L->gate, L->up, L->mix, B, FFN, 2 * FFN, 0);
+        ok = ok && mlc_hip_matmul_q4_0_batched("bench.ffn_down", L->w_down, L->w_down_bytes, L->mix, B,
+                                               HID, FFN, s_ffn, 1, L->down, 0);
+        ok = ok && mlc_hip_add_batched(L->resid, L->down, L->out, B * HID, 0);
+        if (!ok) return 0;
+    }
+    const float ms = mlc_hip_timer_stop();
+    if (ms < 0.f) return 0;
+    if (!mlc_hip_flush()) return 0;
+    const auto t1 = std::chrono::steady_clock::now();
+    if (event_ms) *event_ms = ms;
+    if (wall_s) *wall_s = std::chrono::duration<double>(t1 - t0).count();
+    return 1;
+}
+
 }  // extern "C"

@@ -12,6 +12,8 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <map>
+#include <tuple>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -98,6 +100,29 @@ struct Ctx {
     long opt_q4_ksplit = 0;  // 0 = automatic
     MetaSlot ring[8];
     int ring_next = 0;
+    // Small host arrays that callers pass again and again with the same content (norm weights,
+    // the page ids of a decode step across its layers): kept on the device, uploaded only when
+    // the content changes.
+    struct Resident {
+        std::vector<unsigned char> content;
+        void* dev = nullptr;
+        size_t cap = 0;
+    };
+    std::map<std::tuple<int, const void*, size_t>, Resident> resident;
+    // Row-local operators of the open pass that have been encoded but not launched yet: a chain
+    // that one row_program_kernel launch can run (walker_kernels.h).  Everything else that
+    // touches the stream or device memory calls settle() first.
+    struct RowPending {
+        bool active = false;
+        RowProgram p{};
+        size_t batch = 0;            // 0 while only the flat element count is known (a lone add)
+        size_t n_flat = 0;
+        size_t len = 0;              // current row length
+        const void* cur = nullptr;   // buffer that will hold the chain's current values
+        size_t grid_rows = 0;        // rows launched (padded to a multiple of 32 for the split stage)
+    } rows;
+    long opt_fuse_rows = 1;          // 0 = every operator is launched when it is encoded
+    long row_launches = 0;           // row_program_kernel launches (for tests)
     MetaSlot plan_slots[4];
     int plan_next = 0;
     DecodePlan plan;
@@ -173,6 +198,40 @@ int slot_mark(MetaSlot& s) {
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
+// Device copy of a small host blob, uploaded only when (kind, key, bytes) has not been seen
+// with this content.  The copy is ordered on the library stream, so kernels already enqueued
+// that read the previous content are not disturbed.  nullptr on failure (error recorded).
+const void* resident_blob(int kind, const void* key, const void* blob, size_t bytes) {
+    if (g.resident.size() > 1024) {  // a caller that never repeats itself: start over
+        if (hipStreamSynchronize(g.stream) != hipSuccess) { fail("resident: synchronize failed"); return nullptr; }
+        for (auto& kv : g.resident)
+            if (kv.second.dev) (void)hipFree(kv.second.dev);
+        g.resident.clear();
+    }
+    Ctx::Resident& r = g.resident[std::make_tuple(kind, key, bytes)];
+    if (r.dev && r.content.size() == bytes && std::memcmp(r.content.data(), blob, bytes) == 0) return r.dev;
+    if (bytes > r.cap) {
+        if (r.dev && hipFree(r.dev) != hipSuccess) { fail("resident: hipFree failed"); return nullptr; }
+        r.dev = nullptr;
+        r.cap = 0;
+        const size_t cap = std::max<size_t>(256, align_up(bytes, 256));
+        if (hipMalloc(&r.dev, cap) != hipSuccess) { r.dev = nullptr; fail("resident: hipMalloc failed"); return nullptr; }
+        r.cap = cap;
+    }
+    r.content.clear();  // not valid until the copy has been enqueued
+    MetaSlot& s = g.ring[g.ring_next];
+    g.ring_next = (g.ring_next + 1) % 8;
+    if (!slot_reserve(s, bytes)) return nullptr;
+    std::memcpy(s.host, blob, bytes);
+    if (hipMemcpyAsync(r.dev, s.host, bytes, hipMemcpyHostToDevice, g.stream) != hipSuccess) {
+        fail("resident: upload failed");
+        return nullptr;
+    }
+    if (!slot_mark(s)) return nullptr;
+    r.content.assign(static_cast<const unsigned char*>(blob), static_cast<const unsigned char*>(blob) + bytes);
+    return r.dev;
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 size_t known_bytes(const void* p) {
@@ -180,10 +239,85 @@ size_t known_bytes(const void* p) {
     return it == g.allocs.end() ? 0 : it->second;
 }
 
+constexpr size_t kRowMaxLen = 16384;  // row_program_kernel: 8 groups of 8 elements per thread
+
+bool row_len_ok(size_t len) { return len > 0 && len % 8 == 0 && len <= kRowMaxLen; }
+
+// Launches what the pending chain holds.
+int settle() {
+    Ctx::RowPending& r = g.rows;
+    if (!r.active) return 1;
+    r.active = false;
+    const RowProgram& p = r.p;
+    if (r.batch == 0) {  // a lone add over a flat range
+        hipLaunchKernelGGL(add_kernel, dim3((unsigned)((r.n_flat + 255) / 256)), dim3(256), 0, g.stream, p.src,
+                           p.addend, p.add_out, (uint32_t)r.n_flat);
+        HIP_OK(hipGetLastError());
+        return 1;
+    }
+    if (r.len > kRowMaxLen) {  // only a sum over K slices can be this long (nothing joined it)
+        const uint32_t n = (uint32_t)(r.batch * r.len);
+        hipLaunchKernelGGL(q4_sum_slices_kernel, dim3((n + 255) / 256), dim3(256), 0, g.stream, p.src, p.src_store, n,
+                           p.n_slices);
+        HIP_OK(hipGetLastError());
+        return 1;
+    }
+    const dim3 grid((unsigned)(p.frag ? r.grid_rows : r.batch));
+    if (r.len <= 8 * (size_t)kRowThreads) hipLaunchKernelGGL((row_program_kernel<1>), grid, dim3(kRowThreads), 0, g.stream, p);
+    else hipLaunchKernelGGL((row_program_kernel<2>), grid, dim3(kRowThreads), 0, g.stream, p);
+    ++g.row_launches;
+    HIP_OK(hipGetLastError());
+    return 1;
+}
+
+// True when the pending chain's current values are those of `buf` as rows of `len` floats; fixes
+// the row shape of a chain that so far only knew its element count.
+bool rows_continue(const void* buf, size_t batch, size_t len) {
+    Ctx::RowPending& r = g.rows;
+    if (!g.opt_fuse_rows || !r.active || r.cur != buf || r.p.frag) return false;
+    if (r.batch == 0) {
+        if (r.n_flat != batch * len || !row_len_ok(len)) return false;
+        r.batch = batch;
+        r.len = len;
+        r.p.len_src = (uint32_t)len;
+        r.p.batch = (uint32_t)batch;
+        return true;
+    }
+    return r.batch == batch && r.len == len;  // callers check that the length they go on with fits
+}
+
+// Starts a chain whose source is a plain buffer of rows.
+void rows_begin(const void* src, size_t batch, size_t len) {
+    Ctx::RowPending& r = g.rows;
+    r = Ctx::RowPending{};
+    r.active = true;
+    r.p.src = static_cast<const float*>(src);
+    r.p.n_slices = 1;
+    r.p.len_src = (uint32_t)len;
+    r.p.batch = (uint32_t)batch;
+    r.batch = batch;
+    r.len = len;
+    r.n_flat = batch * len;
+    r.cur = src;
+}
+
 int finish(int sync) {
     HIP_OK(hipGetLastError());
-    if (sync) HIP_OK(hipStreamSynchronize(g.stream));
+    if (sync) {
+        if (!settle()) return 0;
+        HIP_OK(hipStreamSynchronize(g.stream));
+    }
     return 1;
+}
+
+// Page ids and slots of one batched KV write, side by side in one resident blob: the layers of
+// a decode step all write to the same (page, slot) per request, so only the first of them uploads.
+const void* resident_ids(const uint32_t* page_ids, const uint32_t* slots, size_t batch, size_t ids_bytes) {
+    static thread_local std::vector<unsigned char> blob;
+    blob.assign(ids_bytes * 2, 0);
+    std::memcpy(blob.data(), page_ids, batch * 4);
+    std::memcpy(blob.data() + ids_bytes, slots, batch * 4);
+    return resident_blob(1, nullptr, blob.data(), blob.size());
 }
 
 // ---------------------------------------------------------------- decode plan
@@ -443,12 +577,15 @@ void* mlc_hip_alloc(size_t bytes) {
 
 void mlc_hip_free(void* buffer) {
     if (!buffer || !init_once()) return;
+    (void)settle();
     (void)hipStreamSynchronize(g.stream);
     g.allocs.erase(buffer);
     (void)hipFree(buffer);
 }
 
-void* mlc_hip_cached(const char* name, size_t bytes) {
+namespace {
+// Named grow-only device buffer; does not touch the pending row chain.
+void* cached_buffer(const char* name, size_t bytes) {
     if (!init_once() || !name) return nullptr;
     auto it = g.cached.find(name);
     if (it != g.cached.end() && it->second.second >= bytes) return it->second.first;
@@ -468,9 +605,16 @@ void* mlc_hip_cached(const char* name, size_t bytes) {
     g.allocs[p] = bytes;
     return p;
 }
+}  // namespace
+
+void* mlc_hip_cached(const char* name, size_t bytes) {
+    if (!init_once() || !settle()) return nullptr;
+    return cached_buffer(name, bytes);
+}
 
 int mlc_hip_upload(void* buffer, const void* src, size_t bytes, size_t dst_offset) {
     if (!init_once()) return fail("GPU unavailable");
+    if (!settle()) return 0;
     if (!buffer || (!src && bytes)) return fail("upload: null pointer");
     if (!bytes) return 1;
     const size_t known = known_bytes(buffer);
@@ -483,6 +627,7 @@ int mlc_hip_upload(void* buffer, const void* src, size_t bytes, size_t dst_offse
 
 int mlc_hip_download(const void* buffer, void* dst, size_t bytes, size_t src_offset) {
     if (!init_once()) return fail("GPU unavailable");
+    if (!settle()) return 0;
     if (!buffer || (!dst && bytes)) return fail("download: null pointer");
     if (!bytes) return 1;
     const size_t known = known_bytes(buffer);
@@ -495,6 +640,7 @@ int mlc_hip_download(const void* buffer, void* dst, size_t bytes, size_t src_off
 
 int mlc_hip_zero(void* buffer, size_t bytes) {
     if (!init_once()) return fail("GPU unavailable");
+    if (!settle()) return 0;
     if (!buffer) return fail("zero: null pointer");
     const size_t known = known_bytes(buffer);
     if (known && bytes > known) return fail("zero: beyond the buffer");
@@ -510,6 +656,7 @@ int mlc_hip_begin(void) {
 
 int mlc_hip_flush(void) {
     if (!init_once()) return fail("GPU unavailable");
+    if (!settle()) return 0;
     if (!g.pass_open) return 1;
     g.pass_open = false;
     HIP_OK(hipStreamSynchronize(g.stream));
@@ -525,6 +672,7 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
                               size_t kv_heads, size_t head_dim, size_t page_size_tokens,
                               int apply_causal, int sync) {
     if (!init_once()) return fail("GPU unavailable");
+    if (!settle()) return 0;
     if (!sync && !g.pass_open) return fail("encode: no open forward pass");  // :7090
     // metal_runtime.mm:7742-7750
     if (!q || !k_pages || !v_pages || !o) return fail("decode: null buffer");
@@ -608,6 +756,7 @@ int mlc_hip_scatter_kv_paged_batched_f16(void* page_storage, const uint32_t* pag
                                          size_t n_kv_heads, size_t head_dim, size_t batch,
                                          const void* src, int sync) {
     if (!init_once()) return fail("GPU unavailable");
+    if (!settle()) return 0;
     if (!sync && !g.pass_open) return fail("encode: no open forward pass");  // :7178
     // metal_runtime.mm:7241-7243
     if (!page_storage || !src) return fail("scatter: null buffer");
@@ -628,15 +777,11 @@ int mlc_hip_scatter_kv_paged_batched_f16(void* page_storage, const uint32_t* pag
     const size_t known_src = known_bytes(src);
     if (known_src && batch * row_bytes > known_src) return fail("scatter: src too small");
 
-    MetaSlot& s = g.ring[g.ring_next];
-    g.ring_next = (g.ring_next + 1) % 8;
     const size_t ids_bytes = align_up(batch * 4, 16);
-    if (!slot_reserve(s, ids_bytes * 2)) return 0;
-    std::memcpy(s.host, page_ids, batch * 4);
-    std::memcpy(static_cast<char*>(s.host) + ids_bytes, slots_in_page, batch * 4);
-    if (!slot_upload(s, ids_bytes * 2)) return 0;
-    const uint32_t* d_ids = static_cast<const uint32_t*>(s.dev);
-    const uint32_t* d_slots = reinterpret_cast<const uint32_t*>(static_cast<char*>(s.dev) + ids_bytes);
+    const char* d_blob = static_cast<const char*>(resident_ids(page_ids, slots_in_page, batch, ids_bytes));
+    if (!d_blob) return 0;
+    const uint32_t* d_ids = reinterpret_cast<const uint32_t*>(d_blob);
+    const uint32_t* d_slots = reinterpret_cast<const uint32_t*>(d_blob + ids_bytes);
 
     const unsigned block = 256;
     if ((row_bytes % 16) == 0 && aligned16(page_storage) && aligned16(src)) {
@@ -654,7 +799,6 @@ int mlc_hip_scatter_kv_paged_batched_f16(void* page_storage, const uint32_t* pag
                            static_cast<const uint16_t*>(src), static_cast<uint16_t*>(page_storage),
                            d_ids, d_slots, (uint32_t)batch, row_units, (uint32_t)page_size_tokens);
     }
-    if (!slot_mark(s)) return 0;
     return finish(sync);
 }
 
@@ -663,6 +807,7 @@ int mlc_hip_scatter_kv_paged(void* page_storage, const uint32_t* page_table, siz
                              size_t tokens, size_t start_slot, const void* src,
                              size_t dtype_bytes) {
     if (!init_once()) return fail("GPU unavailable");
+    if (!settle()) return 0;
     // metal_runtime.mm:7839-7845
     if (!page_storage || !src) return fail("scatter_paged: null buffer");
     if (page_size_tokens == 0 || n_kv_heads == 0 || head_dim == 0 || tokens == 0)
@@ -718,6 +863,7 @@ int mlc_hip_gather_kv_pages(const void* page_storage, const uint32_t* page_table
                             size_t n_page_table, size_t page_size_tokens, size_t n_kv_heads,
                             size_t head_dim, size_t num_tokens, void* dst, size_t dtype_bytes) {
     if (!init_once()) return fail("GPU unavailable");
+    if (!settle()) return 0;
     // metal_runtime.mm:7657-7662
     if (!page_storage || !dst) return fail("gather: null buffer");
     if (page_size_tokens == 0 || n_kv_heads == 0 || head_dim == 0 || num_tokens == 0)
@@ -804,6 +950,7 @@ int mlc_hip_qkv_split_rope_cast(const void* qkv, void* q, void* k, void* v, void
                                 size_t q_rows, size_t k_rows, size_t v_rows, size_t rotary_dim,
                                 int sync) {
     if (!init_once()) return fail("GPU unavailable");
+    if (!settle()) return 0;
     if (!sync && !g.pass_open) return fail("encode: no open forward pass");  // :7936
     if (const char* why = rope_args_problem(qkv, q, cos_buf, sin_buf, batch, num_heads, kv_heads,
                                             head_dim, qkv_rows, q_rows, k_rows, v_rows, rotary_dim))
@@ -841,6 +988,7 @@ int mlc_hip_qkv_split_rope_scatter(const void* qkv, void* q, void* k_pages, void
                                    size_t kv_heads, size_t head_dim, size_t qkv_rows, size_t q_rows,
                                    size_t k_rows, size_t v_rows, size_t rotary_dim, int sync) {
     if (!init_once()) return fail("GPU unavailable");
+    if (!settle()) return 0;
     if (!sync && !g.pass_open) return fail("encode: no open forward pass");
     if (const char* why = rope_args_problem(qkv, q, cos_buf, sin_buf, batch, num_heads, kv_heads,
                                             head_dim, qkv_rows, q_rows, k_rows, v_rows, rotary_dim))
@@ -860,13 +1008,9 @@ int mlc_hip_qkv_split_rope_scatter(const void* qkv, void* q, void* k_pages, void
         if ((known_k && end > known_k) || (known_v && end > known_v))
             return fail("qkv split: page id beyond the pool");
     }
-    MetaSlot& s = g.ring[g.ring_next];
-    g.ring_next = (g.ring_next + 1) % 8;
     const size_t ids_bytes = align_up(batch * 4, 16);
-    if (!slot_reserve(s, ids_bytes * 2)) return 0;
-    std::memcpy(s.host, page_ids, batch * 4);
-    std::memcpy(static_cast<char*>(s.host) + ids_bytes, slots_in_page, batch * 4);
-    if (!slot_upload(s, ids_bytes * 2)) return 0;
+    const char* d_blob = static_cast<const char*>(resident_ids(page_ids, slots_in_page, batch, ids_bytes));
+    if (!d_blob) return 0;
     RopeArgs a{};
     a.qkv = static_cast<const float*>(qkv);
     a.q = static_cast<float*>(q);
@@ -876,13 +1020,12 @@ int mlc_hip_qkv_split_rope_scatter(const void* qkv, void* q, void* k_pages, void
     a.v_pages = static_cast<_Float16*>(v_pages);
     a.cos_table = static_cast<const float*>(cos_buf);
     a.sin_table = static_cast<const float*>(sin_buf);
-    a.page_ids = static_cast<const uint32_t*>(s.dev);
-    a.slots = reinterpret_cast<const uint32_t*>(static_cast<char*>(s.dev) + ids_bytes);
+    a.page_ids = reinterpret_cast<const uint32_t*>(d_blob);
+    a.slots = reinterpret_cast<const uint32_t*>(d_blob + ids_bytes);
     a.batch = (uint32_t)batch; a.head_dim = (uint32_t)head_dim; a.qkv_rows = (uint32_t)qkv_rows;
     a.q_rows = (uint32_t)q_rows; a.k_rows = (uint32_t)k_rows; a.v_rows = (uint32_t)v_rows;
     a.rotary_dim = (uint32_t)rotary_dim; a.page_size = (uint32_t)page_size_tokens;
     launch_qkv_split_rope_cast<true>(a, g.stream);
-    if (!slot_mark(s)) return 0;
     return finish(sync);
 }
 
@@ -898,17 +1041,28 @@ int mlc_hip_rms_norm_batched(const void* in, const float* weight, size_t n_weigh
     const size_t ki = known_bytes(in), ko = known_bytes(out);
     if ((ki && batch * length * 4 > ki) || (ko && batch * length * 4 > ko))
         return fail("rms norm: buffer too small");
-    // the weight vector is borrowed for the call: staged like the other metadata
-    MetaSlot& s = g.ring[g.ring_next];
-    g.ring_next = (g.ring_next + 1) % 8;
-    const size_t w_bytes = std::max<size_t>(align_up(n_weight * 4, 16), 16);
-    if (!slot_reserve(s, w_bytes)) return 0;
-    if (n_weight) std::memcpy(s.host, weight, n_weight * 4);
-    if (!slot_upload(s, w_bytes)) return 0;
+    const bool fusable = row_len_ok(length) && aligned16(in) && aligned16(out);
+    const bool joins = fusable && !g.rows.p.rms && rows_continue(in, batch, length);
+    if (!joins && !settle()) return 0;  // before the weight's device copy may be replaced
+    // the weight vector is borrowed for the call; its device copy is kept between calls
+    const float one = 1.0f;
+    const void* d_weight = resident_blob(0, weight, n_weight ? (const void*)weight : (const void*)&one,
+                                         n_weight ? n_weight * 4 : 4);
+    if (!d_weight) return 0;
+    if (fusable && g.opt_fuse_rows) {
+        if (!joins) rows_begin(in, batch, length);
+        RowProgram& p = g.rows.p;
+        p.rms = 1;
+        p.rms_weight = static_cast<const float*>(d_weight);
+        p.n_weight = (uint32_t)n_weight;
+        p.epsilon = epsilon;
+        p.rms_out = static_cast<float*>(out);
+        g.rows.cur = out;
+        return finish(sync);
+    }
     hipLaunchKernelGGL(rms_norm_batched_kernel, dim3((unsigned)batch), dim3(256), 0, g.stream,
-                       static_cast<const float*>(in), static_cast<const float*>(s.dev),
+                       static_cast<const float*>(in), static_cast<const float*>(d_weight),
                        (uint32_t)n_weight, epsilon, (uint32_t)length, static_cast<float*>(out));
-    if (!slot_mark(s)) return 0;
     return finish(sync);
 }
 
@@ -929,6 +1083,25 @@ int mlc_hip_add_batched(const void* a, const void* b, void* out, size_t total_el
     if (!init_once()) return fail("GPU unavailable");
     if (!sync && !g.pass_open) return fail("encode: no open forward pass");
     if (const char* why = flat3_problem(a, b, out, total_elements, "add")) return fail(why);  // :7018
+    const bool fusable = g.opt_fuse_rows && total_elements % 8 == 0 && aligned16(a) && aligned16(b) && aligned16(out);
+    Ctx::RowPending& r = g.rows;
+    const bool joins = fusable && r.active && (r.cur == a || r.cur == b) && !r.p.addend && !r.p.rms && !r.p.frag &&
+                       (r.batch ? r.batch * r.len == total_elements && row_len_ok(r.len) : r.n_flat == total_elements);
+    if (!joins && !settle()) return 0;
+    if (fusable) {
+        const void* other = a;
+        if (joins) {
+            other = r.cur == a ? b : a;
+        } else {
+            rows_begin(a, 0, 0);
+            r.n_flat = total_elements;
+            other = b;
+        }
+        r.p.addend = static_cast<const float*>(other);
+        r.p.add_out = static_cast<float*>(out);
+        r.cur = out;
+        return finish(sync);
+    }
     hipLaunchKernelGGL(add_kernel, dim3((unsigned)((total_elements + 255) / 256)), dim3(256), 0, g.stream,
                        static_cast<const float*>(a), static_cast<const float*>(b),
                        static_cast<float*>(out), (uint32_t)total_elements);
@@ -938,6 +1111,7 @@ int mlc_hip_add_batched(const void* a, const void* b, void* out, size_t total_el
 int mlc_hip_silu_mul_batched(const void* gate, const void* up, void* out, size_t total_elements,
                              int sync) {
     if (!init_once()) return fail("GPU unavailable");
+    if (!settle()) return 0;
     if (!sync && !g.pass_open) return fail("encode: no open forward pass");
     if (const char* why = flat3_problem(gate, up, out, total_elements, "silu mul")) return fail(why);  // :7048
     hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((total_elements + 255) / 256)), dim3(256), 0,
@@ -957,6 +1131,22 @@ int mlc_hip_gate_up_split_silu_mul(const void* gate_up, void* gate, void* up, vo
     if (batch * ffn_gate_up_rows > 0x7FFFFFFFull) return fail("gate/up split: too many elements");
     const size_t kg = known_bytes(gate_up);
     if (kg && batch * ffn_gate_up_rows * 4 > kg) return fail("gate/up split: gate_up buffer too small");
+    {
+        Ctx::RowPending& r = g.rows;
+        const bool joins = ffn_gate_up_rows == 2 * ffn_inner && row_len_ok(ffn_inner) && aligned16(gate) &&
+                           aligned16(up) && aligned16(out) && !r.p.silu && !r.p.addend && !r.p.rms &&
+                           rows_continue(gate_up, batch, ffn_gate_up_rows);
+        if (joins) {
+            r.p.silu = 1;
+            r.p.gate_out = static_cast<float*>(gate);
+            r.p.up_out = static_cast<float*>(up);
+            r.p.silu_out = static_cast<float*>(out);
+            r.len = ffn_inner;
+            r.cur = out;
+            return finish(sync);
+        }
+        if (!settle()) return 0;
+    }
     const size_t n = batch * ffn_inner;
     hipLaunchKernelGGL(gate_up_split_silu_mul_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
                        g.stream, static_cast<const float*>(gate_up), static_cast<float*>(gate),
@@ -1026,10 +1216,16 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
     if (batch * rows > 0x7FFFFFFFull || batch * cols > 0x7FFFFFFFull) return fail("q4 matmul: too many elements");
     const size_t ki = known_bytes(in), ko = known_bytes(out);
     if ((ki && batch * cols * 4 > ki) || (ko && batch * rows * 4 > ko)) return fail("q4 matmul: buffer too small");
+    // does the pending chain end in this matmul's input?  (decided before anything below can
+    // replace a buffer the chain still refers to)
+    const bool feeds = batch <= 64 && !g.opt_q4_force_generic && !(reinterpret_cast<uintptr_t>(out) & 15u) &&
+                       q4_fast_shape(rows, cols, row_stride) && rows_continue(in, batch, cols);
+    if (!feeds && !settle()) return 0;
     Ctx::Q4Weight* w = q4_weight(weight_name, static_cast<const uint8_t*>(weights), weight_bytes, rows, cols, row_stride);
     if (!w) return 0;
 
     if (!w->qs || g.opt_q4_force_generic || (reinterpret_cast<uintptr_t>(out) & 15u)) {
+        if (!settle()) return 0;
         const size_t waves = batch * rows;
         hipLaunchKernelGGL(q4_0_matmul_generic_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, g.stream,
                            static_cast<const uint8_t*>(w->raw), static_cast<const float*>(in),
@@ -1038,36 +1234,39 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
         return finish(sync);
     }
 
-    // MFMA path, one pass over at most 64 requests at a time
-    const size_t nblocks = cols / 32, pairs = rows / 64;
+    // MFMA path, one pass over at most 64 requests at a time.  A workgroup takes one or two
+    // 32-row tiles and, unless K is split, all of K; two tiles when one would give more
+    // workgroups than CUs.  K is split only to fill CUs that would otherwise idle, and only as
+    // far as a workgroup keeps about 64 blocks of work.
+    const size_t nblocks = cols / 32, tiles = rows / 32;
+    const int row_tiles = tiles > 256 ? 2 : 1;
+    const size_t wgs = tiles / row_tiles;
     size_t ksplit = (size_t)g.opt_q4_ksplit;
-    if (ksplit == 0) {
-        // One workgroup (8 waves, 256 rows, one slice) per CU and round: the kernel is bound by
-        // its MFMAs, about 1 us per block and round; every slice also costs writing and
-        // re-reading one partial result (about 3 TB/s).
-        const size_t groups = (pairs + 3) / 4, cus = 256;
-        const double slice_us = (double)std::min<size_t>(batch, 64) * (double)rows * 8.0 / 3.0e6;
-        double best = 1e30;
-        for (size_t ks = 1; ks <= std::min<size_t>(32, std::max<size_t>(1, nblocks / 4)); ++ks) {
-            const double rounds = (double)((groups * ks + cus - 1) / cus);
-            const double cost = rounds * (double)((nblocks + ks - 1) / ks) + (ks > 1 ? slice_us * (double)ks : 0.0);
-            if (cost < best) { best = cost; ksplit = ks; }
-        }
-    }
-    ksplit = std::min(ksplit, nblocks);
+    if (ksplit == 0)
+        ksplit = std::max<size_t>(1, std::min<size_t>(256 / std::max<size_t>(wgs, 1), (nblocks * row_tiles + 63) / 64));
+    ksplit = std::min(ksplit, std::max<size_t>(1, nblocks / 16));
     const size_t per_slice = (nblocks + ksplit - 1) / ksplit;
     ksplit = (nblocks + per_slice - 1) / per_slice;
     for (size_t bo = 0; bo < batch; bo += 64) {
         const size_t bn = std::min<size_t>(64, batch - bo);
         const size_t bpad = (bn + 31) / 32 * 32;
-        _Float16* frag = static_cast<_Float16*>(mlc_hip_cached("q4_x_fragments", bpad * cols * 4));
-        float* inv = static_cast<float*>(mlc_hip_cached("q4_x_inv_scale", 64 * 4));
-        float* slices = ksplit > 1 ? static_cast<float*>(mlc_hip_cached("q4_k_slices", ksplit * bn * rows * 4)) : nullptr;
-        if (!frag || !inv || (ksplit > 1 && !slices)) return fail("q4 matmul: scratch allocation failed");
+        _Float16* frag = static_cast<_Float16*>(cached_buffer("q4_x_fragments", bpad * cols * 4));
+        float* inv = static_cast<float*>(cached_buffer("q4_x_inv_scale", 64 * 4));
+        if (!frag || !inv) return fail("q4 matmul: scratch allocation failed");
         const float* xin = static_cast<const float*>(in) + bo * cols;
         float* o = static_cast<float*>(out) + bo * rows;
-        hipLaunchKernelGGL(q4_split_activations_kernel, dim3((unsigned)bpad), dim3(256), 0, g.stream, xin, frag,
-                           inv, (uint32_t)bn, (uint32_t)cols);
+        if (feeds) {  // the chain that produces the input also splits it (batch <= 64: one round)
+            g.rows.p.frag = frag;
+            g.rows.p.inv_scale = inv;
+            g.rows.grid_rows = bpad;
+            if (!settle()) return 0;
+        } else {
+            hipLaunchKernelGGL(q4_split_activations_kernel, dim3((unsigned)bpad), dim3(256), 0, g.stream, xin, frag,
+                               inv, (uint32_t)bn, (uint32_t)cols);
+        }
+        // (the chain has been launched: its K-slice source may be replaced now)
+        float* slices = ksplit > 1 ? static_cast<float*>(cached_buffer("q4_k_slices", ksplit * bn * rows * 4)) : nullptr;
+        if (ksplit > 1 && !slices) return fail("q4 matmul: scratch allocation failed");
         Q4Args a;
         a.qs = static_cast<const uint2*>(w->qs);
         a.d = static_cast<const _Float16*>(w->d);
@@ -1076,13 +1275,28 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
         a.out = ksplit > 1 ? slices : o;
         a.batch = (uint32_t)bn; a.rows = (uint32_t)rows; a.nblocks = (uint32_t)nblocks;
         a.blocks_per_slice = (uint32_t)per_slice; a.ksplit = (uint32_t)ksplit;
-        const dim3 grid((unsigned)((pairs + 3) / 4), (unsigned)ksplit);
-        if (bpad == 32) hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<1>), grid, dim3(512), 0, g.stream, a);
-        else hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<2>), grid, dim3(512), 0, g.stream, a);
+        const dim3 grid((unsigned)wgs, (unsigned)ksplit);
+        if (bpad == 32) {
+            if (row_tiles == 1) hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<1, 1, 16>), grid, dim3(1024), 0, g.stream, a);
+            else hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<1, 2, 16>), grid, dim3(1024), 0, g.stream, a);
+        } else {
+            if (row_tiles == 1) hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<2, 1, 8>), grid, dim3(512), 0, g.stream, a);
+            else hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<2, 2, 8>), grid, dim3(512), 0, g.stream, a);
+        }
         if (ksplit > 1) {
             const uint32_t n = (uint32_t)(bn * rows);
-            hipLaunchKernelGGL(q4_sum_slices_kernel, dim3((n + 255) / 256), dim3(256), 0, g.stream, slices, o, n,
-                               (uint32_t)ksplit);
+            if (g.opt_fuse_rows && batch <= 64 && rows <= 2 * kRowMaxLen) {
+                // the sum over the slices starts the next chain: whatever row-local operator
+                // consumes this matmul's output joins it
+                rows_begin(slices, bn, rows);
+                g.rows.p.n_slices = (uint32_t)ksplit;
+                g.rows.p.slice_stride = n;
+                g.rows.p.src_store = o;
+                g.rows.cur = o;
+            } else {
+                hipLaunchKernelGGL(q4_sum_slices_kernel, dim3((n + 255) / 256), dim3(256), 0, g.stream, slices, o, n,
+                                   (uint32_t)ksplit);
+            }
         }
     }
     return finish(sync);
@@ -1095,6 +1309,7 @@ int mlc_hip_paged_attn_prefill(const void* q_f16, const void* k_pages, const voi
                                size_t num_heads, size_t kv_heads, size_t head_dim,
                                size_t page_size_tokens, int sync) {
     if (!init_once()) return fail("GPU unavailable");
+    if (!settle()) return 0;
     if (!sync && !g.pass_open) return fail("encode: no open forward pass");
     if (!q_f16 || !k_pages || !v_pages || !o) return fail("prefill: null buffer");
     if (batch == 0 || chunk == 0 || num_heads == 0 || head_dim == 0 || page_size_tokens == 0)
@@ -1152,16 +1367,21 @@ int mlc_hip_paged_attn_prefill(const void* q_f16, const void* k_pages, const voi
     return finish(sync);
 }
 
-void* mlc_hip_stream(void) { return init_once() ? static_cast<void*>(g.stream) : nullptr; }
+void* mlc_hip_stream(void) {
+    if (!init_once() || !settle()) return nullptr;  // the caller may enqueue behind what has been encoded
+    return static_cast<void*>(g.stream);
+}
 
 int mlc_hip_timer_start(void) {
     if (!init_once()) return fail("GPU unavailable");
+    if (!settle()) return 0;
     HIP_OK(hipEventRecord(g.ev0, g.stream));
     return 1;
 }
 
 float mlc_hip_timer_stop(void) {
     if (!init_once()) return -1.f;
+    if (!settle()) return -1.f;
     if (hipEventRecord(g.ev1, g.stream) != hipSuccess) return -1.f;
     if (hipEventSynchronize(g.ev1) != hipSuccess) return -1.f;
     float ms = -1.f;
@@ -1171,9 +1391,12 @@ float mlc_hip_timer_stop(void) {
 
 int mlc_hip_last_decode_launches(void) { return g.last_launches; }
 int mlc_hip_last_decode_work_items(void) { return g.last_items; }
+long mlc_hip_row_program_launches(void) { return g.row_launches; }
 
 int mlc_hip_set_option(const char* name, long value) {
     if (!name) return 0;
+    if (g.inited && g.available && !settle()) return 0;
+    if (!std::strcmp(name, "fuse_row_ops")) { g.opt_fuse_rows = value ? 1 : 0; return 1; }
     if (!std::strcmp(name, "decode_target_items")) { g.opt_target_items = value; return 1; }
     if (!std::strcmp(name, "decode_force_generic")) { g.opt_force_generic = value; return 1; }
     if (!std::strcmp(name, "decode_pv_fp16")) { g.opt_pv_fp16 = value ? 1 : 0; return 1; }

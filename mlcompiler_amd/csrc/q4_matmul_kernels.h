@@ -16,8 +16,9 @@
 // The weights are repacked once, when they enter the library's weight cache, so that the A
 // operand of a 32-row tile is one coalesced 8-byte load per lane and block; the activations
 // are split by a small kernel into the B-operand layout, so that a fragment is one 16-byte
-// load per lane.  K is split over workgroups when there are too few row tiles to fill the
-// chip; the slices are summed in a fixed order by a second small kernel.
+// load per lane.  K is split over workgroups only when there are too few row tiles to fill the
+// chip and K is long; the slices are then summed in a fixed order (q4_sum_slices_kernel, or
+// the fused row kernel of walker_kernels.h).
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -148,184 +149,135 @@ __device__ __forceinline__ q4_half2 q4_pair(uint32_t bytes, uint32_t sel) {
     return __builtin_bit_cast(q4_half2, m) - k1032;
 }
 
-static constexpr int kQ4ChunkBlocks = 8;  // Q4_0 blocks (of 32 columns) staged in LDS at a time
-
-// One workgroup: 256 weight rows x NBT batch tiles of 32 x one K slice, taken in chunks of 8
-// blocks that are double buffered.  8 waves: wave w works on the 64 rows (two 32-row tiles) number w % 4 and on the
-// blocks of parity w / 4, so every SIMD holds two waves whose unpacking (VALU) and MFMAs
-// overlap; the two halves are added through LDS at the end.  Per chunk the waves copy the
-// chunk's activation fragments into LDS (global -> LDS loads, shared by all waves) and their
-// own nibbles and scales into registers, wait once, and then run unpack + MFMA.
-template <int NBT>
-__global__ __launch_bounds__(512) void q4_0_matmul_mfma_kernel(const Q4Args a) {
-    constexpr int CB = kQ4ChunkBlocks;
-    constexpr int FRAGS = CB * NBT * 4;  // 1 KiB fragments per chunk: [block][batch tile][k step][hi, lo]
-    __shared__ __attribute__((aligned(16))) unsigned char xs[FRAGS * 1024];
-    __shared__ __attribute__((aligned(16))) unsigned char xs1[FRAGS * 1024];
+// One workgroup: RT tiles of 32 weight rows x NBT batch tiles of 32 x one K slice.  The
+// slice's blocks are dealt out to the WAVES waves (block b0 + wave, + WAVES, ...); a wave streams
+// its blocks' nibbles, scales and activation fragments straight from memory into registers, PF
+// blocks ahead, unpacks and multiplies; there is no staging memory and no barrier until the
+// waves' sums meet in LDS at the end.  With the whole K range in one workgroup (ksplit = 1) the
+// result goes straight to the output; K slices are only worth it when there are too few row
+// tiles to fill the chip and K is long.
+template <int NBT, int RT, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Args a) {
+    constexpr int PF = WAVES >= 16 ? 2 : 4;  // blocks in flight per wave
+    constexpr int PITCH = 65;                // floats per accumulator register in LDS (bank spread)
+    __shared__ float red[WAVES * RT * NBT * 16 * PITCH];
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const uint32_t lane = threadIdx.x % 64;
-    const uint32_t l32 = lane % 32, half = lane / 32;
-    const uint32_t pairs = a.rows / 64;
-    const uint32_t khalf = wave / 4;                        // parity of the blocks this wave takes
-    const uint32_t pair_raw = blockIdx.x * 4 + wave % 4;    // index of the 64-row pair of tiles
-    const bool active = pair_raw < pairs;             // idle waves still take part in staging
-    const uint32_t pair = active ? pair_raw : pairs - 1;
+    const uint32_t l32 = lane % 32;
+    const uint32_t tile0 = blockIdx.x * RT;
     const uint32_t slice = blockIdx.y;
     const uint32_t b0 = slice * a.blocks_per_slice;
     const uint32_t b1 = min(b0 + a.blocks_per_slice, a.nblocks);
     const uint32_t ksteps = a.nblocks * 2;
 
-    q4_float16 acc[2][NBT];
+    q4_float16 acc[RT][NBT];
 #pragma unroll
-    for (int r = 0; r < 2; ++r)
+    for (int r = 0; r < RT; ++r)
 #pragma unroll
         for (int t = 0; t < NBT; ++t)
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[r][t][i] = 0.f;
 
-    // A chunk's loads: this wave's weights (blocks 2*jj + khalf of the chunk) -> registers, and
-    // its share of the chunk's activation fragments -> LDS (fragment f by wave f % 8).
-    struct Weights {
-        uint2 q[CB / 2][2];
-        _Float16 d[CB / 2][2];
+    struct Block {
+        uint2 q[RT];
+        _Float16 d[RT];
+        q4_half8 x[NBT][2][2];  // [batch tile][k step][hi, lo]
+        bool real;               // false: a repeat past the end of the slice, multiplied with scale 0
     };
-    auto issue = [&](uint32_t cb, unsigned char* xbuf, Weights& w) __attribute__((always_inline)) {
-        const uint32_t nbk = min((uint32_t)CB, b1 - cb);
+    auto load = [&](uint32_t blk_raw, Block& k) __attribute__((always_inline)) {
+        // Past the end of the slice: a repeat of its last block, multiplied with the scale set to
+        // zero, so that the multiply needs no branch (a branch lets the compiler sink these loads
+        // into it, next to their use, which undoes the prefetch).
+        const uint32_t blk = min(blk_raw, b1 - 1u);
+        k.real = blk_raw < b1;
 #pragma unroll
-        for (int jj = 0; jj < CB / 2; ++jj)
-#pragma unroll
-            for (int r = 0; r < 2; ++r) {
-                const uint32_t blk = cb + min(2u * jj + khalf, nbk - 1u);  // past the end: a repeat, unused
-                const size_t tb = (size_t)(pair * 2 + r) * a.nblocks + blk;
-                w.q[jj][r] = a.qs[tb * 64 + lane];
-                w.d[jj][r] = a.d[tb * 32 + l32];
-            }
-#pragma unroll
-        for (int i = 0; i < FRAGS / 8; ++i) {
-            const uint32_t f = i * 8 + wave;
-            const uint32_t p = f % 2, ks = (f / 2) % 2, t = (f / 4) % NBT;
-            const uint32_t j = min(f / (4 * NBT), nbk - 1u);
-            const _Float16* src =
-                a.xfrag + ((((size_t)t * ksteps + (cb + j) * 2 + ks) * 2 + p) * 64 + lane) * 8;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                             (__attribute__((address_space(3))) void*)(xbuf + f * 1024), 16, 0, 0);
+        for (int r = 0; r < RT; ++r) {
+            const size_t tb = (size_t)(tile0 + r) * a.nblocks + blk;
+            k.q[r] = a.qs[tb * 64 + lane];
+            k.d[r] = a.d[tb * 32 + l32];
         }
+#pragma unroll
+        for (int t = 0; t < NBT; ++t)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                for (int p = 0; p < 2; ++p)
+                    k.x[t][ks][p] = *reinterpret_cast<const q4_half8*>(
+                        a.xfrag + ((((size_t)t * ksteps + blk * 2 + ks) * 2 + p) * 64 + lane) * 8);
     };
-    // unpack + MFMA over the chunk's blocks of this wave
-    auto compute = [&](uint32_t cb, const unsigned char* xbuf, const Weights& w) __attribute__((always_inline)) {
-        const uint32_t nbk = min((uint32_t)CB, b1 - cb);
+    auto multiply = [&](const Block& k) __attribute__((always_inline)) {
 #pragma unroll
-        for (int jj = 0; jj < CB / 2; ++jj) {
-            const uint32_t j = 2u * jj + khalf;
-            if (j >= nbk) break;
-            q4_half8 xf[NBT][2][2];
+        for (int r = 0; r < RT; ++r) {
+            const _Float16 d = k.real ? k.d[r] : (_Float16)0.0f;
+            const q4_half2 d2 = {d, d};
+            // k step 0: low nibbles of this lane's 8 bytes, k step 1: high nibbles
 #pragma unroll
-            for (int t = 0; t < NBT; ++t)
+            for (int ks = 0; ks < 2; ++ks) {
+                const uint32_t w0 = (ks ? (k.q[r].x >> 4) : k.q[r].x) & 0x0F0F0F0Fu;
+                const uint32_t w1 = (ks ? (k.q[r].y >> 4) : k.q[r].y) & 0x0F0F0F0Fu;
+                q4_half2 n[4] = {q4_pair(w0, 0x04010400u), q4_pair(w0, 0x04030402u),
+                                 q4_pair(w1, 0x04010400u), q4_pair(w1, 0x04030402u)};
+                q4_half8 whi, wlo;
 #pragma unroll
-                for (int ks = 0; ks < 2; ++ks)
+                for (int e = 0; e < 4; ++e) {
+                    const q4_half2 h = d2 * n[e];
+                    const q4_half2 l = __builtin_elementwise_fma(d2, n[e], -h);
+                    whi[2 * e] = h[0]; whi[2 * e + 1] = h[1];
+                    wlo[2 * e] = l[0]; wlo[2 * e + 1] = l[1];
+                }
 #pragma unroll
-                    for (int p = 0; p < 2; ++p)
-                        xf[t][ks][p] = *reinterpret_cast<const q4_half8*>(
-                            xbuf + (size_t)((((j * NBT + t) * 2 + ks) * 2 + p) * 1024) + lane * 16);
-#pragma unroll
-            for (int r = 0; r < 2; ++r) {
-                const q4_half2 d2 = {w.d[jj][r], w.d[jj][r]};
-                // k step 0: low nibbles of this lane's 8 bytes, k step 1: high nibbles
-#pragma unroll
-                for (int ks = 0; ks < 2; ++ks) {
-                    const uint32_t w0 = (ks ? (w.q[jj][r].x >> 4) : w.q[jj][r].x) & 0x0F0F0F0Fu;
-                    const uint32_t w1 = (ks ? (w.q[jj][r].y >> 4) : w.q[jj][r].y) & 0x0F0F0F0Fu;
-                    q4_half2 n[4] = {q4_pair(w0, 0x04010400u), q4_pair(w0, 0x04030402u),
-                                     q4_pair(w1, 0x04010400u), q4_pair(w1, 0x04030402u)};
-                    q4_half8 whi, wlo;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const q4_half2 h = d2 * n[e];
-                        const q4_half2 l = __builtin_elementwise_fma(d2, n[e], -h);
-                        whi[2 * e] = h[0]; whi[2 * e + 1] = h[1];
-                        wlo[2 * e] = l[0]; wlo[2 * e + 1] = l[1];
-                    }
-#pragma unroll
-                    for (int t = 0; t < NBT; ++t) {
-                        acc[r][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi, xf[t][ks][0], acc[r][t], 0, 0, 0);
-                        acc[r][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi, xf[t][ks][1], acc[r][t], 0, 0, 0);
-                        acc[r][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wlo, xf[t][ks][0], acc[r][t], 0, 0, 0);
-                    }
+                for (int t = 0; t < NBT; ++t) {
+                    acc[r][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi, k.x[t][ks][0], acc[r][t], 0, 0, 0);
+                    acc[r][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi, k.x[t][ks][1], acc[r][t], 0, 0, 0);
+                    acc[r][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wlo, k.x[t][ks][0], acc[r][t], 0, 0, 0);
                 }
             }
         }
     };
-    // Two staging buffers and two register sets: the loads of chunk c+1 are in flight while
-    // chunk c is multiplied.  One barrier per chunk: it says that everybody's loads of chunk c
-    // have landed and that everybody has left chunk c-1, whose buffer chunk c+1 overwrites.
-    Weights wa, wb;
-    issue(b0, xs, wa);
-    for (uint32_t cb = b0; cb < b1; cb += 2 * CB) {
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
-        if (cb + CB < b1) issue(cb + CB, xs1, wb);
-        compute(cb, xs, wa);
-        if (cb + CB >= b1) break;
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
-        if (cb + 2 * CB < b1) issue(cb + 2 * CB, xs, wa);
-        compute(cb + CB, xs1, wb);
-    }
-    __syncthreads();  // everyone is done with the staging memory: the steps below reuse it
 
-    // ---- the odd-block waves hand their sums to the even-block waves (staging memory is free:
-    // the loop ended with a barrier)
-    static_assert(4 * 2 * NBT * 16 * 64 * 4 <= FRAGS * 1024, "partial sums fit the staging buffer");
-    float* red = reinterpret_cast<float*>(xs) + (size_t)(wave % 4) * (2 * NBT * 16 * 64);
-    if (khalf == 1) {
+    // The empty asm statements (they claim to touch memory) pin every group of loads where it
+    // is written: without them the compiler moves the loads for a later block down to just
+    // before their use, across the loop's back edge too, and the prefetch is gone.
+    Block k[PF];
 #pragma unroll
-        for (int r = 0; r < 2; ++r)
-#pragma unroll
-            for (int t = 0; t < NBT; ++t)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) red[((r * NBT + t) * 16 + i) * 64 + lane] = acc[r][t][i];
+    for (int i = 0; i < PF; ++i) {
+        load(b0 + wave + i * WAVES, k[i]);
+        asm volatile("" ::: "memory");
     }
+    for (uint32_t base = b0 + wave; base < b1; base += PF * WAVES) {
+#pragma unroll
+        for (int i = 0; i < PF; ++i) {
+            multiply(k[i]);
+            load(base + (i + PF) * WAVES, k[i]);
+            asm volatile("" ::: "memory");
+        }
+    }
+
+    // ---- the waves' sums meet in LDS.  Accumulator layout: lane holds batch column l32 of the
+    // tile and, in register i, weight row (i/4)*8 + (lane/32)*4 + i%4 of the 32-row tile.
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+        for (int t = 0; t < NBT; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                red[(((wave * RT + r) * NBT + t) * 16 + i) * PITCH + lane] = acc[r][t][i];
     __syncthreads();
-    if (khalf == 0) {
-#pragma unroll
-        for (int r = 0; r < 2; ++r)
-#pragma unroll
-            for (int t = 0; t < NBT; ++t)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) acc[r][t][i] += red[((r * NBT + t) * 16 + i) * 64 + lane];
-    }
-    __syncthreads();  // the epilogue below reuses the same memory
-    if (!active || khalf == 1) return;
-
-    // Accumulator layout: lane holds batch column l32 of the tile and, in register i, weight
-    // row (i/4)*8 + half*4 + i%4 of the 32-row tile.  The tile goes through this wave's part of
-    // the (now free) staging memory so that every store instruction writes whole 128-byte runs
-    // of out[b][row..].
-    static_assert(4 * 32 * 33 * 4 <= FRAGS * 1024, "epilogue tiles fit the staging buffer");
-    float (*tl)[33] = reinterpret_cast<float (*)[33]>(xs + (wave % 4) * (32 * 33 * 4));
+    // thread -> (weight row, batch column): consecutive threads write consecutive rows of out[b][..]
+    constexpr uint32_t ROWS = 32 * RT, COLS_PER_PASS = WAVES * 64 / ROWS;
+    const uint32_t row = threadIdx.x % ROWS, bsub = threadIdx.x / ROWS;
+    const uint32_t r = row / 32, rr = row % 32;
+    const uint32_t i = (rr / 8) * 4 + rr % 4, hf = (rr % 8) / 4;
     float* out = a.out + (size_t)slice * a.batch * a.rows;
 #pragma unroll
-    for (int t = 0; t < NBT; ++t) {
-        const uint32_t b = t * 32 + l32;
-        const float inv = b < a.batch ? a.inv_scale[b] : 0.f;
+    for (uint32_t pass = 0; pass < 32 * NBT / COLS_PER_PASS; ++pass) {
+        const uint32_t b = pass * COLS_PER_PASS + bsub;
+        if (b >= a.batch) continue;
+        const uint32_t t = b / 32, ln = hf * 32 + b % 32;
+        float sum = 0.f;
 #pragma unroll
-        for (int r = 0; r < 2; ++r) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) tl[l32][(i / 4) * 8 + half * 4 + (i % 4)] = acc[r][t][i] * inv;
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            // lane -> (batch row bb = pass*2 + half, weight row l32): 32 consecutive floats per half wave
-#pragma unroll
-            for (int pass = 0; pass < 16; ++pass) {
-                const uint32_t bl = pass * 2 + half;
-                const uint32_t bb = t * 32 + bl;
-                if (bb < a.batch) out[(size_t)bb * a.rows + (pair * 2 + r) * 32 + l32] = tl[bl][l32];
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        }
+        for (int w = 0; w < WAVES; ++w) sum += red[(((w * RT + r) * NBT + t) * 16 + i) * PITCH + ln];
+        out[(size_t)b * a.rows + tile0 * 32 + row] = sum * a.inv_scale[b];
     }
 }
 

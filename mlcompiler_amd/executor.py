@@ -242,6 +242,10 @@ class HipExecutor:
     def lastDecodeWorkItems(self) -> int:
         return int(self._lib.mlc_hip_last_decode_work_items())
 
+    def rowProgramLaunches(self) -> int:
+        """Fused row-operator launches so far (option "fuse_row_ops")."""
+        return int(self._lib.mlc_hip_row_program_launches())
+
     def setOption(self, name: str, value: int) -> bool:
         return bool(self._lib.mlc_hip_set_option(name.encode(), int(value)))
 

@@ -15,26 +15,19 @@ from oracle import paged_oracle as po
 
 pytestmark = pytest.mark.gpu
 
-HID, H, HKV, D, FFN, P = 2048, 32, 4, 64, 5632, 64
-Q_ROWS, KV_ROWS = H * D, HKV * D
-QKV_ROWS = Q_ROWS + 2 * KV_ROWS
-
-
-def _weights(rng, rows, cols, scale):
-    return po.quantize_q4_0((rng.standard_normal((rows, cols)) * scale).astype(np.float32))
+from layer_case import D, FFN, H, HID, HKV, KV_ROWS, P, Q_ROWS, QKV_ROWS, make_layer_weights, oracle_chain, rotary_tables
 
 
 @pytest.mark.timeout(300)
+@pytest.mark.parametrize("fuse", [1, 0])
 @pytest.mark.parametrize("batch", [6, 33])
-def test_decoder_layer_matches_oracle_chain(exe, batch):
-    print(f"[layer] batch={batch}", flush=True)
+def test_decoder_layer_matches_oracle_chain(exe, batch, fuse):
+    """fuse = 1: the row-local operators between the matmuls run as fused launches (the default);
+    fuse = 0: every operator is launched on its own.  Same expected values either way."""
+    print(f"[layer] batch={batch} fuse_row_ops={fuse}", flush=True)
     rng = np.random.default_rng(100 + batch)
-    w_qkv = _weights(rng, QKV_ROWS, HID, 0.03)
-    w_o = _weights(rng, HID, HID, 0.03)
-    w_gu = _weights(rng, 2 * FFN, HID, 0.03)
-    w_down = _weights(rng, HID, FFN, 0.02)
-    g_attn = rng.uniform(0.5, 1.5, HID).astype(np.float32)
-    g_ffn = rng.uniform(0.5, 1.5, HID).astype(np.float32)
+    w = make_layer_weights(200 + batch)
+    w_qkv, w_o, w_gu, w_down, g_attn, g_ffn = (w[n] for n in ("w_qkv", "w_o", "w_gu", "w_down", "g_attn", "g_ffn"))
     x = rng.standard_normal((batch, HID)).astype(np.float32)
 
     # paged KV state before the step: request r holds ctx[r] tokens; this step appends one
@@ -54,27 +47,11 @@ def test_decoder_layer_matches_oracle_chain(exe, batch):
     qpos = seq - 1
     flat = np.concatenate([np.array(r.page_table, np.uint32) for r in reqs])
     off = np.concatenate([[0], np.cumsum([len(r.page_table) for r in reqs])]).astype(np.uint32)
-    cos = np.zeros((batch, D // 2), np.float32)
-    sin = np.zeros((batch, D // 2), np.float32)
-    for r in range(batch):
-        cos[r], sin[r] = po.rotary_coefficients(int(qpos[r]), D)
+    cos, sin = rotary_tables(qpos)
 
     # ---- oracle chain
-    n1 = po.rms_norm_batched(x, g_attn, 1e-5, batch, HID)
-    qkv = po.matmul_q4_0_batched(w_qkv, n1, batch, QKV_ROWS, HID)
-    q, k, v, k16, v16 = po.qkv_split_rope_cast(qkv, cos, sin, batch, H, HKV, D, QKV_ROWS, Q_ROWS, KV_ROWS,
-                                               KV_ROWS, D)
-    want_k, want_v = k_pool.copy(), v_pool.copy()
-    assert po.scatter_kv_paged_batched_f16(want_k, page_ids, slots, P, HKV, D, batch, k16)
-    assert po.scatter_kv_paged_batched_f16(want_v, page_ids, slots, P, HKV, D, batch, v16)
-    attn = po.paged_attention_executor(q, want_k, want_v, flat, off, seq, qpos, batch, H, HKV, D, P, True)
-    o = po.matmul_q4_0_batched(w_o, attn.reshape(batch, HID), batch, HID, HID)
-    r1 = po.add(x, o)
-    n2 = po.rms_norm_batched(r1, g_ffn, 1e-5, batch, HID)
-    gu = po.matmul_q4_0_batched(w_gu, n2, batch, 2 * FFN, HID)
-    _, _, mix = po.gate_up_split_silu_mul(gu, batch, FFN, 2 * FFN)
-    down = po.matmul_q4_0_batched(w_down, mix, batch, HID, FFN)
-    want = po.add(r1, down)
+    ref = oracle_chain(w, x, cos, sin, k_pool, v_pool, page_ids, slots, flat, off, seq, qpos)
+    want, attn, k, want_k = ref["out"], ref["attn"], ref["k"], ref["k_pool"]
 
     # ---- the same on the device, one pass
     def dev(n_floats):
@@ -90,6 +67,8 @@ def test_decoder_layer_matches_oracle_chain(exe, batch):
     bufs = [d_x, d_cos, d_sin, d_k, d_v, d_n, d_qkv, d_q, d_attn, d_o, d_r1, d_gu, d_gate, d_upb, d_mix,
             d_down, d_out]
     tag = f"layer{batch}"
+    assert exe.setOption("fuse_row_ops", fuse)
+    fused_before = exe.rowProgramLaunches()
     try:
         assert exe.beginForwardPassCB()
         ok = exe.encodeRmsNormBatched(d_x, g_attn, 1e-5, batch, HID, d_n)
@@ -112,8 +91,12 @@ def test_decoder_layer_matches_oracle_chain(exe, batch):
         assert exe.downloadFromBuffer(d_out, got) and exe.downloadFromBuffer(d_attn, got_attn)
         assert exe.downloadFromBuffer(d_k, got_k)
     finally:
+        exe.setOption("fuse_row_ops", 1)
         for b in bufs:
             exe.releaseScratchBuffer(b)
+    fused = exe.rowProgramLaunches() - fused_before
+    print(f"  fused row-operator launches: {fused}", flush=True)
+    assert (fused >= 2) if fuse else (fused == 0)
 
     # the KV rows written on the way: fp16 of values that went through two matmul implementations,
     # so equal up to one fp16 step on a few elements
