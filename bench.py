@@ -195,7 +195,7 @@ def bench_layer(args) -> int:
     class Layer(C.Structure):
         _fields_ = ([(n, C.c_void_p) for n in
                      ("x", "norm", "qkv", "q", "attn", "o", "resid", "gate_up", "gate", "up", "mix",
-                      "down", "out", "cos", "sin")]
+                      "down", "out", "out2", "cos", "sin")]
                     + [("attn_norm_w", f32p), ("ffn_norm_w", f32p)]
                     + [(n, t) for wn in ("w_qkv", "w_o", "w_gate_up", "w_down")
                        for n, t in ((wn, C.c_void_p), (wn + "_bytes", C.c_size_t))]
@@ -238,7 +238,12 @@ def bench_layer(args) -> int:
         return ms.value, wall_s.value
 
     loop(max(args.warmup, n_layers))     # also uploads and repacks the weights (first use of a name)
+    # timed: every step reads the step before's output, like the layers of a model (the
+    # residual add of one layer and the RMSNorm of the next are neighbours in the pass)
+    L.out2 = dev(B * lc.HID)
     ev_ms, wall = loop(args.steps)
+    L.out2 = None
+    loop(1)                              # one step from the known input, for the parity check
     out = np.empty((B, lc.HID), np.float32)
     exe.downloadFromBuffer(L.out, out)
 
@@ -258,7 +263,8 @@ def bench_layer(args) -> int:
         "config": {
             "workload": f"decoder layer, TinyLlama-1.1B shape (hidden {lc.HID}, {lc.H}q/{lc.HKV}kv heads, "
                         f"head_dim {lc.D}, ffn {lc.FFN}), batch {B}, contexts of {c.name} "
-                        f"(sum {int(c.seq_lens.sum())}), 11 operators per step, {n_layers} K/V pools rotated",
+                        f"(sum {int(c.seq_lens.sum())}), 11 operators per step, each step's output is the next "
+                        f"step's input, {n_layers} K/V pools rotated",
             "weight_bytes_per_step": w_bytes, "kv_bytes_per_step": c.kv_bytes,
             "us_per_layer": round(us, 2),
             "tokens_per_s_at_22_layers": round(B / (22 * us * 1e-6), 1),

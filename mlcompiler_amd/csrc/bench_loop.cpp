@@ -137,6 +137,8 @@ struct MlcBenchLayer {
     const void* x;            // [batch][hidden] fp32 input of the layer
     void* norm; void* qkv; void* q; void* attn; void* o; void* resid; void* gate_up;
     void* gate; void* up; void* mix; void* down; void* out;
+    void* out2;               // when set: step i reads step i-1's output (out, out2 alternate), like
+                              // consecutive layers of a model; otherwise every step reads x
     const void* cos; const void* sin;
     const float* attn_norm_w; const float* ffn_norm_w;
     const void* w_qkv; size_t w_qkv_bytes;
@@ -160,7 +162,9 @@ int mlc_bench_layer_loop(const MlcBenchLayer* L, void* const* k_pools, void* con
     if (!mlc_hip_timer_start()) return 0;
     for (size_t i = 0; i < steps; ++i) {
         const size_t l = i % n_layers;
-        int ok = mlc_hip_rms_norm_batched(L->x, L->attn_norm_w, HID, 1e-5f, B, HID, L->norm, 0);
+        const void* x = (L->out2 && i > 0) ? ((i - 1) % 2 ? L->out2 : L->out) : L->x;
+        void* out = (L->out2 && i % 2) ? L->out2 : L->out;
+        int ok = mlc_hip_rms_norm_batched(x, L->attn_norm_w, HID, 1e-5f, B, HID, L->norm, 0);
         ok = ok && mlc_hip_matmul_q4_0_batched("bench.attn_qkv", L->w_qkv, L->w_qkv_bytes, L->norm, B,
                                                qkv_rows, HID, s_hid, 1, L->qkv, 0);
         ok = ok && mlc_hip_qkv_split_rope_scatter(L->qkv, L->q, k_pools[l], v_pools[l], nullptr, nullptr,
@@ -174,14 +178,14 @@ int mlc_bench_layer_loop(const MlcBenchLayer* L, void* const* k_pools, void* con
                                              L->page_size_tokens, 1, 0);
         ok = ok && mlc_hip_matmul_q4_0_batched("bench.attn_output", L->w_o, L->w_o_bytes, L->attn, B, HID,
                                                HID, s_hid, 1, L->o, 0);
-        ok = ok && mlc_hip_add_batched(L->x, L->o, L->resid, B * HID, 0);
+        ok = ok && mlc_hip_add_batched(x, L->o, L->resid, B * HID, 0);
         ok = ok && mlc_hip_rms_norm_batched(L->resid, L->ffn_norm_w, HID, 1e-5f, B, HID, L->norm, 0);
         ok = ok && mlc_hip_matmul_q4_0_batched("bench.ffn_gate_up", L->w_gate_up, L->w_gate_up_bytes,
                                                L->norm, B, 2 * FFN, HID, s_hid, 1, L->gate_up, 0);
         ok = ok && mlc_hip_gate_up_split_silu_mul(L->gate_up, L->gate, L->up, L->mix, B, FFN, 2 * FFN, 0);
         ok = ok && mlc_hip_matmul_q4_0_batched("bench.ffn_down", L->w_down, L->w_down_bytes, L->mix, B,
                                                HID, FFN, s_ffn, 1, L->down, 0);
-        ok = ok && mlc_hip_add_batched(L->resid, L->down, L->out, B * HID, 0);
+        ok = ok && mlc_hip_add_batched(L->resid, L->down, out, B * HID, 0);
         if (!ok) return 0;
     }
     const float ms = mlc_hip_timer_stop();

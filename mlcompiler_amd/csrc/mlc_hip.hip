@@ -1146,6 +1146,19 @@ int mlc_hip_gate_up_split_silu_mul(const void* gate_up, void* gate, void* up, vo
             return finish(sync);
         }
         if (!settle()) return 0;
+        // nothing to join: the operator starts a chain of its own, so that the split of the
+        // down-projection's input can join it
+        if (g.opt_fuse_rows && ffn_gate_up_rows == 2 * ffn_inner && row_len_ok(ffn_inner) && aligned16(gate_up) &&
+            aligned16(gate) && aligned16(up) && aligned16(out)) {
+            rows_begin(gate_up, batch, ffn_gate_up_rows);
+            r.p.silu = 1;
+            r.p.gate_out = static_cast<float*>(gate);
+            r.p.up_out = static_cast<float*>(up);
+            r.p.silu_out = static_cast<float*>(out);
+            r.len = ffn_inner;
+            r.cur = out;
+            return finish(sync);
+        }
     }
     const size_t n = batch * ffn_inner;
     hipLaunchKernelGGL(gate_up_split_silu_mul_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,

