@@ -112,3 +112,112 @@ def test_walker_ops_argument_errors(exe):
         assert not exe.encodeGateUpSplitSiluMul(buf, buf, buf, buf, 2, 8, 12, sync=True)  # 2*inner > rows
     finally:
         exe.releaseScratchBuffer(buf)
+
+
+# ---- operators encoded back to back in one pass run as one fused launch: same results ---------
+
+def _chain_case(rng, batch, hid, ffn):
+    x = rng.standard_normal((batch, hid)).astype(np.float32)
+    y = rng.standard_normal((batch, hid)).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, hid).astype(np.float32)
+    gu = rng.standard_normal((batch, 2 * ffn)).astype(np.float32)
+    return x, y, w, gu
+
+
+@pytest.mark.parametrize("batch,hid,ffn", [(5, 2048, 5632), (33, 256, 64), (64, 4096, 1024), (2, 16384, 8)])
+@pytest.mark.parametrize("fuse", [1, 0])
+def test_add_then_rms_norm_in_one_pass(exe, batch, hid, ffn, fuse):
+    """add -> RMSNorm (the residual add of one layer and the norm of the next), then a second,
+    unrelated add: with fusion on, the first two are one launch; all three outputs are written."""
+    print(f"[chain add+rms] batch={batch} hid={hid} fuse={fuse}", flush=True)
+    rng = np.random.default_rng(batch + hid)
+    x, y, w, _ = _chain_case(rng, batch, hid, ffn)
+    r1 = po.add(x, y)
+    want_n = po.rms_norm_batched(r1, w, 1e-5, batch, hid)
+    bufs = [_up(exe, x), _up(exe, y)] + [exe.allocateScratchBuffer(x.nbytes) for _ in range(3)]
+    d_x, d_y, d_r1, d_n, d_z = bufs
+    assert exe.setOption("fuse_row_ops", fuse)
+    before = exe.rowProgramLaunches()
+    try:
+        assert exe.beginForwardPassCB()
+        assert exe.encodeAddBatched(d_x, d_y, d_r1, batch * hid)
+        assert exe.encodeRmsNormBatched(d_r1, w, 1e-5, batch, hid, d_n)
+        assert exe.encodeAddBatched(d_n, d_x, d_z, batch * hid)      # reads the chain's result
+        assert exe.flushForwardPassCB(), exe.lastError()
+        got_r1, got_n, got_z = (_down(exe, b, x.shape) for b in (d_r1, d_n, d_z))
+    finally:
+        exe.setOption("fuse_row_ops", 1)
+        for b in bufs:
+            exe.releaseScratchBuffer(b)
+    assert np.array_equal(got_r1, r1)
+    assert np.max(np.abs(got_n - want_n) / (np.abs(want_n) + 1e-6)) < 5e-6
+    assert np.array_equal(got_z, got_n + x)
+    launches = exe.rowProgramLaunches() - before
+    assert launches == (1 if fuse else 0), launches
+
+
+@pytest.mark.parametrize("fuse", [1, 0])
+def test_in_place_add_and_download_without_flush(exe, fuse):
+    """out == a (the residual stream updated in place), and the result read back while the pass
+    is still open: the download has to see the pending operators' results."""
+    rng = np.random.default_rng(3)
+    a = rng.standard_normal((7, 512)).astype(np.float32)
+    b = rng.standard_normal((7, 512)).astype(np.float32)
+    d_a, d_b = _up(exe, a), _up(exe, b)
+    assert exe.setOption("fuse_row_ops", fuse)
+    try:
+        assert exe.beginForwardPassCB()
+        assert exe.encodeAddBatched(d_a, d_b, d_a, a.size)
+        got = _down(exe, d_a, a.shape)            # no flush before
+        assert exe.encodeAddBatched(d_a, d_b, d_a, a.size)
+        assert exe.flushForwardPassCB()
+        got2 = _down(exe, d_a, a.shape)
+    finally:
+        exe.setOption("fuse_row_ops", 1)
+        exe.releaseScratchBuffer(d_a)
+        exe.releaseScratchBuffer(d_b)
+    assert np.array_equal(got, a + b)
+    assert np.array_equal(got2, (a + b) + b)
+
+
+@pytest.mark.parametrize("batch,hid,ffn,rows", [(6, 2048, 5632, 2048), (33, 256, 64, 192), (64, 1024, 512, 64)])
+@pytest.mark.parametrize("fuse", [1, 0])
+def test_gate_up_then_matmul_then_add_in_one_pass(exe, batch, hid, ffn, rows, fuse):
+    """gate/up split + SiLU -> Q4_0 down-projection -> residual add: the fp16 split of the
+    matmul's input joins the SiLU launch and (when the matmul splits K) the sum of its slices
+    joins the add.  Every buffer the three operators are specified to write is checked."""
+    print(f"[chain silu+matmul+add] batch={batch} ffn={ffn} rows={rows} fuse={fuse}", flush=True)
+    rng = np.random.default_rng(batch * 7 + ffn)
+    _, _, _, gu = _chain_case(rng, batch, hid, ffn)
+    resid = rng.standard_normal((batch, rows)).astype(np.float32)
+    wq = po.quantize_q4_0((rng.standard_normal((rows, ffn)) * 0.05).astype(np.float32))
+    want_gate, want_up, want_mix = po.gate_up_split_silu_mul(gu, batch, ffn, 2 * ffn)
+    want_down = po.matmul_q4_0_batched(wq, want_mix, batch, rows, ffn)
+    want_out = po.add(resid, want_down)
+    d_gu, d_res = _up(exe, gu), _up(exe, resid)
+    d_gate, d_upb, d_mix = (exe.allocateScratchBuffer(batch * ffn * 4) for _ in range(3))
+    d_down, d_out = (exe.allocateScratchBuffer(batch * rows * 4) for _ in range(2))
+    bufs = [d_gu, d_res, d_gate, d_upb, d_mix, d_down, d_out]
+    assert exe.setOption("fuse_row_ops", fuse)
+    try:
+        for ks in (0, 2):   # automatic, and a forced K split (the sum of the slices joins the add)
+            assert exe.setOption("q4_ksplit", ks)
+            assert exe.beginForwardPassCB()
+            assert exe.encodeGateUpSplitSiluMul(d_gu, d_gate, d_upb, d_mix, batch, ffn, 2 * ffn)
+            assert exe.encodeMatMulQ4_0Batched(f"chain.down.{rows}x{ffn}", wq, d_mix, batch, rows, ffn,
+                                               wq.shape[1], 1, d_down), exe.lastError()
+            assert exe.encodeAddBatched(d_res, d_down, d_out, batch * rows)
+            assert exe.flushForwardPassCB(), exe.lastError()
+            got_gate, got_up, got_mix = (_down(exe, b, (batch, ffn)) for b in (d_gate, d_upb, d_mix))
+            got_down, got_out = (_down(exe, b, (batch, rows)) for b in (d_down, d_out))
+            assert np.array_equal(got_gate, want_gate) and np.array_equal(got_up, want_up)
+            assert np.max(np.abs(got_mix - want_mix) / (np.abs(want_mix) + 1e-6)) < 5e-6
+            scale = float(np.max(np.abs(want_down)))
+            assert np.max(np.abs(got_down - want_down)) < 2e-5 * scale
+            assert np.array_equal(got_out, resid + got_down)
+            assert np.max(np.abs(got_out - want_out)) < 2e-5 * max(scale, 1.0)
+    finally:
+        exe.setOption("fuse_row_ops", 1)
+        exe.setOption("q4_ksplit", 0)
+        for b in bufs:
+            exe.releaseScratchBuffer(b)
