@@ -211,6 +211,23 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
                                 const void* in, size_t batch, size_t rows, size_t cols,
                                 size_t row_stride, uint32_t quant_version, void* out, int sync);
 
+/* MetalExecutor::encodeMatMulQ6KBatched (metal_runtime.hpp:491-498,
+ * metal_runtime.mm:6973-7012; kernel q6_k_matmul_v3_batched :1581-1655), the
+ * lm_head of the batched decode step (batched_walker.cpp:429-431), and with
+ * sync = 1 MetalExecutor::runMatMulQ6KBatched (metal_runtime.hpp:452-459):
+ * out[b][r] = sum_c W[r][c] * in[b][c]; W is `rows` Q6_K rows of `cols`
+ * weights, row_stride bytes apart (210-byte blocks of 256: 128 bytes of low
+ * nibbles, 64 bytes of high bit pairs, 16 int8 scales, fp16 d;
+ * compiler/runtime/quantization.cpp:142-147, 1469-1499).  `weights` is the
+ * HOST copy, uploaded the first time a weight_name is seen and kept on the
+ * device; in/out are device fp32 [batch][cols] / [batch][rows].  Same
+ * constraints as the reference (cols >= 64, rows % 4 == 0).  Shapes with
+ * rows % 32 == 0 and cols % 256 == 0 run on the matrix cores with fp32-grade
+ * accuracy, others on a scalar kernel. */
+int mlc_hip_matmul_q6_k_batched(const char* weight_name, const void* weights, size_t weight_bytes,
+                                const void* in, size_t batch, size_t rows, size_t cols,
+                                size_t row_stride, void* out, int sync);
+
 /* Chunked prefill over paged KV (MFMA path).  No counterpart in the reference,
  * which prefills by looping the decode path once per prompt token
  * (compiler/runtime/batched_executor.cpp:454-466); semantics are the decode

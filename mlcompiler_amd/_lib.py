@@ -42,6 +42,7 @@ SIGNATURES = {
     "mlc_hip_gate_up_split_silu_mul": (C.c_int, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, C.c_int]),
     "mlc_hip_matmul_q4_0_batched": (C.c_int, [C.c_char_p, _vp, _sz, _vp, _sz, _sz, _sz, _sz, C.c_uint32, _vp,
                                               C.c_int]),
+    "mlc_hip_matmul_q6_k_batched": (C.c_int, [C.c_char_p, _vp, _sz, _vp, _sz, _sz, _sz, _sz, _vp, C.c_int]),
     "mlc_hip_paged_attn_prefill": (C.c_int, [_vp, _vp, _vp, _vp, _u32p, _sz, _u32p, _u32p, _u32p,
                                              _sz, _sz, _sz, _sz, _sz, _sz, C.c_int]),
     "mlc_hip_stream": (_vp, []),

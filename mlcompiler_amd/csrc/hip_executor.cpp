@@ -169,6 +169,22 @@ bool HipExecutor::encodeMatMulQ4_0Batched(const std::string& weight_name,
                                        /*sync=*/0) != 0;
 }
 
+bool HipExecutor::encodeMatMulQ6KBatched(const std::string& weight_name,
+                                         const std::vector<uint8_t>& weights, void* in_buf,
+                                         size_t batch, size_t rows, size_t cols, size_t row_stride,
+                                         void* out_buf) const {
+    return mlc_hip_matmul_q6_k_batched(weight_name.c_str(), weights.data(), weights.size(), in_buf,
+                                       batch, rows, cols, row_stride, out_buf, /*sync=*/0) != 0;
+}
+
+bool HipExecutor::runMatMulQ6KBatched(const std::string& weight_name,
+                                      const std::vector<uint8_t>& weights, void* in_buf, size_t batch,
+                                      size_t rows, size_t cols, size_t row_stride,
+                                      void* out_buf) const {
+    return mlc_hip_matmul_q6_k_batched(weight_name.c_str(), weights.data(), weights.size(), in_buf,
+                                       batch, rows, cols, row_stride, out_buf, /*sync=*/1) != 0;
+}
+
 bool HipExecutor::runPagedPrefillAttention(void* q_f16_buffer, void* k_pages_buffer,
                                            void* v_pages_buffer, void* o_buffer,
                                            const std::vector<uint32_t>& page_tables_flat,

@@ -104,6 +104,14 @@ public:
                                  void* in_buf, size_t batch, size_t rows, size_t cols,
                                  size_t row_stride, uint32_t quant_version, void* out_buf) const;
 
+    // metal_runtime.hpp:491-498 (lm_head of the batched step) and :452-459 (the waiting form)
+    bool encodeMatMulQ6KBatched(const std::string& weight_name, const std::vector<uint8_t>& weights,
+                                void* in_buf, size_t batch, size_t rows, size_t cols,
+                                size_t row_stride, void* out_buf) const;
+    bool runMatMulQ6KBatched(const std::string& weight_name, const std::vector<uint8_t>& weights,
+                             void* in_buf, size_t batch, size_t rows, size_t cols,
+                             size_t row_stride, void* out_buf) const;
+
     // Chunked prefill over paged KV: no reference method (the reference loops its
     // decode path per prompt token, batched_executor.cpp:454-466).
     bool runPagedPrefillAttention(void* q_f16_buffer, void* k_pages_buffer, void* v_pages_buffer,

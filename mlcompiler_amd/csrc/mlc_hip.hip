@@ -25,6 +25,7 @@
 #include "paged_rope_kernels.h"
 #include "walker_kernels.h"
 #include "q4_matmul_kernels.h"
+#include "q6k_matmul_kernels.h"
 
 namespace mlc_hip {
 // Defined in paged_decode_inst.hip, one object per (head_dim, heads-per-wave).
@@ -96,6 +97,14 @@ struct Ctx {
         void* d = nullptr;
     };
     std::unordered_map<std::string, Q4Weight> q4_weights;
+    struct Q6KWeight {
+        size_t bytes = 0, rows = 0, cols = 0, stride = 0;
+        void* raw = nullptr;
+        void* qa = nullptr;
+        void* sc = nullptr;
+        void* d = nullptr;
+    };
+    std::unordered_map<std::string, Q6KWeight> q6k_weights;
     long opt_q4_force_generic = 0;
     long opt_q4_ksplit = 0;  // 0 = automatic
     MetaSlot ring[8];
@@ -1311,6 +1320,134 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
                                    (uint32_t)ksplit);
             }
         }
+    }
+    return finish(sync);
+}
+
+// ---- batched Q6_K matmul -------------------------------------------------------------------
+
+namespace {
+
+bool q6k_fast_shape(size_t rows, size_t cols, size_t row_stride) {
+    return rows % 32 == 0 && cols % 256 == 0 && row_stride >= cols / 256 * 210;
+}
+
+// Uploads the weight matrix on first use of its name (or when its size changed); shapes the
+// matrix-core kernel takes are also repacked (layout: q6k_matmul_kernels.h).
+Ctx::Q6KWeight* q6k_weight(const char* name, const uint8_t* host, size_t bytes, size_t rows, size_t cols,
+                           size_t stride) {
+    Ctx::Q6KWeight& w = g.q6k_weights[name];
+    if (w.raw && w.bytes == bytes && w.rows == rows && w.cols == cols && w.stride == stride) return &w;
+    (void)hipStreamSynchronize(g.stream);
+    for (void** p : {&w.raw, &w.qa, &w.sc, &w.d})
+        if (*p) { (void)hipFree(*p); *p = nullptr; }
+    w = Ctx::Q6KWeight{};
+    void* raw = nullptr;
+    if (hipMalloc(&raw, bytes) != hipSuccess) { (void)hipGetLastError(); fail("q6_k matmul: hipMalloc failed"); return nullptr; }
+    if (hipMemcpy(raw, host, bytes, hipMemcpyHostToDevice) != hipSuccess) { (void)hipFree(raw); fail("q6_k matmul: upload failed"); return nullptr; }
+    w.raw = raw; w.bytes = bytes; w.rows = rows; w.cols = cols; w.stride = stride;
+    if (q6k_fast_shape(rows, cols, stride)) {
+        const size_t nb = cols / 256, tiles = rows / 32, groups = nb * 4;
+        std::vector<uint8_t> qa(tiles * groups * 3 * 64 * 8);
+        std::vector<uint8_t> sc(tiles * groups * 32 * 4);
+        std::vector<uint16_t> d(tiles * nb * 32);
+        for (size_t t = 0; t < tiles; ++t)
+            for (size_t m = 0; m < 32; ++m) {
+                const uint8_t* row = host + (t * 32 + m) * stride;
+                for (size_t b = 0; b < nb; ++b) {
+                    const uint8_t* blk = row + b * 210;
+                    std::memcpy(&d[(t * nb + b) * 32 + m], blk + 208, 2);
+                    for (size_t hi = 0; hi < 2; ++hi)
+                        for (size_t l0i = 0; l0i < 2; ++l0i) {
+                            const size_t gi = b * 4 + hi * 2 + l0i, tg = t * groups + gi;
+                            for (size_t h = 0; h < 2; ++h) {
+                                const size_t lane = h * 32 + m, l = l0i * 16 + h * 8;
+                                std::memcpy(&qa[((tg * 3 + 0) * 64 + lane) * 8], blk + hi * 64 + l, 8);
+                                std::memcpy(&qa[((tg * 3 + 1) * 64 + lane) * 8], blk + hi * 64 + 32 + l, 8);
+                                std::memcpy(&qa[((tg * 3 + 2) * 64 + lane) * 8], blk + 128 + hi * 32 + l, 8);
+                            }
+                            for (size_t q = 0; q < 4; ++q) sc[(tg * 32 + m) * 4 + q] = blk[192 + hi * 8 + q * 2 + l0i];
+                        }
+                }
+            }
+        if (hipMalloc(&w.qa, qa.size()) != hipSuccess || hipMalloc(&w.sc, sc.size()) != hipSuccess ||
+            hipMalloc(&w.d, d.size() * 2) != hipSuccess ||
+            hipMemcpy(w.qa, qa.data(), qa.size(), hipMemcpyHostToDevice) != hipSuccess ||
+            hipMemcpy(w.sc, sc.data(), sc.size(), hipMemcpyHostToDevice) != hipSuccess ||
+            hipMemcpy(w.d, d.data(), d.size() * 2, hipMemcpyHostToDevice) != hipSuccess) {
+            (void)hipGetLastError();
+            fail("q6_k matmul: repacked upload failed");
+            return nullptr;
+        }
+    }
+    return &w;
+}
+
+}  // namespace
+
+int mlc_hip_matmul_q6_k_batched(const char* weight_name, const void* weights, size_t weight_bytes,
+                                const void* in, size_t batch, size_t rows, size_t cols,
+                                size_t row_stride, void* out, int sync) {
+    if (!init_once()) return fail("GPU unavailable");
+    if (!sync && !g.pass_open) return fail("encode: no open forward pass");
+    if (!in || !out || batch == 0 || rows == 0 || cols == 0) return fail("q6_k matmul: null buffer or zero size");  // :6983
+    if (cols < 64 || (rows % 4u) != 0) return fail("q6_k matmul: needs cols >= 64 and rows % 4 == 0");          // :6985
+    if (!weight_name || !weights) return fail("q6_k matmul: null weights");
+    const size_t nb = (cols + 255) / 256;
+    if (row_stride < nb * 210 || weight_bytes < (rows - 1) * row_stride + nb * 210)
+        return fail("q6_k matmul: weight bytes do not cover rows x row_stride");
+    if (batch * rows > 0x7FFFFFFFull || batch * cols > 0x7FFFFFFFull) return fail("q6_k matmul: too many elements");
+    const size_t ki = known_bytes(in), ko = known_bytes(out);
+    if ((ki && batch * cols * 4 > ki) || (ko && batch * rows * 4 > ko)) return fail("q6_k matmul: buffer too small");
+    const bool fast = q6k_fast_shape(rows, cols, row_stride) && !g.opt_q4_force_generic;
+    const bool feeds = fast && batch <= 64 && rows_continue(in, batch, cols);
+    if (!feeds && !settle()) return 0;
+    Ctx::Q6KWeight* w = q6k_weight(weight_name, static_cast<const uint8_t*>(weights), weight_bytes, rows, cols, row_stride);
+    if (!w) return 0;
+
+    if (!fast || !w->qa) {
+        if (!settle()) return 0;
+        const size_t waves = batch * rows;
+        hipLaunchKernelGGL(q6_k_matmul_generic_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, g.stream,
+                           static_cast<const uint8_t*>(w->raw), static_cast<const float*>(in),
+                           static_cast<float*>(out), (uint32_t)batch, (uint32_t)rows, (uint32_t)cols,
+                           (uint32_t)row_stride);
+        return finish(sync);
+    }
+
+    // matrix cores, at most 64 requests per pass; two row tiles per workgroup when one would give
+    // more workgroups than CUs (and the batch fits one batch tile)
+    const size_t tiles = rows / 32;
+    for (size_t bo = 0; bo < batch; bo += 64) {
+        const size_t bn = std::min<size_t>(64, batch - bo);
+        const size_t bpad = (bn + 31) / 32 * 32;
+        _Float16* frag = static_cast<_Float16*>(cached_buffer("q4_x_fragments", bpad * cols * 4));
+        float* inv = static_cast<float*>(cached_buffer("q4_x_inv_scale", 64 * 4));
+        if (!frag || !inv) return fail("q6_k matmul: scratch allocation failed");
+        const float* xin = static_cast<const float*>(in) + bo * cols;
+        if (feeds) {
+            g.rows.p.frag = frag;
+            g.rows.p.inv_scale = inv;
+            g.rows.grid_rows = bpad;
+            if (!settle()) return 0;
+        } else {
+            hipLaunchKernelGGL(q4_split_activations_kernel, dim3((unsigned)bpad), dim3(256), 0, g.stream, xin, frag,
+                               inv, (uint32_t)bn, (uint32_t)cols);
+        }
+        Q6KArgs a;
+        a.qa = static_cast<const uint2*>(w->qa);
+        a.sc = static_cast<const uint32_t*>(w->sc);
+        a.d = static_cast<const _Float16*>(w->d);
+        a.xfrag = frag;
+        a.inv_scale = inv;
+        a.out = static_cast<float*>(out) + bo * rows;
+        a.batch = (uint32_t)bn; a.rows = (uint32_t)rows; a.nblocks = (uint32_t)(cols / 256);
+        if (bpad == 32 && tiles > 256 && tiles % 2 == 0)
+            hipLaunchKernelGGL((q6_k_matmul_mfma_kernel<1, 2>), dim3((unsigned)(tiles / 2)), dim3(512), 0, g.stream, a);
+        else if (bpad == 32)
+            hipLaunchKernelGGL((q6_k_matmul_mfma_kernel<1, 1>), dim3((unsigned)tiles), dim3(512), 0, g.stream, a);
+        else
+            hipLaunchKernelGGL((q6_k_matmul_mfma_kernel<2, 1>), dim3((unsigned)tiles), dim3(512), 0, g.stream, a);
     }
     return finish(sync);
 }

@@ -213,6 +213,15 @@ class HipExecutor:
             quant_version, out_buf, int(bool(sync))))
 
     # -- chunked prefill (no reference method; see include/mlc_hip.h)
+
+    def encodeMatMulQ6KBatched(self, weight_name, weights, in_buf, batch, rows, cols, row_stride,
+                               out_buf, sync: bool = False) -> bool:
+        """metal_runtime.hpp:491-498 (sync=True: runMatMulQ6KBatched, :452-459); `weights` is the
+        host byte array of the Q6_K rows."""
+        w = np.ascontiguousarray(weights, np.uint8)
+        return bool(self._lib.mlc_hip_matmul_q6_k_batched(
+            weight_name.encode(), w.ctypes.data, w.size, in_buf, batch, rows, cols, row_stride,
+            out_buf, int(bool(sync))))
     def runPagedPrefillAttention(self, q_f16_buffer, k_pages_buffer, v_pages_buffer, o_buffer,
                                  page_tables_flat, page_table_offsets, seq_lens, q_start, batch,
                                  chunk, num_heads, kv_heads, head_dim, page_size_tokens,

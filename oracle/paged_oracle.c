@@ -358,6 +358,130 @@ void oracle_quantize_row_q4_0(const float* src, size_t cols, uint8_t* dst) {
     }
 }
 
+/* ---- Q6_K (compiler/runtime/quantization.cpp:142-147: 256 weights per 210-byte block =
+ * 128 bytes of low nibbles, 64 bytes of high bit pairs, 16 int8 group scales, fp16 d) */
+
+/* dequantizeRowQ6_K, quantization.cpp:1469-1499, one block */
+static void q6k_block_values(const uint8_t* block, float* y) {
+    const uint8_t* ql = block;
+    const uint8_t* qh = block + 128;
+    const int8_t* sc = (const int8_t*)(block + 192);
+    uint16_t dh;
+    memcpy(&dh, block + 208, 2);
+    const float d = oracle_fp16_to_float(dh);
+    for (size_t n = 0; n < 256; n += 128) {
+        for (int l = 0; l < 32; ++l) {
+            const int is = l / 16;
+            const int8_t q1 = (int8_t)((int8_t)((ql[l + 0] & 0xF) | (((qh[l] >> 0) & 3) << 4)) - 32);
+            const int8_t q2 = (int8_t)((int8_t)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32);
+            const int8_t q3 = (int8_t)((int8_t)((ql[l + 0] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32);
+            const int8_t q4 = (int8_t)((int8_t)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32);
+            y[l + 0] = d * (float)sc[is + 0] * (float)q1;
+            y[l + 32] = d * (float)sc[is + 2] * (float)q2;
+            y[l + 64] = d * (float)sc[is + 4] * (float)q3;
+            y[l + 96] = d * (float)sc[is + 6] * (float)q4;
+        }
+        y += 128;
+        ql += 64;
+        qh += 32;
+        sc += 8;
+    }
+}
+
+void oracle_dequantize_row_q6_k(const uint8_t* src, size_t cols, float* dst) {
+    const size_t nb = (cols + 255) / 256;
+    for (size_t b = 0; b < nb; ++b) {
+        float buf[256];
+        q6k_block_values(src + b * 210, buf);
+        const size_t n = cols - b * 256 < 256 ? cols - b * 256 : 256;
+        memcpy(dst + b * 256, buf, n * sizeof(float));
+    }
+}
+
+int oracle_matmul_q6_k_batched(const uint8_t* weights, const float* in, size_t batch, size_t rows,
+                               size_t cols, size_t row_stride, float* out, int n_threads) {
+    if (!weights || !in || !out || batch == 0 || rows == 0 || cols == 0) return 0;
+    if (cols < 64 || (rows % 4u) != 0) return 0; /* metal_runtime.mm:6985 */
+    const size_t nb = (cols + 255) / 256;
+    if (row_stride < nb * 210) return 0;
+    if (n_threads < 1) n_threads = 1;
+#pragma omp parallel for num_threads(n_threads) schedule(static)
+    for (long long r = 0; r < (long long)rows; ++r) {
+        const uint8_t* row = weights + (size_t)r * row_stride;
+        float* tmp = (float*)malloc(nb * 256 * sizeof(float));
+        for (size_t b = 0; b < nb; ++b) q6k_block_values(row + b * 210, tmp + b * 256);
+        for (size_t b = 0; b < batch; ++b) {
+            const float* vec = in + b * cols;
+            float acc = 0.0f; /* dotProductRowQ6_K, quantization.cpp:1570-1586 */
+            for (size_t i = 0; i < cols; ++i) acc += tmp[i] * vec[i];
+            out[b * rows + (size_t)r] = acc;
+        }
+        free(tmp);
+    }
+    return 1;
+}
+
+static int q6k_clamp(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+/* quantizeRowQ6_K, quantization.cpp:1588-1663 */
+void oracle_quantize_row_q6_k(const float* src, size_t cols, uint8_t* dst) {
+    const size_t blocks = (cols + 255) / 256;
+    size_t offset = 0;
+    for (size_t b = 0; b < blocks; ++b) {
+        const size_t be = cols - offset < 256 ? cols - offset : 256;
+        float data[256] = {0};
+        memcpy(data, src + offset, be * sizeof(float));
+        float chunk_scale[16];
+        float max_scale = 0.0f;
+        for (size_t j = 0; j < 16; ++j) {
+            const size_t start = j * 16;
+            if (start >= be) {
+                chunk_scale[j] = 0.0f;
+                continue;
+            }
+            float max_abs = 0.0f;
+            for (size_t i = start; i < start + 16 && i < be; ++i) max_abs = fmaxf(max_abs, fabsf(data[i]));
+            float scale = max_abs / 32.0f;
+            if (scale < 1e-8f) scale = 0.0f;
+            chunk_scale[j] = scale;
+            max_scale = fmaxf(max_scale, scale);
+        }
+        const float base = max_scale > 0.0f ? max_scale / 127.0f : 0.0f;
+        uint8_t* out = dst + b * 210;
+        const uint16_t dh = oracle_float_to_fp16_ref(base);
+        memcpy(out + 208, &dh, 2);
+        uint8_t enc[256];
+        for (size_t j = 0; j < 16; ++j) {
+            int8_t sc = 0;
+            if (base > 0.0f && chunk_scale[j] > 0.0f)
+                sc = (int8_t)q6k_clamp((int)roundf(chunk_scale[j] / base), -127, 127);
+            out[192 + j] = (uint8_t)sc;
+            const float actual = base * (float)sc;
+            for (size_t i = 0; i < 16; ++i) {
+                const size_t idx = j * 16 + i;
+                const float value = idx < be ? data[idx] : 0.0f;
+                const float qf = actual != 0.0f ? roundf(value / actual) : 0.0f;
+                enc[idx] = (uint8_t)(q6k_clamp((int)qf, -32, 31) + 32);
+            }
+        }
+        memset(out, 0, 192);
+        uint8_t* ql = out;
+        uint8_t* qh = out + 128;
+        for (size_t n = 0; n < 256; n += 128) {
+            for (size_t l = 0; l < 32; ++l) {
+                const uint8_t q1 = enc[n + l], q2 = enc[n + l + 32], q3 = enc[n + l + 64], q4 = enc[n + l + 96];
+                ql[l + 0] = (uint8_t)((q1 & 0xF) | ((q3 & 0xF) << 4));
+                ql[l + 32] = (uint8_t)((q2 & 0xF) | ((q4 & 0xF) << 4));
+                qh[l] = (uint8_t)(((q1 >> 4) & 3) | (((q2 >> 4) & 3) << 2) | (((q3 >> 4) & 3) << 4) |
+                                  (((q4 >> 4) & 3) << 6));
+            }
+            ql += 64;
+            qh += 32;
+        }
+        offset += be;
+    }
+}
+
 /* ------------------------------------------------------------- attention */
 
 static int attention_args_ok(const void* q, const void* k, const void* v, const void* o,

@@ -156,6 +156,21 @@ int oracle_matmul_q4_0_batched(const uint8_t* weights, const float* in, size_t b
  * reference's floatToFp16.  dst must hold ceil(cols/32)*18 bytes. */
 void oracle_quantize_row_q4_0(const float* src, size_t cols, uint8_t* dst);
 
+/* Q6_K rows: 210-byte blocks of 256 weights (128 bytes of low nibbles, 64 bytes of high bit
+ * pairs, 16 int8 scales of 16 weights each, fp16 d; value d * scale * (q - 32)),
+ * compiler/runtime/quantization.cpp:142-147.
+ * oracle_dequantize_row_q6_k = dequantizeRowQ6_K (quantization.cpp:1469-1499);
+ * oracle_matmul_q6_k_batched: out[b][r] = the CPU dotProductRowQ6_K (quantization.cpp:1570-1586,
+ * the row dequantized block by block, then summed left to right in fp32) of weight row r with
+ * input row b; result layout and constraints of q6_k_matmul_v3_batched
+ * (compiler/runtime/metal_runtime.mm:1581-1655, host :6973-7012: cols >= 64, rows % 4 == 0);
+ * oracle_quantize_row_q6_k = quantizeRowQ6_K (quantization.cpp:1588-1663), used to make test
+ * weights.  All three are checked against the reference's own build of these functions. */
+void oracle_dequantize_row_q6_k(const uint8_t* src, size_t cols, float* dst);
+int oracle_matmul_q6_k_batched(const uint8_t* weights, const float* in, size_t batch, size_t rows,
+                               size_t cols, size_t row_stride, float* out, int n_threads);
+void oracle_quantize_row_q6_k(const float* src, size_t cols, uint8_t* dst);
+
 /* The executor-CPU attention, compiler/runtime/attention_cpu.cpp:437-470
  * (per head: left-to-right dot over every cached row :99-105, softmax that
  * subtracts the max, exponentiates and divides each weight by the sum :21-33,

@@ -76,6 +76,12 @@ def lib() -> C.CDLL:
         L.oracle_matmul_q4_0_batched.argtypes = [C.c_void_p, _f32p, _sz, _sz, _sz, _sz, _f32p, C.c_int]
         L.oracle_quantize_row_q4_0.restype = None
         L.oracle_quantize_row_q4_0.argtypes = [_f32p, _sz, C.c_void_p]
+        L.oracle_matmul_q6_k_batched.restype = C.c_int
+        L.oracle_matmul_q6_k_batched.argtypes = [C.c_void_p, _f32p, _sz, _sz, _sz, _sz, _f32p, C.c_int]
+        L.oracle_quantize_row_q6_k.restype = None
+        L.oracle_quantize_row_q6_k.argtypes = [_f32p, _sz, C.c_void_p]
+        L.oracle_dequantize_row_q6_k.restype = None
+        L.oracle_dequantize_row_q6_k.argtypes = [C.c_void_p, _sz, _f32p]
         L.oracle_gather_kv_pages.restype = C.c_int
         L.oracle_gather_kv_pages.argtypes = [C.c_void_p, _u32p, _sz, _sz, _sz, _sz, _sz,
                                              C.c_void_p, _sz]
@@ -280,6 +286,39 @@ def matmul_q4_0_batched(weights, x, batch, rows, cols, row_stride=None, n_thread
     return out if ok else None
 
 
+def q6_k_row_bytes(cols: int) -> int:
+    return (cols + 255) // 256 * 210
+
+
+def quantize_q6_k(w) -> np.ndarray:
+    """Rows of floats -> Q6_K rows (uint8 [rows][q6_k_row_bytes(cols)]), quantizeRowQ6_K."""
+    w = _c(w, np.float32)
+    rows, cols = w.shape
+    out = np.zeros((rows, q6_k_row_bytes(cols)), np.uint8)
+    L = lib()
+    for r in range(rows):
+        L.oracle_quantize_row_q6_k(_p(w[r], _f32p), cols, out[r].ctypes.data)
+    return out
+
+
+def dequantize_q6_k(weights, cols) -> np.ndarray:
+    wq = _c(weights, np.uint8)
+    out = np.zeros((wq.shape[0], cols), np.float32)
+    L = lib()
+    for r in range(wq.shape[0]):
+        L.oracle_dequantize_row_q6_k(wq[r].ctypes.data, cols, _p(out[r], _f32p))
+    return out
+
+
+def matmul_q6_k_batched(weights, x, batch, rows, cols, row_stride=None, n_threads=8):
+    wq = _c(weights, np.uint8)
+    x = _c(x, np.float32)
+    out = np.zeros((batch, rows), np.float32)
+    ok = lib().oracle_matmul_q6_k_batched(wq.ctypes.data, _p(x, _f32p), batch, rows, cols,
+                                          row_stride or q6_k_row_bytes(cols), _p(out, _f32p), n_threads)
+    return out if ok else None
+
+
 # ------------------------------------------------------------ attention
 
 def _attn_args(q, k_pages, v_pages, pt_flat, pt_off, seq_lens, q_pos, batch, num_heads, head_dim):
@@ -479,6 +518,12 @@ def ref_lib():
         R.ref_dot_q4_0.argtypes = [C.c_void_p, _sz, _f32p]
         R.ref_dequantize_row_q4_0.restype = None
         R.ref_dequantize_row_q4_0.argtypes = [C.c_void_p, _sz, _f32p]
+        R.ref_quantize_row_q6_k.restype = _sz
+        R.ref_quantize_row_q6_k.argtypes = [_f32p, _sz, C.c_void_p, _sz]
+        R.ref_dot_q6_k.restype = C.c_float
+        R.ref_dot_q6_k.argtypes = [C.c_void_p, _sz, _f32p]
+        R.ref_dequantize_row_q6_k.restype = None
+        R.ref_dequantize_row_q6_k.argtypes = [C.c_void_p, _sz, _f32p]
         R.ref_run_attention_cpu.restype = C.c_int
         R.ref_run_attention_cpu.argtypes = [_f32p, _u16p, _u16p, _sz, _sz, _sz, _sz, _sz, _f32p,
                                             _f32p, _f32p]

@@ -8,6 +8,7 @@
 //   mlc::runtime::applyRotaryEmbedding / computeRotaryCoefficients
 //                                         compiler/runtime/quantization.cpp:772-823
 //   mlc::runtime::quantizeRowQ4_0 / dotProductRowQ4_0 / dequantizeRowQ4_0
+//   mlc::runtime::quantizeRowQ6_K / dotProductRowQ6_K / dequantizeRowQ6_K
 //                                         compiler/runtime/quantization.cpp:235-311
 // the way the reference's own test does (tests/test_runtime.cpp:1659-1690):
 // an ExecutionGraph with one Attention node, state tensors {Hkv, ctx, D}
@@ -159,6 +160,20 @@ float ref_dot_q4_0(const uint8_t* row, size_t cols, const float* vec) {
 }
 void ref_dequantize_row_q4_0(const uint8_t* row, size_t cols, float* dst) {
     mlc::runtime::dequantizeRowQ4_0(row, cols, 1, dst);
+}
+
+// dequantizeRowQ6_K / dotProductRowQ6_K / quantizeRowQ6_K (compiler/runtime/quantization.cpp:1469-1663)
+void ref_dequantize_row_q6_k(const uint8_t* row, size_t cols, float* dst) {
+    mlc::runtime::dequantizeRowQ6_K(row, cols, dst);
+}
+float ref_dot_q6_k(const uint8_t* row, size_t cols, const float* vec) {
+    return mlc::runtime::dotProductRowQ6_K(row, cols, vec);
+}
+size_t ref_quantize_row_q6_k(const float* src, size_t cols, uint8_t* dst, size_t dst_cap) {
+    std::vector<uint8_t> out;
+    mlc::runtime::quantizeRowQ6_K(src, cols, out);
+    if (out.size() <= dst_cap) std::memcpy(dst, out.data(), out.size());
+    return out.size();
 }
 
 }  // extern "C"

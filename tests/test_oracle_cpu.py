@@ -622,3 +622,78 @@ def test_q4_0_bit_exact_with_reference_build():
             for r in range(4):
                 want = R.ref_dot_q4_0(q[r].ctypes.data, cols, x[b].ctypes.data_as(po._f32p))
                 assert np.float32(want).view(np.uint32) == got[b, r].view(np.uint32)
+
+
+def _q6k_block_by_hand(rng):
+    """One Q6_K block written field by field, with the weights it stands for computed from the
+    format's definition (quantization.cpp:142-147, 1469-1499): weight n of the block sits in
+    half n / 128, quarter (n % 128) / 32, position l = n % 32; its low nibble is in ql[half*64 +
+    (quarter & 1)*32 + l] (low nibble for quarters 0-1, high for 2-3), its two high bits in
+    qh[half*32 + l] at bit 2*quarter, its scale is scales[half*8 + quarter*2 + l/16]."""
+    q = rng.integers(0, 64, 256)
+    sc = rng.integers(-100, 101, 16).astype(np.int8)
+    d = np.float16(0.0123)
+    blk = np.zeros(210, np.uint8)
+    w = np.zeros(256, np.float64)
+    for n in range(256):
+        half, quarter, l = n // 128, (n % 128) // 32, n % 32
+        qi = half * 64 + (quarter & 1) * 32 + l
+        blk[qi] |= (q[n] & 0xF) << (4 if quarter >= 2 else 0)
+        blk[128 + half * 32 + l] |= (q[n] >> 4) << (2 * quarter)
+        w[n] = float(d) * float(sc[half * 8 + quarter * 2 + l // 16]) * (int(q[n]) - 32)
+    blk[192:208] = sc.view(np.uint8)
+    blk[208:210] = np.frombuffer(d.tobytes(), np.uint8)
+    return blk, w
+
+
+def test_q6_k_block_by_hand_and_constraints():
+    rng = np.random.default_rng(66)
+    blk, w = _q6k_block_by_hand(rng)
+    deq = po.dequantize_q6_k(blk[None, :], 256)[0]
+    assert np.allclose(deq, w, rtol=3e-7, atol=0)
+    rows = np.tile(blk, (4, 1))
+    x = rng.standard_normal((2, 256)).astype(np.float32)
+    got = po.matmul_q6_k_batched(rows, x, 2, 4, 256)
+    want = x.astype(np.float64) @ w
+    assert np.allclose(got, want[:, None], rtol=1e-5, atol=1e-5)
+    # constraints of the batched kernel (metal_runtime.mm:6985)
+    assert po.matmul_q6_k_batched(rows[:3], x, 2, 3, 256) is None
+    assert po.matmul_q6_k_batched(rows, x[:, :32], 2, 4, 32) is None
+
+
+def test_q6_k_quantize_round_trip_error_bound():
+    rng = np.random.default_rng(67)
+    w = (rng.standard_normal((4, 512)) * rng.uniform(0.1, 4, (4, 1))).astype(np.float32)
+    q = po.quantize_q6_k(w)
+    deq = po.dequantize_q6_k(q, 512)
+    # a group of 16 is quantised with step ~ max|group| / 32 (the scale code rounds it by up to
+    # half a unit of max_scale / 127, the fp16 d by 2^-11): error <= 0.5 steps + the clamp at 31
+    grp = np.abs(w).reshape(4, 32, 16).max(axis=2)
+    blockmax = grp.reshape(4, 2, 16).max(axis=2).repeat(16, axis=1)
+    step = grp / 32 + blockmax / 32 / 127
+    assert np.all(np.abs(deq - w).reshape(4, 32, 16) <= 1.6 * step[:, :, None] + 1e-6)
+
+
+@needs_ref
+def test_q6_k_bit_exact_with_reference_build():
+    """quantizeRowQ6_K / dequantizeRowQ6_K / dotProductRowQ6_K compiled from
+    compiler/runtime/quantization.cpp."""
+    R = po.ref_lib()
+    rng = np.random.default_rng(68)
+    for cols in (256, 320, 2048):     # 320: a partial last block
+        w = (rng.standard_normal((4, cols)) * rng.uniform(0.01, 3)).astype(np.float32)
+        q = po.quantize_q6_k(w)
+        deq = po.dequantize_q6_k(q, cols)
+        for r in range(4):
+            buf = np.zeros(q.shape[1], np.uint8)
+            n = R.ref_quantize_row_q6_k(w[r].ctypes.data_as(po._f32p), cols, buf.ctypes.data, buf.size)
+            assert n == q.shape[1] and np.array_equal(buf, q[r])
+            want = np.zeros(cols, np.float32)
+            R.ref_dequantize_row_q6_k(q[r].ctypes.data, cols, want.ctypes.data_as(po._f32p))
+            assert np.array_equal(want.view(np.uint32), deq[r].view(np.uint32))
+        x = rng.standard_normal((3, cols)).astype(np.float32)
+        got = po.matmul_q6_k_batched(q, x, 3, 4, cols)
+        for b in range(3):
+            for r in range(4):
+                want = R.ref_dot_q6_k(q[r].ctypes.data, cols, x[b].ctypes.data_as(po._f32p))
+                assert np.float32(want).view(np.uint32) == got[b, r].view(np.uint32)
