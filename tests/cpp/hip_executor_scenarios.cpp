@@ -1,7 +1,8 @@
 // The scenarios of the reference's tests/test_paged_flash.cpp:214-275, driven through the C++
 // HipExecutor (same method names and argument order as MetalExecutor), checked against the
 // CPU oracle with the benchmark's bar (cosine >= 0.9999, max-abs <= 2e-3 per head).
-// Also one decode step with KV write through encode* calls.  Exit code 0 = all passed.
+// Also one decode step with KV write through encode* calls, and the feed-forward half of a
+// layer plus final norm and lm_head.  Exit code 0 = all passed.
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -129,6 +130,85 @@ int decode_step() {
     return bad;
 }
 
+// The feed-forward half of a layer and the end of the step through the C++ methods of the
+// layer loop (batched_walker.cpp:346-431): RMSNorm -> Q4_0 gate/up -> gate/up split + SiLU ->
+// Q4_0 down -> residual add -> final RMSNorm -> Q6_K lm_head, one open pass, against the oracles.
+int ffn_and_head() {
+    auto& exec = mlc_amd::HipExecutor::Instance();
+    const size_t B = 5, HID = 256, FFN = 512, VOCAB = 128;
+    std::mt19937 rng(11);
+    std::normal_distribution<float> dist(0.f, 1.f);
+    auto randv = [&](size_t n, float s) { std::vector<float> v(n); for (auto& x : v) x = dist(rng) * s; return v; };
+    const std::vector<float> x = randv(B * HID, 1.f);
+    std::vector<float> g1(HID), g2(HID);
+    for (auto& w : g1) w = 0.5f + 0.01f * (float)(rng() % 100);
+    for (auto& w : g2) w = 0.5f + 0.01f * (float)(rng() % 100);
+    auto q4 = [&](size_t rows, size_t cols) {
+        std::vector<uint8_t> w(rows * (cols / 32) * 18);
+        const std::vector<float> f = randv(rows * cols, 0.05f);
+        for (size_t r = 0; r < rows; ++r) oracle_quantize_row_q4_0(f.data() + r * cols, cols, w.data() + r * (cols / 32) * 18);
+        return w;
+    };
+    const std::vector<uint8_t> w_gu = q4(2 * FFN, HID), w_down = q4(HID, FFN);
+    std::vector<uint8_t> w_head(VOCAB * (HID / 256) * 210);
+    {
+        const std::vector<float> f = randv(VOCAB * HID, 0.05f);
+        for (size_t r = 0; r < VOCAB; ++r) oracle_quantize_row_q6_k(f.data() + r * HID, HID, w_head.data() + r * (HID / 256) * 210);
+    }
+    // oracle chain
+    std::vector<float> n1(B * HID), gu(B * 2 * FFN), gate(B * FFN), up(B * FFN), mix(B * FFN), down(B * HID),
+        out(B * HID), n2(B * HID), logits(B * VOCAB);
+    int ok = oracle_rms_norm_batched(x.data(), g1.data(), HID, 1e-5f, B, HID, n1.data());
+    ok &= oracle_matmul_q4_0_batched(w_gu.data(), n1.data(), B, 2 * FFN, HID, HID / 32 * 18, gu.data(), 1);
+    ok &= oracle_gate_up_split_silu_mul(gu.data(), gate.data(), up.data(), mix.data(), B, FFN, 2 * FFN);
+    ok &= oracle_matmul_q4_0_batched(w_down.data(), mix.data(), B, HID, FFN, FFN / 32 * 18, down.data(), 1);
+    ok &= oracle_add(x.data(), down.data(), out.data(), B * HID);
+    ok &= oracle_rms_norm_batched(out.data(), g2.data(), HID, 1e-5f, B, HID, n2.data());
+    ok &= oracle_matmul_q6_k_batched(w_head.data(), n2.data(), B, VOCAB, HID, HID / 256 * 210, logits.data(), 1);
+    if (!ok) return 1;
+    // device
+    void* dx = exec.allocateScratchBuffer(B * HID * 4);
+    void* dn = exec.allocateScratchBuffer(B * HID * 4);
+    void* dgu = exec.allocateScratchBuffer(B * 2 * FFN * 4);
+    void* dgate = exec.allocateScratchBuffer(B * FFN * 4);
+    void* dup = exec.allocateScratchBuffer(B * FFN * 4);
+    void* dmix = exec.allocateScratchBuffer(B * FFN * 4);
+    void* ddown = exec.allocateScratchBuffer(B * HID * 4);
+    void* dout = exec.allocateScratchBuffer(B * HID * 4);
+    void* dlog = exec.allocateScratchBuffer(B * VOCAB * 4);
+    exec.uploadToBuffer(dx, x.data(), B * HID * 4);
+    int bad = 0;
+    bad |= !exec.beginForwardPassCB();
+    bad |= !exec.encodeRmsNormBatched(dx, g1, 1e-5f, B, HID, dn);
+    bad |= !exec.encodeMatMulQ4_0Batched("cpp.ffn_gate_up", w_gu, dn, B, 2 * FFN, HID, HID / 32 * 18, 1, dgu);
+    bad |= !exec.encodeGateUpSplitSiluMul(dgu, dgate, dup, dmix, B, FFN, 2 * FFN);
+    bad |= !exec.encodeMatMulQ4_0Batched("cpp.ffn_down", w_down, dmix, B, HID, FFN, FFN / 32 * 18, 1, ddown);
+    bad |= !exec.encodeAddBatched(dx, ddown, dout, B * HID);
+    bad |= !exec.encodeRmsNormBatched(dout, g2, 1e-5f, B, HID, dn);
+    bad |= !exec.encodeMatMulQ6KBatched("cpp.head", w_head, dn, B, VOCAB, HID, HID / 256 * 210, dlog);
+    bad |= !exec.flushForwardPassCB();
+    std::vector<float> got_out(B * HID), got_log(B * VOCAB);
+    exec.downloadFromBuffer(dout, got_out.data(), got_out.size() * 4);
+    exec.downloadFromBuffer(dlog, got_log.data(), got_log.size() * 4);
+    auto close = [](const std::vector<float>& a, const std::vector<float>& b) {
+        double worst = 0, scale = 0;
+        for (size_t i = 0; i < a.size(); ++i) {
+            worst = std::fmax(worst, std::fabs((double)a[i] - b[i]));
+            scale = std::fmax(scale, std::fabs((double)b[i]));
+        }
+        return worst <= 1e-4 * scale;
+    };
+    if (!close(got_out, out) || !close(got_log, logits)) bad = 1;
+    // the waiting form gives the same logits
+    bad |= !exec.runMatMulQ6KBatched("cpp.head", w_head, dn, B, VOCAB, HID, HID / 256 * 210, dlog);
+    std::vector<float> again(B * VOCAB);
+    exec.downloadFromBuffer(dlog, again.data(), again.size() * 4);
+    if (std::memcmp(again.data(), got_log.data(), again.size() * 4)) bad = 1;
+    for (void* b : {dx, dn, dgu, dgate, dup, dmix, ddown, dout, dlog}) exec.releaseScratchBuffer(b);
+    std::printf("%-32s %s\n", "FfnAndHead", bad ? "FAIL" : "ok");
+    return bad;
+}
+
 }  // namespace
 
 int main() {
@@ -149,5 +229,6 @@ int main() {
     int bad = 0;
     for (const auto& s : all) bad |= run(s);
     bad |= decode_step();
+    bad |= ffn_and_head();
     return bad;
 }

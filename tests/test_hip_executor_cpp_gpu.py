@@ -15,4 +15,4 @@ def test_cpp_scenarios(exe):
     proc = subprocess.run([EXE], capture_output=True, text=True, timeout=120)
     print(proc.stdout, proc.stderr, flush=True)
     assert proc.returncode == 0, proc.stdout + proc.stderr
-    assert proc.stdout.count(" ok") == 8
+    assert proc.stdout.count(" ok") == 9
