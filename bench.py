@@ -264,7 +264,7 @@ def bench_layer(args) -> int:
             "workload": f"decoder layer, TinyLlama-1.1B shape (hidden {lc.HID}, {lc.H}q/{lc.HKV}kv heads, "
                         f"head_dim {lc.D}, ffn {lc.FFN}), batch {B}, contexts of {c.name} "
                         f"(sum {int(c.seq_lens.sum())}), 11 operators per step, each step's output is the next "
-                        f"step's input, {n_layers} K/V pools rotated",
+                        f"step's input, {n_layers} K/V pools and {n_layers} device copies of the weights rotated",
             "weight_bytes_per_step": w_bytes, "kv_bytes_per_step": c.kv_bytes,
             "us_per_layer": round(us, 2),
             "tokens_per_s_at_22_layers": round(B / (22 * us * 1e-6), 1),

@@ -3,6 +3,8 @@
 // the measured rate is the GPU's and not the Python interpreter's call overhead.
 // It only calls entry points of include/mlc_hip.h; it adds no kernels of its own.
 #include <chrono>
+#include <string>
+#include <vector>
 #include <cstddef>
 #include <cstdint>
 
@@ -131,8 +133,9 @@ int mlc_bench_copy_loop(const void* src, void* dst, size_t bytes, size_t steps, 
 // One whole decoder layer per step, in the order of the reference's layer loop
 // (compiler/runtime/batched_walker.cpp:246-405): RMSNorm, qkv matmul, split + RoPE + KV write,
 // paged attention, out-projection, add, RMSNorm, gate/up matmul, SiLU gate, down-projection,
-// add.  Layer i uses K/V pool i % n_layers (the weights are the same for every layer: they
-// are re-read from HBM all the same, 12 MB do not stay in cache next to the KV traffic).
+// add.  Layer i uses K/V pool i % n_layers and its own device copy of the weights (the host
+// data is the same, the weight names differ), so that neither sits in the Infinity Cache from
+// the step before.
 struct MlcBenchLayer {
     const void* x;            // [batch][hidden] fp32 input of the layer
     void* norm; void* qkv; void* q; void* attn; void* o; void* resid; void* gate_up;
@@ -157,6 +160,11 @@ int mlc_bench_layer_loop(const MlcBenchLayer* L, void* const* k_pools, void* con
     const size_t q_rows = L->num_heads * L->head_dim, kv_rows = L->kv_heads * L->head_dim;
     const size_t qkv_rows = q_rows + 2 * kv_rows;
     const size_t s_hid = HID / 32 * 18, s_ffn = FFN / 32 * 18;
+    std::vector<std::string> names(n_layers * 4);
+    for (size_t l = 0; l < n_layers; ++l) {
+        const char* kinds[4] = {"attn_qkv", "attn_output", "ffn_gate_up", "ffn_down"};
+        for (int k = 0; k < 4; ++k) names[l * 4 + k] = "bench.l" + std::to_string(l) + "." + kinds[k];
+    }
     if (!mlc_hip_begin()) return 0;
     const auto t0 = std::chrono::steady_clock::now();
     if (!mlc_hip_timer_start()) return 0;
@@ -165,7 +173,7 @@ int mlc_bench_layer_loop(const MlcBenchLayer* L, void* const* k_pools, void* con
         const void* x = (L->out2 && i > 0) ? ((i - 1) % 2 ? L->out2 : L->out) : L->x;
         void* out = (L->out2 && i % 2) ? L->out2 : L->out;
         int ok = mlc_hip_rms_norm_batched(x, L->attn_norm_w, HID, 1e-5f, B, HID, L->norm, 0);
-        ok = ok && mlc_hip_matmul_q4_0_batched("bench.attn_qkv", L->w_qkv, L->w_qkv_bytes, L->norm, B,
+        ok = ok && mlc_hip_matmul_q4_0_batched(names[l * 4 + 0].c_str(), L->w_qkv, L->w_qkv_bytes, L->norm, B,
                                                qkv_rows, HID, s_hid, 1, L->qkv, 0);
         ok = ok && mlc_hip_qkv_split_rope_scatter(L->qkv, L->q, k_pools[l], v_pools[l], nullptr, nullptr,
                                                   L->cos, L->sin, L->page_ids, L->slots,
@@ -176,14 +184,14 @@ int mlc_bench_layer_loop(const MlcBenchLayer* L, void* const* k_pools, void* con
                                              L->n_flat, L->page_table_offsets, L->seq_lens,
                                              L->q_positions, B, L->num_heads, L->kv_heads, L->head_dim,
                                              L->page_size_tokens, 1, 0);
-        ok = ok && mlc_hip_matmul_q4_0_batched("bench.attn_output", L->w_o, L->w_o_bytes, L->attn, B, HID,
+        ok = ok && mlc_hip_matmul_q4_0_batched(names[l * 4 + 1].c_str(), L->w_o, L->w_o_bytes, L->attn, B, HID,
                                                HID, s_hid, 1, L->o, 0);
         ok = ok && mlc_hip_add_batched(x, L->o, L->resid, B * HID, 0);
         ok = ok && mlc_hip_rms_norm_batched(L->resid, L->ffn_norm_w, HID, 1e-5f, B, HID, L->norm, 0);
-        ok = ok && mlc_hip_matmul_q4_0_batched("bench.ffn_gate_up", L->w_gate_up, L->w_gate_up_bytes,
+        ok = ok && mlc_hip_matmul_q4_0_batched(names[l * 4 + 2].c_str(), L->w_gate_up, L->w_gate_up_bytes,
                                                L->norm, B, 2 * FFN, HID, s_hid, 1, L->gate_up, 0);
         ok = ok && mlc_hip_gate_up_split_silu_mul(L->gate_up, L->gate, L->up, L->mix, B, FFN, 2 * FFN, 0);
-        ok = ok && mlc_hip_matmul_q4_0_batched("bench.ffn_down", L->w_down, L->w_down_bytes, L->mix, B,
+        ok = ok && mlc_hip_matmul_q4_0_batched(names[l * 4 + 3].c_str(), L->w_down, L->w_down_bytes, L->mix, B,
                                                HID, FFN, s_ffn, 1, L->down, 0);
         ok = ok && mlc_hip_add_batched(L->resid, L->down, out, B * HID, 0);
         if (!ok) return 0;
