@@ -203,7 +203,8 @@ def bench_layer(args) -> int:
                                                  "head_dim", "page_size_tokens", "batch")]
                     + [("page_ids", u32p), ("slots", u32p), ("page_tables_flat", u32p),
                        ("n_flat", C.c_size_t), ("page_table_offsets", u32p), ("seq_lens", u32p),
-                       ("q_positions", u32p)])
+                       ("q_positions", u32p), ("head_norm_w", f32p), ("head_w", C.c_void_p),
+                       ("head_bytes", C.c_size_t), ("head_rows", C.c_size_t), ("logits", C.c_void_p)])
 
     meta = {n: np.ascontiguousarray(a, np.uint32) for n, a in
             (("page_ids", page_ids), ("slots", slots), ("page_tables_flat", c.page_tables_flat),
@@ -226,6 +227,17 @@ def bench_layer(args) -> int:
         setattr(L, n, a.ctypes.data_as(u32p))
     L.n_flat = meta["page_tables_flat"].size
 
+    whole_step = args.workload == "step"
+    VOCAB = 32000
+    if whole_step:   # final RMSNorm + Q6_K lm_head after every 22nd layer: one decode step of the model
+        from oracle import paged_oracle as po
+        head_norm = rng.uniform(0.5, 1.5, lc.HID).astype(np.float32)
+        w_head = po.quantize_q6_k((rng.standard_normal((VOCAB, lc.HID)) * 0.03).astype(np.float32))
+        keep.extend([head_norm, w_head])
+        L.head_norm_w = head_norm.ctypes.data_as(f32p)
+        L.head_w, L.head_bytes, L.head_rows = w_head.ctypes.data, w_head.nbytes, VOCAB
+        L.logits = dev(B * VOCAB)
+
     bl = C.CDLL(BENCH_LIB_PATH)
     kp = (C.c_void_p * n_layers)(*k_bufs)
     vp = (C.c_void_p * n_layers)(*v_bufs)
@@ -241,6 +253,9 @@ def bench_layer(args) -> int:
     # timed: every step reads the step before's output, like the layers of a model (the
     # residual add of one layer and the RMSNorm of the next are neighbours in the pass)
     L.out2 = dev(B * lc.HID)
+    if whole_step:
+        return finish_step(args, exe, L, loop, lc, c, w, x, cos, sin, page_ids, slots, qpos, n_layers,
+                           VOCAB, head_norm, w_head)
     ev_ms, wall = loop(args.steps)
     L.out2 = None
     loop(1)                              # one step from the known input, for the parity check
@@ -296,6 +311,69 @@ def bench_layer(args) -> int:
         result["parity_vs_cpu_baseline"] = {"cosine": round(po.cosine(got.ravel(), ref["out"].ravel()), 8),
                                             "max_abs_over_max": float(f"{rel:.3e}"),
                                             "requests_checked": nb}
+    print(json.dumps(result))
+    return 0
+
+
+def finish_step(args, exe, L, loop, lc, c, w, x, cos, sin, page_ids, slots, qpos, n_layers, VOCAB,
+                head_norm, w_head) -> int:
+    """--workload step: times whole decode steps of a TinyLlama-1.1B-shape model (22 decoder
+    layers, final RMSNorm, Q6_K lm_head) and checks the logits of one step against the CPU chain."""
+    from oracle import paged_oracle as po
+    B = c.batch
+    steps = max(1, min(args.steps, 200))
+    loop(n_layers)                                  # first use of the lm_head: upload and repack
+    ev_ms, wall = loop(steps * n_layers)
+    loop(n_layers)                                  # one step from the known input, for the parity check
+    # (with out2 set, layer 0 of a loop reads x and every later layer the one before: a whole step)
+    logits = np.empty((B, VOCAB), np.float32)
+    exe.downloadFromBuffer(L.logits, logits)
+    w_bytes = lc.weight_bytes(w) * n_layers + w_head.nbytes
+    alg_bytes = w_bytes + c.kv_bytes * n_layers
+    s_per_step = wall / steps
+    ev_s = ev_ms / steps * 1e-3
+    result = {
+        "metric": "decode step tokens/s (22 decoder layers + final norm + lm_head), TinyLlama-1.1B shape B=32",
+        "value": round(B / s_per_step, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps,
+        "warmup": 2, "ms_per_step": round(s_per_step * 1e3, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32 (Q4_0 / Q6_K weights, fp16 K/V storage; matmuls on split-fp16 MFMA with fp32 accumulate)",
+        "data": "synthetic",
+        "config": {
+            "workload": f"decode step: {n_layers} decoder layers (hidden {lc.HID}, {lc.H}q/{lc.HKV}kv heads, "
+                        f"head_dim {lc.D}, ffn {lc.FFN}, Q4_0) + RMSNorm + lm_head ({VOCAB} x {lc.HID}, Q6_K), "
+                        f"batch {B}, contexts of {c.name} (sum {int(c.seq_lens.sum())}), random weights "
+                        f"(one host copy, {n_layers} device copies), one open pass per step loop",
+            "weight_bytes_per_step": w_bytes, "kv_bytes_per_step": c.kv_bytes * n_layers,
+            "us_per_layer": round((s_per_step * 1e6) / n_layers, 2),
+        },
+        "roofline": {"bound": "hbm", "achieved": round(alg_bytes / ev_s / 1e9, 2), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(alg_bytes / ev_s / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                     "us_per_launch": round(ev_s * 1e6, 2),
+                     "note": "a whole step (222 kernels) between HIP events / steps; algorithmic bytes = all "
+                             "weights once + the K/V of all layers"},
+    }
+    if not args.no_cpu:
+        nb = 16   # bounded sample: the first 16 requests through all 22 layers and the head, 8 threads
+        off = c.page_table_offsets
+        flat = c.page_tables_flat[:off[nb]]
+        n_thr = min(os.cpu_count() or 1, 8)
+        t0 = time.perf_counter()
+        h = x[:nb]
+        for _ in range(n_layers):
+            h = lc.oracle_chain(w, h, cos[:nb], sin[:nb], c.k_pages, c.v_pages, page_ids[:nb], slots[:nb],
+                                flat, off[:nb + 1], c.seq_lens[:nb], qpos[:nb], n_threads=n_thr)["out"]
+        hn = po.rms_norm_batched(h, head_norm, 1e-5, nb, lc.HID)
+        want = po.matmul_q6_k_batched(w_head, hn, nb, VOCAB, lc.HID, n_threads=n_thr)
+        dt = time.perf_counter() - t0
+        result["cpu_baseline"] = {"value": round(nb / dt, 3), "unit": "tokens/s", "cores": n_thr, "kind": "port",
+                                  "sample": f"{nb} of {B} requests through the same step, {dt:.2f} s"}
+        got = logits[:nb]
+        result["parity_vs_cpu_baseline"] = {
+            "cosine": round(po.cosine(got.ravel(), want.ravel()), 8),
+            "max_abs_over_max": float(f"{float(np.max(np.abs(got - want)) / np.max(np.abs(want))):.3e}"),
+            "argmax_agree": int(np.sum(np.argmax(got, axis=1) == np.argmax(want, axis=1))),
+            "requests_checked": nb}
     print(json.dumps(result))
     return 0
 
@@ -368,7 +446,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=100)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "layer", "copy"])
+    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "layer", "step", "copy"])
     ap.add_argument("--copy-mib", type=int, default=32, help="size of the calibration copy")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU baseline work")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -386,7 +464,7 @@ def main() -> int:
         return bench_prefill(args)
     if args.workload == "copy":
         return bench_copy(args)
-    if args.workload == "layer":
+    if args.workload in ("layer", "step"):
         return bench_layer(args)
 
     from mlcompiler_amd import HipExecutor

@@ -152,6 +152,9 @@ struct MlcBenchLayer {
     const uint32_t* page_ids; const uint32_t* slots;
     const uint32_t* page_tables_flat; size_t n_flat;
     const uint32_t* page_table_offsets; const uint32_t* seq_lens; const uint32_t* q_positions;
+    // when head_w is set: after every n_layers-th layer the final RMSNorm and the Q6_K lm_head
+    // (batched_walker.cpp:415-431), i.e. n_layers steps are one decode step of the model
+    const float* head_norm_w; const void* head_w; size_t head_bytes; size_t head_rows; void* logits;
 };
 
 int mlc_bench_layer_loop(const MlcBenchLayer* L, void* const* k_pools, void* const* v_pools,
@@ -194,6 +197,11 @@ int mlc_bench_layer_loop(const MlcBenchLayer* L, void* const* k_pools, void* con
         ok = ok && mlc_hip_matmul_q4_0_batched(names[l * 4 + 3].c_str(), L->w_down, L->w_down_bytes, L->mix, B,
                                                HID, FFN, s_ffn, 1, L->down, 0);
         ok = ok && mlc_hip_add_batched(L->resid, L->down, out, B * HID, 0);
+        if (ok && L->head_w && l == n_layers - 1) {
+            ok = mlc_hip_rms_norm_batched(out, L->head_norm_w, HID, 1e-5f, B, HID, L->norm, 0);
+            ok = ok && mlc_hip_matmul_q6_k_batched("bench.lm_head", L->head_w, L->head_bytes, L->norm, B,
+                                                   L->head_rows, HID, HID / 256 * 210, L->logits, 0);
+        }
         if (!ok) return 0;
     }
     const float ms = mlc_hip_timer_stop();
