@@ -94,7 +94,7 @@ def reference_scenarios():
 
 
 def baseline_config(idx: int, *, batch=None, seed=1234) -> DecodeCase:
-    """Decode configurations 1-4 of the benchmark definition (BASELINE.json `configs`)."""
+    """Decode configurations 1-4 of the benchmark definition."""
     rng = np.random.default_rng(seed + idx)
     if idx == 1:
         return make_case("cfg1_single", 1, 32, 4, 64, 64, [512], capacity_pages=8, permute=False, seed=seed)
