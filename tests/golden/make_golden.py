@@ -12,6 +12,10 @@ that read them run anywhere:
                          small GQA decode cases, stored with their paged inputs
   allocator_golden.txt   a PagePool / RequestKVState script and the replies of
                          compiler/runtime/paged_kv.cpp, one "command => reply" per line
+  quant_rope_golden.npz  quantizeRowQ4_0 / dotProductRowQ4_0, quantizeRowQ6_K / dequantizeRowQ6_K /
+                         dotProductRowQ6_K (compiler/runtime/quantization.cpp:235-311, 1469-1663)
+                         and computeRotaryCoefficients / applyRotaryEmbedding (:772-823) on seeded
+                         rows, stored with their inputs
 
 Run:  python tests/golden/make_golden.py
 """
@@ -108,7 +112,41 @@ def main() -> int:
     with open(os.path.join(HERE, "allocator_golden.txt"), "w") as fh:
         for cmd, rep in zip(script, replies):
             fh.write(f"{cmd} => {rep}\n")
-    print("wrote fp16_golden.npz, attention_golden.npz, allocator_golden.txt")
+    # ---- quantised rows and RoPE
+    R = po.ref_lib()
+    rng = np.random.default_rng(4242)
+    out = {}
+    for tag, cols in (("a", 64), ("b", 320), ("c", 2048)):       # 320: partial last Q6_K block
+        w = (rng.standard_normal((4, cols)) * rng.uniform(0.01, 3)).astype(np.float32)
+        x = rng.standard_normal((3, cols)).astype(np.float32)
+        q4 = np.zeros((4, po.q4_0_row_bytes(cols)), np.uint8)
+        q6 = np.zeros((4, po.q6_k_row_bytes(cols)), np.uint8)
+        deq6 = np.zeros((4, cols), np.float32)
+        dot4 = np.zeros((3, 4), np.float32)
+        dot6 = np.zeros((3, 4), np.float32)
+        for r in range(4):
+            assert R.ref_quantize_row_q4_0(w[r].ctypes.data_as(po._f32p), cols, q4[r].ctypes.data, q4.shape[1]) == q4.shape[1]
+            assert R.ref_quantize_row_q6_k(w[r].ctypes.data_as(po._f32p), cols, q6[r].ctypes.data, q6.shape[1]) == q6.shape[1]
+            R.ref_dequantize_row_q6_k(q6[r].ctypes.data, cols, deq6[r].ctypes.data_as(po._f32p))
+            for b in range(3):
+                dot4[b, r] = R.ref_dot_q4_0(q4[r].ctypes.data, cols, x[b].ctypes.data_as(po._f32p))
+                dot6[b, r] = R.ref_dot_q6_k(q6[r].ctypes.data, cols, x[b].ctypes.data_as(po._f32p))
+        out.update({f"w_{tag}": w, f"x_{tag}": x, f"q4_{tag}": q4, f"q6_{tag}": q6,
+                    f"deq6_bits_{tag}": deq6.view(np.uint32), f"dot4_bits_{tag}": dot4.view(np.uint32),
+                    f"dot6_bits_{tag}": dot6.view(np.uint32)})
+    rope = []
+    for i, (pos, head_dim, rot, base, scale) in enumerate([(0, 64, 64, 10000.0, 1.0), (1, 64, 64, 10000.0, 1.0),
+                                                           (1234, 128, 128, 500000.0, 1.0), (77, 64, 32, 10000.0, 0.5),
+                                                           (4095, 20, 8, 10000.0, 1.0)]):
+        cos, sin = po.ref_rotary_coefficients(pos, rot, base, scale)
+        vec = rng.standard_normal(head_dim).astype(np.float32)
+        out[f"rope_in_{i}"] = vec
+        out[f"rope_cos_bits_{i}"], out[f"rope_sin_bits_{i}"] = cos.view(np.uint32), sin.view(np.uint32)
+        out[f"rope_out_bits_{i}"] = po.ref_apply_rotary(vec, cos, sin, head_dim, rot).view(np.uint32)
+        rope.append([pos, head_dim, rot, base, scale])
+    out["rope_cases"] = np.array(rope, np.float64)
+    np.savez_compressed(os.path.join(HERE, "quant_rope_golden.npz"), **out)
+    print("wrote fp16_golden.npz, attention_golden.npz, allocator_golden.txt, quant_rope_golden.npz")
     return 0
 
 

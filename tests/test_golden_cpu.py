@@ -58,3 +58,36 @@ def test_allocator_replies_match_golden_transcript():
             want.append(rep)
     assert len(script) > 300
     assert replay_allocator_script(script) == want
+
+
+def test_quantised_rows_bit_exact_with_golden():
+    """Q4_0 / Q6_K quantise, dequantise and dot products as the reference's quantization.cpp
+    produced them."""
+    g = np.load(os.path.join(GOLDEN, "quant_rope_golden.npz"))
+    for tag in "abc":
+        w, x = g[f"w_{tag}"], g[f"x_{tag}"]
+        cols = w.shape[1]
+        assert np.array_equal(po.quantize_q4_0(w), g[f"q4_{tag}"])
+        assert np.array_equal(po.quantize_q6_k(w), g[f"q6_{tag}"])
+        assert np.array_equal(po.dequantize_q6_k(g[f"q6_{tag}"], cols).view(np.uint32), g[f"deq6_bits_{tag}"])
+        got4 = po.matmul_q4_0_batched(g[f"q4_{tag}"], x, 3, 4, cols, n_threads=1)
+        got6 = po.matmul_q6_k_batched(g[f"q6_{tag}"], x, 3, 4, cols, n_threads=1)
+        assert np.array_equal(got4.view(np.uint32), g[f"dot4_bits_{tag}"])
+        assert np.array_equal(got6.view(np.uint32), g[f"dot6_bits_{tag}"])
+
+
+def test_rope_bit_exact_with_golden():
+    """computeRotaryCoefficients and applyRotaryEmbedding outputs of the reference."""
+    g = np.load(os.path.join(GOLDEN, "quant_rope_golden.npz"))
+    for i, (pos, head_dim, rot, base, scale) in enumerate(g["rope_cases"]):
+        pos, head_dim, rot = int(pos), int(head_dim), int(rot)
+        cos, sin = po.rotary_coefficients(pos, rot, float(base), float(scale))
+        assert np.array_equal(cos.view(np.uint32), g[f"rope_cos_bits_{i}"])
+        assert np.array_equal(sin.view(np.uint32), g[f"rope_sin_bits_{i}"])
+        # one request, one head: the fused-row layout of the operator is [q | k | v], q only here
+        vec = g[f"rope_in_{i}"]
+        qkv = np.concatenate([vec, np.zeros(2 * head_dim, np.float32)])[None, :]
+        res = po.qkv_split_rope_cast(qkv, cos[None, :], sin[None, :], 1, 1, 1, head_dim, 3 * head_dim,
+                                     head_dim, head_dim, head_dim, rot)
+        assert res is not None
+        assert np.array_equal(res[0][0].view(np.uint32), g[f"rope_out_bits_{i}"])
