@@ -204,7 +204,8 @@ def bench_layer(args) -> int:
                     + [("page_ids", u32p), ("slots", u32p), ("page_tables_flat", u32p),
                        ("n_flat", C.c_size_t), ("page_table_offsets", u32p), ("seq_lens", u32p),
                        ("q_positions", u32p), ("head_norm_w", f32p), ("head_w", C.c_void_p),
-                       ("head_bytes", C.c_size_t), ("head_rows", C.c_size_t), ("logits", C.c_void_p)])
+                       ("head_bytes", C.c_size_t), ("head_rows", C.c_size_t), ("logits", C.c_void_p),
+                       ("enqueue_s", C.POINTER(C.c_double))])
 
     meta = {n: np.ascontiguousarray(a, np.uint32) for n, a in
             (("page_ids", page_ids), ("slots", slots), ("page_tables_flat", c.page_tables_flat),
@@ -226,6 +227,8 @@ def bench_layer(args) -> int:
     for n, a in meta.items():
         setattr(L, n, a.ctypes.data_as(u32p))
     L.n_flat = meta["page_tables_flat"].size
+    enqueue_s = C.c_double()
+    L.enqueue_s = C.pointer(enqueue_s)
 
     whole_step = args.workload == "step"
     VOCAB = 32000
@@ -257,6 +260,7 @@ def bench_layer(args) -> int:
         return finish_step(args, exe, L, loop, lc, c, w, x, cos, sin, page_ids, slots, qpos, n_layers,
                            VOCAB, head_norm, w_head)
     ev_ms, wall = loop(args.steps)
+    host_encode_us = enqueue_s.value / args.steps * 1e6
     L.out2 = None
     loop(1)                              # one step from the known input, for the parity check
     out = np.empty((B, lc.HID), np.float32)
@@ -282,6 +286,7 @@ def bench_layer(args) -> int:
                         f"step's input, {n_layers} K/V pools and {n_layers} device copies of the weights rotated",
             "weight_bytes_per_step": w_bytes, "kv_bytes_per_step": c.kv_bytes,
             "us_per_layer": round(us, 2),
+            "host_encode_us_per_layer": round(host_encode_us, 2),
             "tokens_per_s_at_22_layers": round(B / (22 * us * 1e-6), 1),
         },
         "roofline": {"bound": "hbm", "achieved": round(ach, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -155,6 +155,7 @@ struct MlcBenchLayer {
     // when head_w is set: after every n_layers-th layer the final RMSNorm and the Q6_K lm_head
     // (batched_walker.cpp:415-431), i.e. n_layers steps are one decode step of the model
     const float* head_norm_w; const void* head_w; size_t head_bytes; size_t head_rows; void* logits;
+    double* enqueue_s;        // when set: receives the host time spent encoding (before the wait)
 };
 
 int mlc_bench_layer_loop(const MlcBenchLayer* L, void* const* k_pools, void* const* v_pools,
@@ -204,6 +205,7 @@ int mlc_bench_layer_loop(const MlcBenchLayer* L, void* const* k_pools, void* con
         }
         if (!ok) return 0;
     }
+    if (L->enqueue_s) *L->enqueue_s = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
     const float ms = mlc_hip_timer_stop();
     if (ms < 0.f) return 0;
     if (!mlc_hip_flush()) return 0;
