@@ -1,0 +1,104 @@
+"""Random sequences of the row-local operators (add, RMSNorm, gate/up SiLU, Q4_0 matmul) with
+shared and in-place buffers, encoded in one pass twice: with the fused chains (the default) and
+with every operator launched on its own.  Deferring and fusing must never change what a
+sequence computes: every buffer is compared at the end (and after a read-back in the middle of
+the pass).  add is exact; RMSNorm sums in another order in the fused kernel, so buffers are
+compared to 1e-4 of their largest value."""
+import numpy as np
+import pytest
+
+from oracle import paged_oracle as po
+
+pytestmark = pytest.mark.gpu
+
+B, L = 5, 256
+
+
+def _program(rng, n_ops):
+    """ops over buffers: 'n' = [B][L] (indices 0..5), 'w' = [B][2L] (indices 0..1)"""
+    ops = []
+    for _ in range(n_ops):
+        kind = rng.choice(["add", "add", "rms", "rms", "mm_n", "mm_w", "silu", "peek"])
+        if kind == "add":
+            a, b, c = (int(v) for v in rng.integers(0, 6, 3))
+            ops.append(("add", a, b, c))                       # c may alias a or b
+        elif kind == "rms":
+            a, c = (int(v) for v in rng.integers(0, 6, 2))
+            ops.append(("rms", a, c, int(rng.integers(0, 2))))  # c may alias a; one of two weight vectors
+        elif kind == "mm_n":
+            a = int(rng.integers(0, 6))
+            c = int(rng.choice([i for i in range(6) if i != a]))
+            ops.append(("mm_n", a, c))
+        elif kind == "mm_w":
+            ops.append(("mm_w", int(rng.integers(0, 6)), int(rng.integers(0, 2))))
+        elif kind == "silu":
+            g, u, m = (int(v) for v in rng.choice(6, 3, replace=False))
+            ops.append(("silu", int(rng.integers(0, 2)), g, u, m))
+        else:
+            ops.append(("peek", int(rng.integers(0, 6))))
+    return ops
+
+
+def _run(exe, ops, init_n, init_w, weights, gammas, fuse, ksplit):
+    # options are set before the pass: setting one launches what is pending
+    assert exe.setOption("fuse_row_ops", fuse)
+    assert exe.setOption("q4_ksplit", ksplit)
+    n = [exe.allocateScratchBuffer(B * L * 4) for _ in range(6)]
+    w = [exe.allocateScratchBuffer(B * 2 * L * 4) for _ in range(2)]
+    peeks = []
+    try:
+        for buf, a in zip(n + w, init_n + init_w):
+            assert exe.uploadToBuffer(buf, a)
+        assert exe.beginForwardPassCB()
+        for op in ops:
+            if op[0] == "add":
+                assert exe.encodeAddBatched(n[op[1]], n[op[2]], n[op[3]], B * L)
+            elif op[0] == "rms":
+                assert exe.encodeRmsNormBatched(n[op[1]], gammas[op[3]], 1e-5, B, L, n[op[2]])
+            elif op[0] == "mm_n":
+                assert exe.encodeMatMulQ4_0Batched("fuzz.n", weights["n"], n[op[1]], B, L, L, weights["n"].shape[1], 1,
+                                                   n[op[2]]), exe.lastError()
+            elif op[0] == "mm_w":
+                assert exe.encodeMatMulQ4_0Batched("fuzz.w", weights["w"], n[op[1]], B, 2 * L, L, weights["w"].shape[1], 1,
+                                                   w[op[2]]), exe.lastError()
+            elif op[0] == "silu":
+                assert exe.encodeGateUpSplitSiluMul(w[op[1]], n[op[2]], n[op[3]], n[op[4]], B, L, 2 * L)
+            else:
+                out = np.empty((B, L), np.float32)
+                assert exe.downloadFromBuffer(n[op[1]], out)      # in the middle of the pass
+                peeks.append(out)
+        assert exe.flushForwardPassCB(), exe.lastError()
+        final = []
+        for buf, shape in zip(n + w, [(B, L)] * 6 + [(B, 2 * L)] * 2):
+            out = np.empty(shape, np.float32)
+            assert exe.downloadFromBuffer(buf, out)
+            final.append(out)
+    finally:
+        exe.setOption("fuse_row_ops", 1)
+        exe.setOption("q4_ksplit", 0)
+        for buf in n + w:
+            exe.releaseScratchBuffer(buf)
+    return final, peeks
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_fused_and_unfused_sequences_agree(exe, seed):
+    rng = np.random.default_rng(1000 + seed)
+    ops = _program(rng, 14)
+    print(f"[fuzz {seed}] " + " ".join(o[0] + ":" + ",".join(str(v) for v in o[1:]) for o in ops), flush=True)
+    init_n = [rng.standard_normal((B, L)).astype(np.float32) for _ in range(6)]
+    init_w = [rng.standard_normal((B, 2 * L)).astype(np.float32) for _ in range(2)]
+    weights = {"n": po.quantize_q4_0((rng.standard_normal((L, L)) * 0.06).astype(np.float32)),
+               "w": po.quantize_q4_0((rng.standard_normal((2 * L, L)) * 0.06).astype(np.float32))}
+    gammas = [rng.uniform(0.5, 1.5, L).astype(np.float32) for _ in range(2)]
+    ksplit = int(rng.choice([0, 2]))     # 2: the matmuls leave K slices for the next chain to sum
+    before = exe.rowProgramLaunches()
+    fused, fused_peeks = _run(exe, ops, init_n, init_w, weights, gammas, 1, ksplit)
+    n_fused = exe.rowProgramLaunches() - before
+    assert n_fused > 0
+    plain, plain_peeks = _run(exe, ops, init_n, init_w, weights, gammas, 0, ksplit)
+    assert exe.rowProgramLaunches() - before == n_fused       # none with fusion off
+    for i, (a, b) in enumerate(list(zip(fused, plain)) + list(zip(fused_peeks, plain_peeks))):
+        assert np.all(np.isfinite(a)) and np.all(np.isfinite(b))
+        scale = max(float(np.max(np.abs(b))), 1e-30)
+        assert float(np.max(np.abs(a - b))) <= 1e-4 * scale, (i, float(np.max(np.abs(a - b))), scale)
