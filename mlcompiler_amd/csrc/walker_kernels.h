@@ -128,7 +128,8 @@ template <int NG>  // groups of 8 elements per thread
 __global__ __launch_bounds__(kRowThreads) void row_program_kernel(const RowProgram p) {
     constexpr int NWAVE = kRowThreads / 64;
     constexpr int SB = 8;  // K slices whose loads are in flight together
-    __shared__ float red[NWAVE];
+    __shared__ float red[NWAVE];      // sum of squares per wave (rms)
+    __shared__ float red_max[NWAVE];  // largest magnitude per wave (split)
     const uint32_t row = blockIdx.x;
     const uint32_t tid = threadIdx.x;
     const bool live = row < p.batch;
@@ -192,8 +193,16 @@ __global__ __launch_bounds__(kRowThreads) void row_program_kernel(const RowProgr
                 store8(p.add_out, col, v[j]);
             }
         }
-        // ---- rms
+        // ---- rms (the weights are fetched before the reduction, not behind its barrier)
         if (p.rms) {
+            float gamma[NG][8];
+#pragma unroll
+            for (int j = 0; j < NG; ++j) {
+                const uint32_t col = (j * kRowThreads + tid) * 8;
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    gamma[j][e] = (col < len && col + e < p.n_weight) ? p.rms_weight[col + e] : 1.0f;
+            }
             float sum = 0.f;
 #pragma unroll
             for (int j = 0; j < NG; ++j) {
@@ -208,17 +217,13 @@ __global__ __launch_bounds__(kRowThreads) void row_program_kernel(const RowProgr
             float total = 0.f;
 #pragma unroll
             for (int w = 0; w < NWAVE; ++w) total += red[w];
-            __syncthreads();  // red is used again by the split stage
             const float scale = 1.0f / sqrtf(total / (float)len + p.epsilon);
 #pragma unroll
             for (int j = 0; j < NG; ++j) {
                 const uint32_t col = (j * kRowThreads + tid) * 8;
                 if (col >= len) continue;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float gamma = col + e < p.n_weight ? p.rms_weight[col + e] : 1.0f;
-                    v[j][e] = v[j][e] * scale * gamma;
-                }
+                for (int e = 0; e < 8; ++e) v[j][e] = v[j][e] * scale * gamma[j][e];
                 store8(p.rms_out, col, v[j]);
             }
         }
@@ -237,10 +242,10 @@ __global__ __launch_bounds__(kRowThreads) void row_program_kernel(const RowProgr
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
-    if (tid % 64 == 0) red[tid / 64] = amax;
+    if (tid % 64 == 0) red_max[tid / 64] = amax;
     __syncthreads();
 #pragma unroll
-    for (int w = 0; w < NWAVE; ++w) amax = fmaxf(amax, red[w]);
+    for (int w = 0; w < NWAVE; ++w) amax = fmaxf(amax, red_max[w]);
     int ex = 0;
     if (amax > 0.f && amax < INFINITY) (void)frexpf(amax, &ex);
     int se = 14 - ex;
