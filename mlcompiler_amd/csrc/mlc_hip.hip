@@ -1241,7 +1241,7 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
     // does the pending chain end in this matmul's input?  (decided before anything below can
     // replace a buffer the chain still refers to)
     const bool feeds = batch <= 64 && !g.opt_q4_force_generic && !(reinterpret_cast<uintptr_t>(out) & 15u) &&
-                       q4_fast_shape(rows, cols, row_stride) && rows_continue(in, batch, cols);
+                       q4_fast_shape(rows, cols, row_stride) && row_len_ok(cols) && rows_continue(in, batch, cols);
     if (!feeds && !settle()) return 0;
     Ctx::Q4Weight* w = q4_weight(weight_name, static_cast<const uint8_t*>(weights), weight_bytes, rows, cols, row_stride);
     if (!w) return 0;
@@ -1400,7 +1400,7 @@ int mlc_hip_matmul_q6_k_batched(const char* weight_name, const void* weights, si
     const size_t ki = known_bytes(in), ko = known_bytes(out);
     if ((ki && batch * cols * 4 > ki) || (ko && batch * rows * 4 > ko)) return fail("q6_k matmul: buffer too small");
     const bool fast = q6k_fast_shape(rows, cols, row_stride) && !g.opt_q4_force_generic;
-    const bool feeds = fast && batch <= 64 && rows_continue(in, batch, cols);
+    const bool feeds = fast && batch <= 64 && row_len_ok(cols) && rows_continue(in, batch, cols);
     if (!feeds && !settle()) return 0;
     Ctx::Q6KWeight* w = q6k_weight(weight_name, static_cast<const uint8_t*>(weights), weight_bytes, rows, cols, row_stride);
     if (!w) return 0;

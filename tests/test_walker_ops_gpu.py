@@ -221,3 +221,30 @@ def test_gate_up_then_matmul_then_add_in_one_pass(exe, batch, hid, ffn, rows, fu
         exe.setOption("q4_ksplit", 0)
         for b in bufs:
             exe.releaseScratchBuffer(b)
+
+
+def test_long_rows_between_two_matmuls(exe):
+    """A matmul whose output rows are longer than the fused row kernel handles (20480 > 16384),
+    split over K so that the sum of its slices is pending, feeding another matmul directly: the
+    sum and the split of the second matmul's input then run as separate kernels."""
+    rng = np.random.default_rng(21)
+    batch, k1, mid, rows2 = 3, 1024, 20480, 64
+    w1 = po.quantize_q4_0((rng.standard_normal((mid, k1)) * 0.05).astype(np.float32))
+    w2 = po.quantize_q4_0((rng.standard_normal((rows2, mid)) * 0.02).astype(np.float32))
+    x = rng.standard_normal((batch, k1)).astype(np.float32)
+    want_mid = po.matmul_q4_0_batched(w1, x, batch, mid, k1)
+    want = po.matmul_q4_0_batched(w2, want_mid, batch, rows2, mid)
+    d_x, d_mid, d_out = _up(exe, x), exe.allocateScratchBuffer(batch * mid * 4), exe.allocateScratchBuffer(batch * rows2 * 4)
+    try:
+        assert exe.setOption("q4_ksplit", 2)
+        assert exe.beginForwardPassCB()
+        assert exe.encodeMatMulQ4_0Batched("long.a", w1, d_x, batch, mid, k1, w1.shape[1], 1, d_mid), exe.lastError()
+        assert exe.encodeMatMulQ4_0Batched("long.b", w2, d_mid, batch, rows2, mid, w2.shape[1], 1, d_out), exe.lastError()
+        assert exe.flushForwardPassCB(), exe.lastError()
+        got_mid, got = _down(exe, d_mid, (batch, mid)), _down(exe, d_out, (batch, rows2))
+    finally:
+        exe.setOption("q4_ksplit", 0)
+        for b in (d_x, d_mid, d_out):
+            exe.releaseScratchBuffer(b)
+    assert np.max(np.abs(got_mid - want_mid)) < 2e-5 * float(np.max(np.abs(want_mid)))
+    assert np.max(np.abs(got - want)) < 1e-4 * float(np.max(np.abs(want)))
