@@ -550,6 +550,41 @@ def main() -> int:
     assert exe.flushForwardPassCB()
     boundary_us = (time.perf_counter() - tb) / n_b * 1e6
 
+    # ---- the layer as the batched step runs it (batched_walker.cpp:304-331): write the step's
+    # new K row and V row (they land on the newest position: the bytes read stay the same), then
+    # attend.  Three launches per layer.
+    rng = np.random.default_rng(5)
+    row = c.kv_heads * c.head_dim
+    new_k = rng.standard_normal((c.batch, row)).astype(np.float16)
+    new_v = rng.standard_normal((c.batch, row)).astype(np.float16)
+    nk_buf, nv_buf = exe.allocateScratchBuffer(new_k.nbytes), exe.allocateScratchBuffer(new_v.nbytes)
+    assert exe.uploadToBuffer(nk_buf, new_k) and exe.uploadToBuffer(nv_buf, new_v)
+    last = np.maximum(c.seq_lens.astype(np.int64) - 1, 0)
+    ids = np.array([c.page_tables_flat[c.page_table_offsets[r] + last[r] // c.page_size] if c.seq_lens[r] else 0
+                    for r in range(c.batch)], np.uint32)
+    slots = (last % c.page_size).astype(np.uint32)
+    n_w = max(1, min(args.steps, 500))
+    ms_w, wall_w = C.c_float(), C.c_double()
+    ok = bl.mlc_bench_decode_step_loop(
+        C.c_void_p(q_buf), kp, vp, C.c_size_t(n_layers), C.c_void_p(o_buf), C.c_void_p(nk_buf), C.c_void_p(nv_buf),
+        ids.ctypes.data_as(u32p), slots.ctypes.data_as(u32p),
+        meta[0].ctypes.data_as(u32p), C.c_size_t(meta[0].size), meta[1].ctypes.data_as(u32p),
+        meta[2].ctypes.data_as(u32p), meta[3].ctypes.data_as(u32p), C.c_size_t(c.batch),
+        C.c_size_t(c.num_heads), C.c_size_t(c.kv_heads), C.c_size_t(c.head_dim), C.c_size_t(c.page_size),
+        C.c_size_t(n_w), C.byref(ms_w), C.byref(wall_w))
+    if not ok:
+        raise RuntimeError("decode step loop failed: " + exe.lastError())
+    kv_write_us = wall_w.value / n_w * 1e6
+    # the pools now hold the new rows at the newest positions: the parity check below uses them
+    kv_after = {}
+    for name, pool, new in (("k", c.k_pages, new_k), ("v", c.v_pages, new_v)):
+        p2 = pool.copy().view(np.uint16).reshape(-1, c.page_size, row)
+        for r in range(c.batch):
+            if c.seq_lens[r]:
+                p2[ids[r], slots[r]] = new[r].view(np.uint16)
+        kv_after[name] = p2.reshape(-1)
+    c.k_pages, c.v_pages = kv_after["k"], kv_after["v"]
+
     out = np.empty(c.q.shape, np.float32)
     exe.beginForwardPassCB()
     step(0)
@@ -592,6 +627,7 @@ def main() -> int:
             "kernels_per_step": launches,
             "work_items": items,
             "us_per_layer_with_metadata_upload": round(boundary_us, 3),
+            "us_per_layer_with_kv_write": round(kv_write_us, 3),
         },
         "roofline": {
             "bound": "hbm",

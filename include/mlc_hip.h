@@ -259,6 +259,9 @@ float mlc_hip_timer_stop(void);
  * number of split-K work items it planned (for benchmarks and tests). */
 int mlc_hip_last_decode_launches(void);
 int mlc_hip_last_decode_work_items(void);
+/* Number of KV writes so far that went out fused with a neighbour: a batched K scatter with its
+ * V twin, or split + RoPE + cast with the scatters of its fp16 rows (for tests). */
+long mlc_hip_fused_kv_write_launches(void);
 /* Number of fused row-operator launches so far (for tests of "fuse_row_ops"). */
 long mlc_hip_row_program_launches(void);
 
@@ -277,7 +280,10 @@ long mlc_hip_row_program_launches(void);
  *                           (sum of matmul K slices, add, RMSNorm, gate/up SiLU, the fp16 split
  *                           of the next matmul's input) are collected and launched as one
  *                           kernel when something else is encoded, the pass is flushed or a
- *                           call has sync = 1; every output buffer is still written.
+ *                           call has sync = 1; every output buffer is still written.  The
+ *                           same holds for the KV write: split + RoPE + cast and the two
+ *                           batched scatters of its fp16 rows (or two batched scatters with
+ *                           the same page ids) become one launch.
  *                           0 = each operator is launched when it is encoded
  *   "prefill_stages"        2, 4, 6 or 8 K/V tiles staged in LDS by the prefill kernel (0 = automatic)
  * Returns 0 for an unknown name or value. */

@@ -130,6 +130,23 @@ struct Ctx {
         const void* cur = nullptr;   // buffer that will hold the chain's current values
         size_t grid_rows = 0;        // rows launched (padded to a multiple of 32 for the split stage)
     } rows;
+    // The KV write of a decode step that has been encoded but not launched: either the split +
+    // RoPE + cast (whose fp16 K / V rows the batched scatters that follow it consume: they join
+    // it, and the three become one launch), or a batched scatter waiting for its twin.
+    struct KvPending {
+        bool active = false;
+        bool rope = false;
+        RopeArgs a{};                       // rope form
+        const void* src[2] = {nullptr, nullptr};   // plain form: fp16 rows of the first / second scatter
+        void* pages[2] = {nullptr, nullptr};
+        int n = 0;
+        bool wide = false;                  // plain form: 16-byte units
+        std::vector<uint32_t> ids, slots;   // of the scatter(s) that joined so far
+        const uint32_t* d_ids = nullptr;
+        const uint32_t* d_slots = nullptr;
+        size_t batch = 0, row_elems = 0, page_size = 0;
+    } kv;
+    long kv_fused = 0;               // KV writes that went out fused with a neighbour (for tests)
     long opt_fuse_rows = 1;          // 0 = every operator is launched when it is encoded
     long row_launches = 0;           // row_program_kernel launches (for tests)
     MetaSlot plan_slots[4];
@@ -252,8 +269,41 @@ constexpr size_t kRowMaxLen = 16384;  // row_program_kernel: 8 groups of 8 eleme
 
 bool row_len_ok(size_t len) { return len > 0 && len % 8 == 0 && len <= kRowMaxLen; }
 
-// Launches what the pending chain holds.
+// Launches the pending KV write.
+int settle_kv() {
+    Ctx::KvPending& kv = g.kv;
+    if (!kv.active) return 1;
+    kv.active = false;
+    if (kv.rope) {
+        if (kv.a.k_pages || kv.a.v_pages) ++g.kv_fused;
+        launch_qkv_split_rope_cast(kv.a, g.stream);
+        HIP_OK(hipGetLastError());
+        return 1;
+    }
+    const unsigned block = 256;
+    const uint32_t row_units = (uint32_t)(kv.row_elems * 2 / (kv.wide ? 16 : 2));
+    const unsigned total = (unsigned)(kv.batch * row_units) * (unsigned)kv.n;
+    const dim3 grid((total + block - 1) / block);
+    if (kv.n == 2) ++g.kv_fused;
+    if (kv.wide)
+        hipLaunchKernelGGL(scatter_kv_pair_kernel<uint4>, grid, dim3(block), 0, g.stream,
+                           static_cast<const uint4*>(kv.src[0]), static_cast<uint4*>(kv.pages[0]),
+                           static_cast<const uint4*>(kv.src[1]), static_cast<uint4*>(kv.pages[1]), kv.d_ids,
+                           kv.d_slots, (uint32_t)kv.batch, row_units, (uint32_t)kv.page_size, (uint32_t)kv.n);
+    else
+        hipLaunchKernelGGL(scatter_kv_pair_kernel<uint16_t>, grid, dim3(block), 0, g.stream,
+                           static_cast<const uint16_t*>(kv.src[0]), static_cast<uint16_t*>(kv.pages[0]),
+                           static_cast<const uint16_t*>(kv.src[1]), static_cast<uint16_t*>(kv.pages[1]), kv.d_ids,
+                           kv.d_slots, (uint32_t)kv.batch, row_units, (uint32_t)kv.page_size, (uint32_t)kv.n);
+    HIP_OK(hipGetLastError());
+    return 1;
+}
+
+// Launches what is pending, in the order it was encoded: a pending KV write is always older
+// than a pending chain (whatever starts the KV write launches the chain first, and a scatter
+// only joins while no chain is pending).
 int settle() {
+    if (!settle_kv()) return 0;
     Ctx::RowPending& r = g.rows;
     if (!r.active) return 1;
     r.active = false;
@@ -765,7 +815,6 @@ int mlc_hip_scatter_kv_paged_batched_f16(void* page_storage, const uint32_t* pag
                                          size_t n_kv_heads, size_t head_dim, size_t batch,
                                          const void* src, int sync) {
     if (!init_once()) return fail("GPU unavailable");
-    if (!settle()) return 0;
     if (!sync && !g.pass_open) return fail("encode: no open forward pass");  // :7178
     // metal_runtime.mm:7241-7243
     if (!page_storage || !src) return fail("scatter: null buffer");
@@ -786,28 +835,59 @@ int mlc_hip_scatter_kv_paged_batched_f16(void* page_storage, const uint32_t* pag
     const size_t known_src = known_bytes(src);
     if (known_src && batch * row_bytes > known_src) return fail("scatter: src too small");
 
+    const bool wide = (row_bytes % 16) == 0 && aligned16(page_storage) && aligned16(src);
+    Ctx::KvPending& kv = g.kv;
+    // ---- does this scatter complete a pending KV write?  (only while nothing younger is pending)
+    if (g.opt_fuse_rows && kv.active && !g.rows.active && kv.batch == batch && kv.row_elems == row_bytes / 2 &&
+        (kv.ids.empty() || (kv.page_size == page_size_tokens &&
+                            std::memcmp(kv.ids.data(), page_ids, batch * 4) == 0 &&
+                            std::memcmp(kv.slots.data(), slots_in_page, batch * 4) == 0))) {
+        bool joined = false;
+        if (kv.rope) {
+            const bool as_k = src == kv.a.k_f16 && !kv.a.k_pages && kv.a.k_rows == row_bytes / 2;
+            const bool as_v = !as_k && src == kv.a.v_f16 && !kv.a.v_pages && kv.a.v_rows == row_bytes / 2;
+            if ((as_k || as_v) && (reinterpret_cast<uintptr_t>(page_storage) & 3u) == 0) {
+                if (kv.ids.empty()) {
+                    const size_t ids_bytes = align_up(batch * 4, 16);
+                    const char* blob = static_cast<const char*>(resident_ids(page_ids, slots_in_page, batch, ids_bytes));
+                    if (!blob) return 0;
+                    kv.a.page_ids = reinterpret_cast<const uint32_t*>(blob);
+                    kv.a.slots = reinterpret_cast<const uint32_t*>(blob + ids_bytes);
+                    kv.a.page_size = (uint32_t)page_size_tokens;
+                    kv.page_size = page_size_tokens;
+                    kv.ids.assign(page_ids, page_ids + batch);
+                    kv.slots.assign(slots_in_page, slots_in_page + batch);
+                }
+                (as_k ? kv.a.k_pages : kv.a.v_pages) = static_cast<_Float16*>(page_storage);
+                joined = true;
+            }
+        } else if (kv.n == 1 && kv.wide == wide && page_storage != kv.pages[0]) {
+            kv.src[1] = src;
+            kv.pages[1] = page_storage;
+            kv.n = 2;
+            joined = true;
+        }
+        if (joined) return finish(sync);
+    }
+    if (!settle()) return 0;
+
     const size_t ids_bytes = align_up(batch * 4, 16);
     const char* d_blob = static_cast<const char*>(resident_ids(page_ids, slots_in_page, batch, ids_bytes));
     if (!d_blob) return 0;
-    const uint32_t* d_ids = reinterpret_cast<const uint32_t*>(d_blob);
-    const uint32_t* d_slots = reinterpret_cast<const uint32_t*>(d_blob + ids_bytes);
-
-    const unsigned block = 256;
-    if ((row_bytes % 16) == 0 && aligned16(page_storage) && aligned16(src)) {
-        const uint32_t row_units = (uint32_t)(row_bytes / 16);
-        const unsigned total = (unsigned)(batch * row_units);
-        hipLaunchKernelGGL(scatter_kv_paged_batched_kernel<uint4>, dim3((total + block - 1) / block),
-                           dim3(block), 0, g.stream, static_cast<const uint4*>(src),
-                           static_cast<uint4*>(page_storage), d_ids, d_slots, (uint32_t)batch,
-                           row_units, (uint32_t)page_size_tokens);
-    } else {
-        const uint32_t row_units = (uint32_t)(row_bytes / 2);
-        const unsigned total = (unsigned)(batch * row_units);
-        hipLaunchKernelGGL(scatter_kv_paged_batched_kernel<uint16_t>,
-                           dim3((total + block - 1) / block), dim3(block), 0, g.stream,
-                           static_cast<const uint16_t*>(src), static_cast<uint16_t*>(page_storage),
-                           d_ids, d_slots, (uint32_t)batch, row_units, (uint32_t)page_size_tokens);
-    }
+    kv = Ctx::KvPending{};
+    kv.active = true;
+    kv.src[0] = src;
+    kv.pages[0] = page_storage;
+    kv.n = 1;
+    kv.wide = wide;
+    kv.ids.assign(page_ids, page_ids + batch);
+    kv.slots.assign(slots_in_page, slots_in_page + batch);
+    kv.d_ids = reinterpret_cast<const uint32_t*>(d_blob);
+    kv.d_slots = reinterpret_cast<const uint32_t*>(d_blob + ids_bytes);
+    kv.batch = batch;
+    kv.row_elems = row_bytes / 2;
+    kv.page_size = page_size_tokens;
+    if (!g.opt_fuse_rows && !settle_kv()) return 0;  // no deferral: launched as encoded
     return finish(sync);
 }
 
@@ -986,7 +1066,15 @@ int mlc_hip_qkv_split_rope_cast(const void* qkv, void* q, void* k, void* v, void
     a.batch = (uint32_t)batch; a.head_dim = (uint32_t)head_dim; a.qkv_rows = (uint32_t)qkv_rows;
     a.q_rows = (uint32_t)q_rows; a.k_rows = (uint32_t)k_rows; a.v_rows = (uint32_t)v_rows;
     a.rotary_dim = (uint32_t)rotary_dim; a.page_size = 0;
-    launch_qkv_split_rope_cast<false>(a, g.stream);
+    // held back: the batched scatters of k_f16 / v_f16 that usually follow join this launch
+    Ctx::KvPending& kv = g.kv;
+    kv = Ctx::KvPending{};
+    kv.active = true;
+    kv.rope = true;
+    kv.a = a;
+    kv.batch = batch;
+    kv.row_elems = k_rows;
+    if (!g.opt_fuse_rows && !settle_kv()) return 0;
     return finish(sync);
 }
 
@@ -1034,7 +1122,7 @@ int mlc_hip_qkv_split_rope_scatter(const void* qkv, void* q, void* k_pages, void
     a.batch = (uint32_t)batch; a.head_dim = (uint32_t)head_dim; a.qkv_rows = (uint32_t)qkv_rows;
     a.q_rows = (uint32_t)q_rows; a.k_rows = (uint32_t)k_rows; a.v_rows = (uint32_t)v_rows;
     a.rotary_dim = (uint32_t)rotary_dim; a.page_size = (uint32_t)page_size_tokens;
-    launch_qkv_split_rope_cast<true>(a, g.stream);
+    launch_qkv_split_rope_cast(a, g.stream);
     return finish(sync);
 }
 
@@ -1541,6 +1629,7 @@ float mlc_hip_timer_stop(void) {
 
 int mlc_hip_last_decode_launches(void) { return g.last_launches; }
 int mlc_hip_last_decode_work_items(void) { return g.last_items; }
+long mlc_hip_fused_kv_write_launches(void) { return g.kv_fused; }
 long mlc_hip_row_program_launches(void) { return g.row_launches; }
 
 int mlc_hip_set_option(const char* name, long value) {

@@ -30,6 +30,27 @@ __global__ void scatter_kv_paged_batched_kernel(const UnitT* __restrict__ src,
     page_storage[dst_row * row_units + u] = src[gid];
 }
 
+// The K row and the V row of a decode step in one launch: two scatter_kv_paged_batched copies
+// with the same (page id, slot) per request.  The batched step encodes them back to back
+// (compiler/runtime/batched_walker.cpp:304-307); each on its own costs a launch for 32 KiB.
+template <typename UnitT>
+__global__ void scatter_kv_pair_kernel(const UnitT* __restrict__ src0, UnitT* __restrict__ pages0,
+                                       const UnitT* __restrict__ src1, UnitT* __restrict__ pages1,
+                                       const uint32_t* __restrict__ page_ids,
+                                       const uint32_t* __restrict__ slots, uint32_t batch,
+                                       uint32_t row_units, uint32_t page_size, uint32_t n_tensors) {
+    // n_tensors = 1: only the first copy exists (src1 / pages1 are null and must not be touched)
+    const uint32_t gid = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t per = batch * row_units;
+    if (gid >= n_tensors * per) return;
+    const uint32_t which = gid / per, e = gid - which * per;
+    const uint32_t req = e / row_units;
+    const uint32_t u = e - req * row_units;
+    const size_t dst_row = (size_t)page_ids[req] * page_size + slots[req];
+    if (which == 0) pages0[dst_row * row_units + u] = src0[e];
+    else pages1[dst_row * row_units + u] = src1[e];
+}
+
 // MSL scatter_kv_paged_f16/f32 (metal_runtime.mm:468-512): src is
 // [kv][token][dim]; token t goes to absolute slot start_slot + t of the page
 // table.  One thread per UNIT of a (kv, token) row of head_dim elements.

@@ -24,14 +24,14 @@ struct RopeArgs {
     float* q;                // [batch][q_rows]            (never null)
     float* k;                // [batch][k_rows] fp32       (may be null in the fused form)
     float* v;                // [batch][v_rows] fp32       (may be null in the fused form)
-    _Float16* k_f16;         // [batch][k_rows]            (unfused form)
+    _Float16* k_f16;         // [batch][k_rows]            (may be null: no fp16 staging copy)
     _Float16* v_f16;         // [batch][v_rows]
-    _Float16* k_pages;       // fused form: KV pools [page][slot][kv_head][dim]
+    _Float16* k_pages;       // KV pools [page][slot][kv_head][dim] (may be null: no paged write)
     _Float16* v_pages;
     const float* cos_table;  // [batch][rotary_dim / 2]
     const float* sin_table;
-    const uint32_t* page_ids;  // fused form: [batch]
-    const uint32_t* slots;     // fused form: [batch]
+    const uint32_t* page_ids;  // [batch], needed when k_pages or v_pages is set
+    const uint32_t* slots;     // [batch]
     uint32_t batch, head_dim, qkv_rows, q_rows, k_rows, v_rows, rotary_dim, page_size;
 };
 
@@ -44,8 +44,8 @@ __device__ __forceinline__ float2 rope_rotate(float2 x, float c, float s) {
 }
 
 // One thread per pair.  Pair index pi of a request counts pairs of the q, then k, then v
-// segment (every segment length is even on this path).
-template <bool SCATTER>
+// segment (every segment length is even on this path).  Which of the k / v outputs exist
+// (fp32 copy, fp16 staging copy, paged write) is decided per launch by the pointers.
 __global__ __launch_bounds__(256) void qkv_split_rope_cast_kernel(const RopeArgs a) {
     const uint32_t pairs_row = (a.q_rows + a.k_rows + a.v_rows) / 2;
     const uint32_t gid = blockIdx.x * blockDim.x + threadIdx.x;
@@ -73,23 +73,20 @@ __global__ __launch_bounds__(256) void qkv_split_rope_cast_kernel(const RopeArgs
     if (f32) *reinterpret_cast<float2*>(f32 + (size_t)req * rows + local) = y;
     typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
     const half2_t h = {(_Float16)y.x, (_Float16)y.y};
-    if (SCATTER) {
+    _Float16* f16 = is_k ? a.k_f16 : a.v_f16;
+    if (f16) *reinterpret_cast<half2_t*>(f16 + (size_t)req * rows + local) = h;
+    _Float16* pool = is_k ? a.k_pages : a.v_pages;
+    if (pool) {
         // scatter_kv_paged_batched_f16 (metal_runtime.mm:418-422): a row of all KV heads is
         // contiguous at page_ids[r]*P*rows + slots[r]*rows
-        _Float16* pool = is_k ? a.k_pages : a.v_pages;
         const size_t dst = ((size_t)a.page_ids[req] * a.page_size + a.slots[req]) * rows + local;
         *reinterpret_cast<half2_t*>(pool + dst) = h;
-    } else {
-        _Float16* f16 = is_k ? a.k_f16 : a.v_f16;
-        *reinterpret_cast<half2_t*>(f16 + (size_t)req * rows + local) = h;
     }
 }
 
-template <bool SCATTER>
 inline void launch_qkv_split_rope_cast(const RopeArgs& a, hipStream_t stream) {
     const uint32_t total = a.batch * ((a.q_rows + a.k_rows + a.v_rows) / 2);
-    hipLaunchKernelGGL((qkv_split_rope_cast_kernel<SCATTER>), dim3((total + 255) / 256), dim3(256), 0,
-                       stream, a);
+    hipLaunchKernelGGL(qkv_split_rope_cast_kernel, dim3((total + 255) / 256), dim3(256), 0, stream, a);
 }
 
 }  // namespace mlc_hip

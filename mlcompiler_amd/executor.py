@@ -251,6 +251,10 @@ class HipExecutor:
     def lastDecodeWorkItems(self) -> int:
         return int(self._lib.mlc_hip_last_decode_work_items())
 
+    def fusedKvWriteLaunches(self) -> int:
+        """KV writes so far that went out fused with a neighbour (option "fuse_row_ops")."""
+        return int(self._lib.mlc_hip_fused_kv_write_launches())
+
     def rowProgramLaunches(self) -> int:
         """Fused row-operator launches so far (option "fuse_row_ops")."""
         return int(self._lib.mlc_hip_row_program_launches())

@@ -255,3 +255,97 @@ def test_cached_buffers_and_offsets(exe):
     assert exe.downloadFromBuffer(b, back, src_offset=1024 + 64 * 4)
     assert np.array_equal(back, data[64:128])
     assert not exe.uploadToBuffer(b, data, dst_offset=4096)   # beyond the buffer
+
+
+# ---- the KV write of a step encoded call by call goes out as one launch: same bytes --------------
+
+@pytest.mark.parametrize("B,Hkv,D,P", [(32, 4, 64, 64), (5, 2, 64, 4), (7, 3, 20, 8)])
+@pytest.mark.parametrize("fuse", [1, 0])
+def test_k_and_v_scatter_pair_in_one_pass(exe, B, Hkv, D, P, fuse):
+    """encodeScatterKVPagedBatched for K, then for V with the same page ids (the two calls of
+    batched_walker.cpp:304-307): one launch with fusion on; a third scatter with other ids, and a
+    scatter into the pool the first one wrote, must not join."""
+    print(f"[scatter pair] B={B} Hkv={Hkv} D={D} P={P} fuse={fuse}", flush=True)
+    rng = np.random.default_rng(B + D)
+    cap = 2 * B + 4
+    n = cap * P * Hkv * D
+    k_pool, v_pool = (rng.integers(0, 65536, n, dtype=np.uint16) for _ in range(2))
+    nk, nv, nk2 = (rng.integers(0, 65536, B * Hkv * D, dtype=np.uint16) for _ in range(3))
+    ids = rng.permutation(cap)[:B].astype(np.uint32)
+    slots = rng.integers(0, P, B).astype(np.uint32)
+    ids2 = ((ids + 1) % cap).astype(np.uint32)
+    want_k, want_v = k_pool.copy(), v_pool.copy()
+    assert po.scatter_kv_paged_batched_f16(want_k, ids, slots, P, Hkv, D, B, nk)
+    assert po.scatter_kv_paged_batched_f16(want_v, ids, slots, P, Hkv, D, B, nv)
+    assert po.scatter_kv_paged_batched_f16(want_k, ids2, slots, P, Hkv, D, B, nk2)   # third call
+    assert po.scatter_kv_paged_batched_f16(want_k, ids2, slots, P, Hkv, D, B, nv)    # fourth: same pool again
+    bufs = [_pool(exe, a) for a in (k_pool, v_pool, nk, nv, nk2)]
+    d_k, d_v, d_nk, d_nv, d_nk2 = bufs
+    assert exe.setOption("fuse_row_ops", fuse)
+    before = exe.fusedKvWriteLaunches()
+    try:
+        assert exe.beginForwardPassCB()
+        assert exe.encodeScatterKVPagedBatched(d_k, ids, slots, P, Hkv, D, B, d_nk)
+        assert exe.encodeScatterKVPagedBatched(d_v, ids, slots, P, Hkv, D, B, d_nv)     # joins
+        assert exe.encodeScatterKVPagedBatched(d_k, ids2, slots, P, Hkv, D, B, d_nk2)   # other ids: on its own
+        assert exe.encodeScatterKVPagedBatched(d_k, ids2, slots, P, Hkv, D, B, d_nv)    # same pool: on its own, later
+        assert exe.flushForwardPassCB(), exe.lastError()
+        got_k, got_v = _read(exe, d_k, k_pool), _read(exe, d_v, v_pool)
+    finally:
+        exe.setOption("fuse_row_ops", 1)
+        for b in bufs:
+            exe.releaseScratchBuffer(b)
+    assert np.array_equal(got_k, want_k) and np.array_equal(got_v, want_v)
+    assert exe.fusedKvWriteLaunches() - before == (1 if fuse else 0)
+
+
+@pytest.mark.parametrize("fuse", [1, 0])
+@pytest.mark.parametrize("only_k", [False, True])
+def test_rope_cast_then_scatters_in_one_pass(exe, fuse, only_k):
+    """encodeQkvSplitRopeCast, then the batched scatters of its fp16 K and V rows
+    (batched_walker.cpp:287-307): one launch with fusion on, every buffer of the three calls
+    written, bit-identical to the calls on their own."""
+    B, H, Hkv, D, P = 9, 8, 2, 64, 16
+    q_rows, kv_rows = H * D, Hkv * D
+    qkv_rows = q_rows + 2 * kv_rows
+    rng = np.random.default_rng(31 + only_k)
+    qkv = rng.standard_normal((B, qkv_rows)).astype(np.float32)
+    pos = rng.integers(0, 500, B)
+    cos = np.zeros((B, D // 2), np.float32)
+    sin = np.zeros((B, D // 2), np.float32)
+    for r in range(B):
+        cos[r], sin[r] = po.rotary_coefficients(int(pos[r]), D)
+    cap = 2 * B
+    k_pool, v_pool = (rng.integers(0, 65536, cap * P * kv_rows, dtype=np.uint16) for _ in range(2))
+    ids = rng.permutation(cap)[:B].astype(np.uint32)
+    slots = rng.integers(0, P, B).astype(np.uint32)
+    wq, wk, wv, wk16, wv16 = po.qkv_split_rope_cast(qkv, cos, sin, B, H, Hkv, D, qkv_rows, q_rows, kv_rows, kv_rows, D)
+    want_k, want_v = k_pool.copy(), v_pool.copy()
+    assert po.scatter_kv_paged_batched_f16(want_k, ids, slots, P, Hkv, D, B, wk16)
+    if not only_k:
+        assert po.scatter_kv_paged_batched_f16(want_v, ids, slots, P, Hkv, D, B, wv16)
+    d_qkv, d_cos, d_sin, d_kp, d_vp = (_pool(exe, a) for a in (qkv, cos, sin, k_pool, v_pool))
+    d_q = exe.allocateScratchBuffer(B * q_rows * 4)
+    d_k, d_v = (exe.allocateScratchBuffer(B * kv_rows * 4) for _ in range(2))
+    d_k16, d_v16 = (exe.allocateScratchBuffer(B * kv_rows * 2) for _ in range(2))
+    bufs = [d_qkv, d_cos, d_sin, d_kp, d_vp, d_q, d_k, d_v, d_k16, d_v16]
+    assert exe.setOption("fuse_row_ops", fuse)
+    before = exe.fusedKvWriteLaunches()
+    try:
+        assert exe.beginForwardPassCB()
+        assert exe.encodeQkvSplitRopeCast(d_qkv, d_q, d_k, d_v, d_k16, d_v16, d_cos, d_sin, B, H, Hkv, D, qkv_rows,
+                                          q_rows, kv_rows, kv_rows, D), exe.lastError()
+        assert exe.encodeScatterKVPagedBatched(d_kp, ids, slots, P, Hkv, D, B, d_k16)
+        if not only_k:
+            assert exe.encodeScatterKVPagedBatched(d_vp, ids, slots, P, Hkv, D, B, d_v16)
+        assert exe.flushForwardPassCB(), exe.lastError()
+        got = {n: _read(exe, b, like) for n, b, like in
+               (("q", d_q, wq), ("k", d_k, wk), ("v", d_v, wv), ("k16", d_k16, wk16), ("v16", d_v16, wv16),
+                ("kp", d_kp, k_pool), ("vp", d_vp, v_pool))}
+    finally:
+        exe.setOption("fuse_row_ops", 1)
+        for b in bufs:
+            exe.releaseScratchBuffer(b)
+    for name, want in (("q", wq), ("k", wk), ("v", wv), ("k16", wk16), ("v16", wv16), ("kp", want_k), ("vp", want_v)):
+        assert np.array_equal(got[name].view(np.uint8), np.ascontiguousarray(want).view(np.uint8)), name
+    assert exe.fusedKvWriteLaunches() - before == (1 if fuse else 0)
