@@ -599,7 +599,7 @@ def main() -> int:
 
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs),
     # scaled by the copy-kernel calibration (x2.0 / x1.0); valid for the default planner only.
-    measured_traffic = {"cfg2": 44_220_000, "cfg3": 142_580_000, "cfg4": 1_191_200_000}
+    measured_traffic = {"cfg2": 44_220_000, "cfg3": 142_580_000, "cfg4": 1_203_400_000}
     traffic = measured_traffic.get(args.workload) if not args.target_items else None
 
     result = {

@@ -431,11 +431,11 @@ int build_plan(const uint32_t* flat, size_t n_flat, const uint32_t* off, const u
     const size_t G = H / Hkv;
     if (p.fast) {
         // query heads per wave (power of two dividing G), waves per workgroup = G / that
-        // Chosen by sweep on MI355X: wide GQA groups (8 query heads per KV head) run fastest
-        // spread over four waves of 2 heads each (more waves to hide the latency of short
-        // items); narrower groups keep 4 heads per wave, which shares the per-tile softmax
-        // and packing work over more heads.
-        const long hpw_cap = g.opt_hpw_max > 0 ? g.opt_hpw_max : (G >= 8 ? 2 : 4);
+        // Chosen by sweep on MI355X: a query-head group runs fastest spread over four waves
+        // (G / 4 heads each; one head per wave for groups of 4 and fewer): more waves hide the
+        // latency of the tile loads and of short items better than sharing the per-tile softmax
+        // and packing work over more heads saves.
+        const long hpw_cap = g.opt_hpw_max > 0 ? g.opt_hpw_max : std::max<long>(1, (long)G / 4);
         int hpw = 8;
         while (hpw > 1 && (hpw > hpw_cap || (G % (size_t)hpw) != 0)) hpw >>= 1;
         size_t nw = G / (size_t)hpw;
@@ -479,7 +479,7 @@ int build_plan(const uint32_t* flat, size_t n_flat, const uint32_t* off, const u
         // Short items cannot use a second buffer; one buffer lets twice the workgroups
         // share a CU and hide each other's memory latency.
         if (g.opt_buffers == 0) p.nbuf = (chunk >= 4 * (size_t)p.ns) ? 2 : 1;
-        for (size_t r = 0; r < B; ++r) {  // the merge pass handles at most kMaxSplits partials
+        for (size_t r = 0; r < B; ++r) {  // the merge handles at most kMaxSplits partials
             const size_t tiles_r = (limits[r] + tile - 1) / tile;
             chunk = std::max(chunk, (tiles_r + kMaxSplits - 1) / kMaxSplits);
         }
@@ -488,12 +488,21 @@ int build_plan(const uint32_t* flat, size_t n_flat, const uint32_t* off, const u
             const size_t ns = std::max<size_t>(1, (tiles_r + chunk - 1) / chunk);
             const size_t per = (tiles_r + ns - 1) / ns;
             size_t ns_eff = tiles_r == 0 ? 1 : (tiles_r + per - 1) / per;
-            if (ns_eff > 0xFFFF) return fail("decode: too many splits");
+            if (ns_eff > kMaxSplits) return fail("decode: too many splits");
+            // Many splits are merged in two levels: groups of about sqrt(splits), a multiple of
+            // the eight partials one round of the merge loads, then the groups' results, which
+            // take n_groups more partial slots (and their arrival counters) behind the splits.
+            size_t group_size = 0, n_groups = 0;
+            if (ns_eff > kFlatMergeSplits) {
+                group_size = 8;
+                while (group_size * group_size < ns_eff) group_size += 8;
+                n_groups = (ns_eff + group_size - 1) / group_size;
+            }
             for (size_t kvh = 0; kvh < Hkv; ++kvh) {
                 uint32_t first_part = kNoPartial;
                 if (ns_eff > 1) {
                     first_part = p.n_part;
-                    p.n_part += (uint32_t)ns_eff;
+                    p.n_part += (uint32_t)(ns_eff + n_groups);
                 }
                 for (size_t s = 0; s < ns_eff; ++s) {
                     DecodeWorkItem it;
@@ -508,7 +517,7 @@ int build_plan(const uint32_t* flat, size_t n_flat, const uint32_t* off, const u
                         const size_t tok = (size_t)it.tok_begin + i * tile;
                         it.first_pages[i] = tok < it.tok_end ? flat[off[r] + tok / P] : 0u;
                     }
-                    it.pad = 0;
+                    it.group_size = (uint32_t)group_size;
                     items.push_back(it);
                 }
             }

@@ -53,11 +53,14 @@ struct DecodeWorkItem {
     uint32_t split;       // this item's split index | number of splits << 16
     uint32_t first_pages[4];  // page ids of the item's first four tiles: the first tile loads
                               // then depend on the item alone, not on a page-table fetch
-    uint32_t pad;
+    uint32_t group_size;  // 0: the last arriver merges all splits; otherwise the splits are
+                          // merged in groups of this many, and the groups' results after them
 };
 static_assert(sizeof(DecodeWorkItem) == 48, "work items are uploaded as raw bytes");
 static constexpr uint32_t kNoPartial = 0xFFFFFFFFu;
-static constexpr uint32_t kMaxSplits = 64;  // partial states merged by one wave pass
+static constexpr uint32_t kMaxSplits = 512;      // per (request, KV head)
+static constexpr uint32_t kFlatMergeSplits = 16;  // up to here one wave merges all partials;
+                                                  // beyond, in two levels (each merge <= 64)
 
 struct DecodeArgs {
     const float* q;             // [B][H][D]
@@ -178,7 +181,7 @@ __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const D
     // The item is read once, into scalar registers: any vector load issued after the tile
     // loads would have to wait for them (loads return in order).
     struct {
-        uint32_t req, kv_head, pt_base, tok_begin, tok_end, part_first, split, pg[4];
+        uint32_t req, kv_head, pt_base, tok_begin, tok_end, part_first, split, pg[4], group_size;
     } it;
     {
         const DecodeWorkItem* gi = a.items + item_idx;
@@ -189,6 +192,7 @@ __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const D
         it.tok_end = __builtin_amdgcn_readfirstlane(gi->tok_end);
         it.part_first = __builtin_amdgcn_readfirstlane(gi->part_first);
         it.split = __builtin_amdgcn_readfirstlane(gi->split);
+        it.group_size = __builtin_amdgcn_readfirstlane(gi->group_size);
 #pragma unroll
         for (int i = 0; i < 4; ++i) it.pg[i] = __builtin_amdgcn_readfirstlane(gi->first_pages[i]);
     }
@@ -559,6 +563,122 @@ __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const D
             const float l = l_all[k / HPK];
             const float inv = l > 0.f ? 1.0f / l : 0.f;
             a.o[((size_t)it.req * a.num_heads + head0) * D + k * 64 + lane] = o_un[k] * inv;
+        }
+        return;
+    }
+
+    if (it.group_size != 0) {
+        // Many splits: groups of group_size partials are merged by their own last arrivers
+        // into the n_groups slots behind the request's partials, and the last of those merges
+        // the groups' results.  (Kept apart from the common case below, whose code is laid out
+        // for the shortest path through publish, ticket and merge.)
+        const uint32_t n_splits = it.split >> 16;
+        const uint32_t my_split = it.split & 0xFFFFu;
+        // Partial state of this wave's heads -> slot `slot`: unnormalised o, running max m, sum l.
+        auto publish = [&](size_t slot, const float (&o)[OPL], const float (&m)[HPW],
+                           const float (&l)[HPW]) __attribute__((always_inline)) {
+            float* po = a.part_o + (slot * G + hg * HPW) * D;
+            float* ml = a.part_ml + (slot * G + hg * HPW) * 2;
+#pragma unroll
+            for (int k = 0; k < OPL; ++k) st_dev(po + k * 64 + lane, o[k]);
+            if (lane < HPW) {
+                float mh = m[0], lh = l[0];
+#pragma unroll
+                for (int hh = 1; hh < HPW; ++hh) {
+                    mh = (lane == hh) ? m[hh] : mh;
+                    lh = (lane == hh) ? l[hh] : lh;
+                }
+                st_dev(ml + lane * 2, mh);
+                st_dev(ml + lane * 2 + 1, lh);
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // stores complete (vmcnt 0)
+        };
+        // Bumps the arrival counter of slot `slot`; true for the last of `expected` arrivers, which
+        // also puts the counter back to zero for the next launch.
+        auto last_arriver = [&](size_t slot, uint32_t expected) __attribute__((always_inline)) {
+            uint32_t ticket = 0;
+            uint32_t* counter = &a.counters[slot * NW + hg];
+            if (lane == 0)
+                ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            ticket = __shfl(ticket, 0);
+            if (ticket != expected - 1) return false;
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+            if (lane == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return true;
+        };
+        // Merges the `count` (<= 64) partials from slot `first` on.  Lane s holds the (m, l) of
+        // partial s for every head; all loads of a round are issued before any is consumed, so
+        // eight partials cost about one memory round trip.
+        auto merge = [&](size_t first, uint32_t count, float (&acc_o)[OPL], float (&m_fin)[HPW],
+                         float (&l_fin)[HPW]) __attribute__((always_inline)) {
+            const float* ml_base = a.part_ml + (first * G + hg * HPW) * 2;
+            const float* po_base = a.part_o + (first * G + hg * HPW) * D;
+            float ms[HPW], ls[HPW];
+#pragma unroll
+            for (int h = 0; h < HPW; ++h) {
+                ms[h] = kNegBig;
+                ls[h] = 0.f;
+                if ((uint32_t)lane < count) {
+                    ms[h] = ld_dev(ml_base + ((size_t)lane * G + h) * 2);
+                    ls[h] = ld_dev(ml_base + ((size_t)lane * G + h) * 2 + 1);
+                }
+            }
+            constexpr int UNR = 8;
+#pragma unroll
+            for (int k = 0; k < OPL; ++k) acc_o[k] = 0.f;
+            float wgt[HPW];
+            bool have_w = false;
+            for (uint32_t s0 = 0; s0 < count; s0 += UNR) {
+                float pv[UNR][OPL];
+#pragma unroll
+                for (int u = 0; u < UNR; ++u) {
+#pragma unroll
+                    for (int k = 0; k < OPL; ++k) {
+                        pv[u][k] = 0.f;
+                        if (s0 + u < count) pv[u][k] = ld_dev(po_base + (size_t)(s0 + u) * G * D + k * 64 + lane);
+                    }
+                }
+                if (!have_w) {
+#pragma unroll
+                    for (int h = 0; h < HPW; ++h) {
+                        m_fin[h] = wave_max(ms[h]);
+                        wgt[h] = fast_exp2(ms[h] - m_fin[h]);  // lanes >= count: exp2(-1e30 - m) = 0
+                        l_fin[h] = wave_sum(wgt[h] * ls[h]);
+                    }
+                    have_w = true;
+                }
+#pragma unroll
+                for (int u = 0; u < UNR; ++u) {
+                    if (s0 + u < count) {
+#pragma unroll
+                        for (int k = 0; k < OPL; ++k)
+                            acc_o[k] += __shfl(wgt[k / HPK], (int)(s0 + u)) * pv[u][k];
+                    }
+                }
+            }
+        };
+
+        const uint32_t gs = it.group_size;
+        const uint32_t group = my_split / gs;
+        float acc_o[OPL], m_fin[HPW], l_fin[HPW];
+        publish((size_t)it.part_first + my_split, o_un, m_all, l_all);
+        size_t first = (size_t)it.part_first + (size_t)group * gs;
+        uint32_t count = min(gs, n_splits - group * gs);
+        uint32_t groups_left = (n_splits + gs - 1) / gs;
+        for (;;) {
+            if (!last_arriver(first, count)) return;
+            merge(first, count, acc_o, m_fin, l_fin);
+            if (groups_left == 0) break;
+            first = (size_t)it.part_first + n_splits;
+            count = groups_left;
+            groups_left = 0;
+            publish(first + group, acc_o, m_fin, l_fin);
+        }
+#pragma unroll
+        for (int k = 0; k < OPL; ++k) {
+            const float l = l_fin[k / HPK];
+            const float inv = l > 0.f ? 1.0f / l : 0.f;
+            a.o[((size_t)it.req * a.num_heads + head0) * D + k * 64 + lane] = acc_o[k] * inv;
         }
         return;
     }

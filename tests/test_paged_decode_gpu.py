@@ -152,6 +152,34 @@ def test_split_k_targets_agree(exe):
     assert np.max(np.abs(outs[0] - outs[2])) < 3e-4, np.max(np.abs(outs[0] - outs[2]))
 
 
+@pytest.mark.parametrize("shape", [(32, 8, 128, [8192 + 17, 3001]), (32, 4, 64, [5000, 1100, 70]),
+                                   (8, 8, 64, [16384 + 1])],
+                         ids=["d128", "d64", "mha"])
+def test_many_splits_merge_in_two_levels(exe, shape):
+    """Few long requests: each (request, KV head) is cut into far more than the 16 partials one
+    wave merges at once, so groups of partials are merged first and the groups' results after
+    them (also with a last group of one partial).  Planned automatically, with one tile per item,
+    and as one item per (request, KV head); repeated, because the arrival counters must be
+    back at zero after every launch."""
+    heads, kv_heads, dim, lens = shape
+    case = make_case("long", len(lens), heads, kv_heads, dim, 64, lens, seed=11)
+    want = oracle_decode(case)
+    dev = DeviceCase(exe, case)
+    outs = {}
+    try:
+        for target in (0, 1000000, 1):
+            assert exe.setOption("decode_target_items", target)
+            for rep in range(2):
+                got = dev.run()
+                print("target", target, "items", exe.lastDecodeWorkItems(), flush=True)
+                assert_parity(got, want, dim, f"target={target} rep={rep}")
+            outs[target] = got
+    finally:
+        exe.setOption("decode_target_items", 0)
+        dev.free()
+    assert np.max(np.abs(outs[1000000] - outs[1])) < 1e-3
+
+
 def test_generic_kernel_agrees_with_fast(exe):
     case = baseline_config(2, batch=4)
     dev = DeviceCase(exe, case)
