@@ -261,6 +261,23 @@ def bench_layer(args) -> int:
                            VOCAB, head_norm, w_head)
     ev_ms, wall = loop(args.steps)
     host_encode_us = enqueue_s.value / args.steps * 1e6
+    graph_us = graph_nodes = None
+    if args.graph:   # the same n_layers launches captured once into a HIP graph and replayed
+        g_ms, g_nodes = C.c_float(), C.c_size_t()
+        replays = max(1, args.steps // n_layers)
+        loop(n_layers)                   # the same pass launched call by call: the replays must reproduce it
+        eager_out = np.empty((B, lc.HID), np.float32)
+        exe.downloadFromBuffer(L.out2, eager_out)
+        rc = bl.mlc_bench_layer_loop_graph(C.byref(L), kp, vp, C.c_size_t(n_layers), C.c_size_t(replays),
+                                           C.byref(g_ms), C.byref(g_nodes))
+        if rc == 0:
+            raise RuntimeError("graph replay of the layer loop failed: " + exe.lastError())
+        graph_nodes = g_nodes.value
+        replay_out = np.empty((B, lc.HID), np.float32)
+        exe.downloadFromBuffer(L.out2, replay_out)
+        if rc == 1 and not np.array_equal(eager_out, replay_out):
+            raise RuntimeError("graph replays of the layer loop differ from the eager pass")
+        graph_us = round(g_ms.value / (replays * n_layers) * 1e3, 2) if rc == 1 else "captured pass holds non-kernel nodes"
     L.out2 = None
     loop(1)                              # one step from the known input, for the parity check
     out = np.empty((B, lc.HID), np.float32)
@@ -288,6 +305,7 @@ def bench_layer(args) -> int:
             "us_per_layer": round(us, 2),
             "host_encode_us_per_layer": round(host_encode_us, 2),
             "tokens_per_s_at_22_layers": round(B / (22 * us * 1e-6), 1),
+            **({"us_per_layer_graph_replay": graph_us, "graph_nodes": graph_nodes} if args.graph else {}),
         },
         "roofline": {"bound": "hbm", "achieved": round(ach, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None,
@@ -458,6 +476,8 @@ def main() -> int:
     ap.add_argument("--target-items", type=int, default=0)
     ap.add_argument("--prefill-stages", type=int, default=0, help="cfg5: LDS pipeline depth (0 = automatic)")
     ap.add_argument("--q4-ksplit", type=int, default=0, help="layer: K slices of the Q4_0 matmuls (0 = automatic)")
+    ap.add_argument("--graph", action="store_true",
+                    help="layer workload: also replay the layers from a captured HIP graph")
     ap.add_argument("--no-fuse", action="store_true", help="layer: launch every operator on its own")
     args = ap.parse_args()
     if args.gpus != 1:

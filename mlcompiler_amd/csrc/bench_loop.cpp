@@ -158,53 +158,64 @@ struct MlcBenchLayer {
     double* enqueue_s;        // when set: receives the host time spent encoding (before the wait)
 };
 
-int mlc_bench_layer_loop(const MlcBenchLayer* L, void* const* k_pools, void* const* v_pools,
-                         size_t n_layers, size_t steps, float* event_ms, double* wall_s) {
-    const size_t B = L->batch, HID = L->hidden, FFN = L->ffn_inner;
-    const size_t q_rows = L->num_heads * L->head_dim, kv_rows = L->kv_heads * L->head_dim;
-    const size_t qkv_rows = q_rows + 2 * kv_rows;
-    const size_t s_hid = HID / 32 * 18, s_ffn = FFN / 32 * 18;
+// Weight-cache names of layer l's four matrices.
+static std::vector<std::string> layer_weight_names(size_t n_layers) {
     std::vector<std::string> names(n_layers * 4);
     for (size_t l = 0; l < n_layers; ++l) {
         const char* kinds[4] = {"attn_qkv", "attn_output", "ffn_gate_up", "ffn_down"};
         for (int k = 0; k < 4; ++k) names[l * 4 + k] = "bench.l" + std::to_string(l) + "." + kinds[k];
     }
+    return names;
+}
+
+// Encodes step i of the layer loop (layer i % n_layers, input = the step before's output).
+static int encode_layer_step(const MlcBenchLayer* L, const std::vector<std::string>& names,
+                             void* const* k_pools, void* const* v_pools, size_t n_layers, size_t i) {
+    const size_t B = L->batch, HID = L->hidden, FFN = L->ffn_inner;
+    const size_t q_rows = L->num_heads * L->head_dim, kv_rows = L->kv_heads * L->head_dim;
+    const size_t qkv_rows = q_rows + 2 * kv_rows;
+    const size_t s_hid = HID / 32 * 18, s_ffn = FFN / 32 * 18;
+    const size_t l = i % n_layers;
+    const void* x = (L->out2 && i > 0) ? ((i - 1) % 2 ? L->out2 : L->out) : L->x;
+    void* out = (L->out2 && i % 2) ? L->out2 : L->out;
+    int ok = mlc_hip_rms_norm_batched(x, L->attn_norm_w, HID, 1e-5f, B, HID, L->norm, 0);
+    ok = ok && mlc_hip_matmul_q4_0_batched(names[l * 4 + 0].c_str(), L->w_qkv, L->w_qkv_bytes, L->norm, B,
+                                           qkv_rows, HID, s_hid, 1, L->qkv, 0);
+    ok = ok && mlc_hip_qkv_split_rope_scatter(L->qkv, L->q, k_pools[l], v_pools[l], nullptr, nullptr,
+                                              L->cos, L->sin, L->page_ids, L->slots,
+                                              L->page_size_tokens, B, L->num_heads, L->kv_heads,
+                                              L->head_dim, qkv_rows, q_rows, kv_rows, kv_rows,
+                                              L->head_dim, 0);
+    ok = ok && mlc_hip_paged_attn_decode(L->q, k_pools[l], v_pools[l], L->attn, L->page_tables_flat,
+                                         L->n_flat, L->page_table_offsets, L->seq_lens,
+                                         L->q_positions, B, L->num_heads, L->kv_heads, L->head_dim,
+                                         L->page_size_tokens, 1, 0);
+    ok = ok && mlc_hip_matmul_q4_0_batched(names[l * 4 + 1].c_str(), L->w_o, L->w_o_bytes, L->attn, B, HID,
+                                           HID, s_hid, 1, L->o, 0);
+    ok = ok && mlc_hip_add_batched(x, L->o, L->resid, B * HID, 0);
+    ok = ok && mlc_hip_rms_norm_batched(L->resid, L->ffn_norm_w, HID, 1e-5f, B, HID, L->norm, 0);
+    ok = ok && mlc_hip_matmul_q4_0_batched(names[l * 4 + 2].c_str(), L->w_gate_up, L->w_gate_up_bytes,
+                                           L->norm, B, 2 * FFN, HID, s_hid, 1, L->gate_up, 0);
+    ok = ok && mlc_hip_gate_up_split_silu_mul(L->gate_up, L->gate, L->up, L->mix, B, FFN, 2 * FFN, 0);
+    ok = ok && mlc_hip_matmul_q4_0_batched(names[l * 4 + 3].c_str(), L->w_down, L->w_down_bytes, L->mix, B,
+                                           HID, FFN, s_ffn, 1, L->down, 0);
+    ok = ok && mlc_hip_add_batched(L->resid, L->down, out, B * HID, 0);
+    if (ok && L->head_w && l == n_layers - 1) {
+        ok = mlc_hip_rms_norm_batched(out, L->head_norm_w, HID, 1e-5f, B, HID, L->norm, 0);
+        ok = ok && mlc_hip_matmul_q6_k_batched("bench.lm_head", L->head_w, L->head_bytes, L->norm, B,
+                                               L->head_rows, HID, HID / 256 * 210, L->logits, 0);
+    }
+    return ok;
+}
+
+int mlc_bench_layer_loop(const MlcBenchLayer* L, void* const* k_pools, void* const* v_pools,
+                         size_t n_layers, size_t steps, float* event_ms, double* wall_s) {
+    const std::vector<std::string> names = layer_weight_names(n_layers);
     if (!mlc_hip_begin()) return 0;
     const auto t0 = std::chrono::steady_clock::now();
     if (!mlc_hip_timer_start()) return 0;
-    for (size_t i = 0; i < steps; ++i) {
-        const size_t l = i % n_layers;
-        const void* x = (L->out2 && i > 0) ? ((i - 1) % 2 ? L->out2 : L->out) : L->x;
-        void* out = (L->out2 && i % 2) ? L->out2 : L->out;
-        int ok = mlc_hip_rms_norm_batched(x, L->attn_norm_w, HID, 1e-5f, B, HID, L->norm, 0);
-        ok = ok && mlc_hip_matmul_q4_0_batched(names[l * 4 + 0].c_str(), L->w_qkv, L->w_qkv_bytes, L->norm, B,
-                                               qkv_rows, HID, s_hid, 1, L->qkv, 0);
-        ok = ok && mlc_hip_qkv_split_rope_scatter(L->qkv, L->q, k_pools[l], v_pools[l], nullptr, nullptr,
-                                                  L->cos, L->sin, L->page_ids, L->slots,
-                                                  L->page_size_tokens, B, L->num_heads, L->kv_heads,
-                                                  L->head_dim, qkv_rows, q_rows, kv_rows, kv_rows,
-                                                  L->head_dim, 0);
-        ok = ok && mlc_hip_paged_attn_decode(L->q, k_pools[l], v_pools[l], L->attn, L->page_tables_flat,
-                                             L->n_flat, L->page_table_offsets, L->seq_lens,
-                                             L->q_positions, B, L->num_heads, L->kv_heads, L->head_dim,
-                                             L->page_size_tokens, 1, 0);
-        ok = ok && mlc_hip_matmul_q4_0_batched(names[l * 4 + 1].c_str(), L->w_o, L->w_o_bytes, L->attn, B, HID,
-                                               HID, s_hid, 1, L->o, 0);
-        ok = ok && mlc_hip_add_batched(x, L->o, L->resid, B * HID, 0);
-        ok = ok && mlc_hip_rms_norm_batched(L->resid, L->ffn_norm_w, HID, 1e-5f, B, HID, L->norm, 0);
-        ok = ok && mlc_hip_matmul_q4_0_batched(names[l * 4 + 2].c_str(), L->w_gate_up, L->w_gate_up_bytes,
-                                               L->norm, B, 2 * FFN, HID, s_hid, 1, L->gate_up, 0);
-        ok = ok && mlc_hip_gate_up_split_silu_mul(L->gate_up, L->gate, L->up, L->mix, B, FFN, 2 * FFN, 0);
-        ok = ok && mlc_hip_matmul_q4_0_batched(names[l * 4 + 3].c_str(), L->w_down, L->w_down_bytes, L->mix, B,
-                                               HID, FFN, s_ffn, 1, L->down, 0);
-        ok = ok && mlc_hip_add_batched(L->resid, L->down, out, B * HID, 0);
-        if (ok && L->head_w && l == n_layers - 1) {
-            ok = mlc_hip_rms_norm_batched(out, L->head_norm_w, HID, 1e-5f, B, HID, L->norm, 0);
-            ok = ok && mlc_hip_matmul_q6_k_batched("bench.lm_head", L->head_w, L->head_bytes, L->norm, B,
-                                                   L->head_rows, HID, HID / 256 * 210, L->logits, 0);
-        }
-        if (!ok) return 0;
-    }
+    for (size_t i = 0; i < steps; ++i)
+        if (!encode_layer_step(L, names, k_pools, v_pools, n_layers, i)) return 0;
     if (L->enqueue_s) *L->enqueue_s = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
     const float ms = mlc_hip_timer_stop();
     if (ms < 0.f) return 0;
@@ -213,6 +224,67 @@ int mlc_bench_layer_loop(const MlcBenchLayer* L, void* const* k_pools, void* con
     if (event_ms) *event_ms = ms;
     if (wall_s) *wall_s = std::chrono::duration<double>(t1 - t0).count();
     return 1;
+}
+
+// The same loop with one pass over the n_layers layers (n_layers even, so that a pass ends in
+// the buffer the next one starts from) captured into a HIP graph and replayed `replays` times:
+// measures what replaying prebuilt launches saves over encoding them call by call.  The pass
+// is run once uncaptured first, so that every weight, norm vector, page table and scratch
+// buffer is already on the device and the captured pass holds kernel launches only.
+// event_ms receives the time of all replays.  Returns 1 on success, 0 on failure, and -1 when
+// the captured pass held something other than kernels (then nothing is replayed).
+int mlc_bench_layer_loop_graph(const MlcBenchLayer* L, void* const* k_pools, void* const* v_pools,
+                               size_t n_layers, size_t replays, float* event_ms, size_t* n_nodes) {
+    if (n_layers == 0 || n_layers % 2 != 0) return 0;
+    const std::vector<std::string> names = layer_weight_names(n_layers);
+    if (!mlc_hip_begin()) return 0;
+    for (size_t i = 0; i < n_layers; ++i)
+        if (!encode_layer_step(L, names, k_pools, v_pools, n_layers, i)) return 0;
+    if (!mlc_hip_flush() || !mlc_hip_begin()) return 0;
+    hipStream_t stream = static_cast<hipStream_t>(mlc_hip_stream());
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    if (hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal) != hipSuccess) return 0;
+    int ok = 1;
+    for (size_t i = 0; ok && i < n_layers; ++i) ok = encode_layer_step(L, names, k_pools, v_pools, n_layers, i);
+    (void)mlc_hip_stream();  // launches what the library still holds back
+    if (hipStreamEndCapture(stream, &graph) != hipSuccess || !ok || !graph) {
+        (void)hipGetLastError();
+        if (graph) (void)hipGraphDestroy(graph);
+        return 0;
+    }
+    size_t count = 0;
+    int rc = 1;
+    std::vector<hipGraphNode_t> nodes;
+    if (hipGraphGetNodes(graph, nullptr, &count) != hipSuccess) rc = 0;
+    if (rc) {
+        nodes.resize(count);
+        if (count && hipGraphGetNodes(graph, nodes.data(), &count) != hipSuccess) rc = 0;
+    }
+    for (size_t i = 0; rc == 1 && i < count; ++i) {
+        hipGraphNodeType type;
+        if (hipGraphNodeGetType(nodes[i], &type) != hipSuccess) rc = 0;
+        else if (type != hipGraphNodeTypeKernel) rc = -1;
+    }
+    if (n_nodes) *n_nodes = count;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (rc == 1 && hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0) != hipSuccess) rc = 0;
+    if (rc == 1 && (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)) rc = 0;
+    if (rc == 1) {
+        rc = hipGraphLaunch(exec, stream) == hipSuccess && hipStreamSynchronize(stream) == hipSuccess;
+        rc = rc && hipEventRecord(e0, stream) == hipSuccess;
+        for (size_t i = 0; rc == 1 && i < replays; ++i) rc = hipGraphLaunch(exec, stream) == hipSuccess;
+        rc = rc && hipEventRecord(e1, stream) == hipSuccess && hipEventSynchronize(e1) == hipSuccess;
+        float ms = 0.f;
+        rc = rc && hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
+        if (event_ms) *event_ms = ms;
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (exec) (void)hipGraphExecDestroy(exec);
+    (void)hipGraphDestroy(graph);
+    if (!mlc_hip_flush()) return 0;
+    return rc;
 }
 
 }  // extern "C"
