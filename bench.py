@@ -373,7 +373,7 @@ def finish_step(args, exe, L, loop, lc, c, w, x, cos, sin, page_ids, slots, qpos
         "roofline": {"bound": "hbm", "achieved": round(alg_bytes / ev_s / 1e9, 2), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(alg_bytes / ev_s / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
                      "us_per_launch": round(ev_s * 1e6, 2),
-                     "note": "a whole step (222 kernels) between HIP events / steps; algorithmic bytes = all "
+                     "note": "a whole step (200 kernels) between HIP events / steps; algorithmic bytes = all "
                              "weights once + the K/V of all layers"},
     }
     if not args.no_cpu:

@@ -262,6 +262,9 @@ int mlc_hip_last_decode_work_items(void);
 /* Number of KV writes so far that went out fused with a neighbour: a batched K scatter with its
  * V twin, or split + RoPE + cast with the scatters of its fp16 rows (for tests). */
 long mlc_hip_fused_kv_write_launches(void);
+/* Number of Q4_0 matmuls so far that went out with the split + RoPE + cast (and KV write) of
+ * their output as epilogue (for tests). */
+long mlc_hip_fused_matmul_rope_launches(void);
 /* Number of fused row-operator launches so far (for tests of "fuse_row_ops"). */
 long mlc_hip_row_program_launches(void);
 

@@ -136,6 +136,7 @@ struct Ctx {
     struct KvPending {
         bool active = false;
         bool rope = false;
+        bool from_gemm = false;             // rope form: runs as the epilogue of the pending matmul
         RopeArgs a{};                       // rope form
         const void* src[2] = {nullptr, nullptr};   // plain form: fp16 rows of the first / second scatter
         void* pages[2] = {nullptr, nullptr};
@@ -146,6 +147,18 @@ struct Ctx {
         const uint32_t* d_slots = nullptr;
         size_t batch = 0, row_elems = 0, page_size = 0;
     } kv;
+    // A Q4_0 matmul of the open pass whose launch is held back for one call: when that call is
+    // the split + RoPE + cast of the matmul's output (the qkv projection of a layer), the
+    // matmul's epilogue does it and the two -- with the KV scatters that join -- are one launch.
+    struct GemmPending {
+        bool active = false;
+        Q4Args a{};
+        unsigned grid_x = 0;
+        int nbt = 1, rt = 1;
+        const void* out = nullptr;
+        size_t batch = 0, rows = 0;
+    } gemm;
+    long gemm_rope_fused = 0;        // matmuls launched with the RoPE epilogue (for tests)
     long kv_fused = 0;               // KV writes that went out fused with a neighbour (for tests)
     long opt_fuse_rows = 1;          // 0 = every operator is launched when it is encoded
     long row_launches = 0;           // row_program_kernel launches (for tests)
@@ -269,6 +282,38 @@ constexpr size_t kRowMaxLen = 16384;  // row_program_kernel: 8 groups of 8 eleme
 
 bool row_len_ok(size_t len) { return len > 0 && len % 8 == 0 && len <= kRowMaxLen; }
 
+// Launches the held-back matmul, with the split + RoPE + cast of its output as epilogue when
+// `rope` is given.
+int settle_gemm(const RopeArgs* rope = nullptr) {
+    Ctx::GemmPending& m = g.gemm;
+    if (!m.active) return 1;
+    m.active = false;
+    Q4Args a = m.a;
+    if (rope) {
+        a.rope_on = 1;
+        a.rope = *rope;
+        ++g.gemm_rope_fused;
+    }
+    const dim3 grid(m.grid_x, 1);
+    if (m.nbt == 1) {
+        if (m.rt == 1) hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<1, 1, 16>), grid, dim3(1024), 0, g.stream, a);
+        else hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<1, 2, 16>), grid, dim3(1024), 0, g.stream, a);
+    } else {
+        if (m.rt == 1) hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<2, 1, 8>), grid, dim3(512), 0, g.stream, a);
+        else hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<2, 2, 8>), grid, dim3(512), 0, g.stream, a);
+    }
+    HIP_OK(hipGetLastError());
+    return 1;
+}
+
+// True when the held-back matmul's output is exactly the fused qkv rows a split + RoPE + cast
+// call describes, so that the matmul's epilogue can do that call's work.
+bool gemm_feeds_rope(const void* qkv, size_t batch, size_t qkv_rows, size_t q_rows, size_t k_rows, size_t v_rows) {
+    const Ctx::GemmPending& m = g.gemm;
+    return g.opt_fuse_rows && m.active && !g.kv.active && !g.rows.active && m.out == qkv && m.batch == batch &&
+           m.rows == qkv_rows && q_rows + k_rows + v_rows == qkv_rows;
+}
+
 // Launches the pending KV write.
 int settle_kv() {
     Ctx::KvPending& kv = g.kv;
@@ -276,6 +321,7 @@ int settle_kv() {
     kv.active = false;
     if (kv.rope) {
         if (kv.a.k_pages || kv.a.v_pages) ++g.kv_fused;
+        if (kv.from_gemm) return settle_gemm(&kv.a);
         launch_qkv_split_rope_cast(kv.a, g.stream);
         HIP_OK(hipGetLastError());
         return 1;
@@ -303,6 +349,9 @@ int settle_kv() {
 // than a pending chain (whatever starts the KV write launches the chain first, and a scatter
 // only joins while no chain is pending).
 int settle() {
+    // a held-back matmul is older than anything else pending, unless the pending KV write is
+    // its own epilogue
+    if (g.gemm.active && !(g.kv.active && g.kv.rope && g.kv.from_gemm) && !settle_gemm()) return 0;
     if (!settle_kv()) return 0;
     Ctx::RowPending& r = g.rows;
     if (!r.active) return 1;
@@ -1048,7 +1097,8 @@ int mlc_hip_qkv_split_rope_cast(const void* qkv, void* q, void* k, void* v, void
                                 size_t q_rows, size_t k_rows, size_t v_rows, size_t rotary_dim,
                                 int sync) {
     if (!init_once()) return fail("GPU unavailable");
-    if (!settle()) return 0;
+    const bool from_gemm = gemm_feeds_rope(qkv, batch, qkv_rows, q_rows, k_rows, v_rows);
+    if (!from_gemm && !settle()) return 0;
     if (!sync && !g.pass_open) return fail("encode: no open forward pass");  // :7936
     if (const char* why = rope_args_problem(qkv, q, cos_buf, sin_buf, batch, num_heads, kv_heads,
                                             head_dim, qkv_rows, q_rows, k_rows, v_rows, rotary_dim))
@@ -1080,6 +1130,7 @@ int mlc_hip_qkv_split_rope_cast(const void* qkv, void* q, void* k, void* v, void
     kv = Ctx::KvPending{};
     kv.active = true;
     kv.rope = true;
+    kv.from_gemm = from_gemm;
     kv.a = a;
     kv.batch = batch;
     kv.row_elems = k_rows;
@@ -1094,7 +1145,8 @@ int mlc_hip_qkv_split_rope_scatter(const void* qkv, void* q, void* k_pages, void
                                    size_t kv_heads, size_t head_dim, size_t qkv_rows, size_t q_rows,
                                    size_t k_rows, size_t v_rows, size_t rotary_dim, int sync) {
     if (!init_once()) return fail("GPU unavailable");
-    if (!settle()) return 0;
+    const bool from_gemm = gemm_feeds_rope(qkv, batch, qkv_rows, q_rows, k_rows, v_rows);
+    if (!from_gemm && !settle()) return 0;
     if (!sync && !g.pass_open) return fail("encode: no open forward pass");
     if (const char* why = rope_args_problem(qkv, q, cos_buf, sin_buf, batch, num_heads, kv_heads,
                                             head_dim, qkv_rows, q_rows, k_rows, v_rows, rotary_dim))
@@ -1131,7 +1183,11 @@ int mlc_hip_qkv_split_rope_scatter(const void* qkv, void* q, void* k_pages, void
     a.batch = (uint32_t)batch; a.head_dim = (uint32_t)head_dim; a.qkv_rows = (uint32_t)qkv_rows;
     a.q_rows = (uint32_t)q_rows; a.k_rows = (uint32_t)k_rows; a.v_rows = (uint32_t)v_rows;
     a.rotary_dim = (uint32_t)rotary_dim; a.page_size = (uint32_t)page_size_tokens;
-    launch_qkv_split_rope_cast(a, g.stream);
+    if (from_gemm && g.gemm.active) {  // (still held back: the id upload above launches nothing)
+        if (!settle_gemm(&a)) return 0;
+    } else {
+        launch_qkv_split_rope_cast(a, g.stream);
+    }
     return finish(sync);
 }
 
@@ -1394,6 +1450,21 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
         a.out = ksplit > 1 ? slices : o;
         a.batch = (uint32_t)bn; a.rows = (uint32_t)rows; a.nblocks = (uint32_t)nblocks;
         a.blocks_per_slice = (uint32_t)per_slice; a.ksplit = (uint32_t)ksplit;
+        a.rope_on = 0;
+        a.rope = RopeArgs{};
+        if (g.opt_fuse_rows && !sync && ksplit == 1 && batch <= 64) {
+            // held back for one call: a split + RoPE + cast of this output becomes the epilogue
+            Ctx::GemmPending& m = g.gemm;
+            m.active = true;
+            m.a = a;
+            m.grid_x = (unsigned)wgs;
+            m.nbt = bpad == 32 ? 1 : 2;
+            m.rt = row_tiles;
+            m.out = out;
+            m.batch = batch;
+            m.rows = rows;
+            return finish(sync);
+        }
         const dim3 grid((unsigned)wgs, (unsigned)ksplit);
         if (bpad == 32) {
             if (row_tiles == 1) hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<1, 1, 16>), grid, dim3(1024), 0, g.stream, a);
@@ -1639,6 +1710,7 @@ float mlc_hip_timer_stop(void) {
 int mlc_hip_last_decode_launches(void) { return g.last_launches; }
 int mlc_hip_last_decode_work_items(void) { return g.last_items; }
 long mlc_hip_fused_kv_write_launches(void) { return g.kv_fused; }
+long mlc_hip_fused_matmul_rope_launches(void) { return g.gemm_rope_fused; }
 long mlc_hip_row_program_launches(void) { return g.row_launches; }
 
 int mlc_hip_set_option(const char* name, long value) {

@@ -24,6 +24,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "paged_rope_kernels.h"
+
 namespace mlc_hip {
 
 typedef _Float16 q4_half2 __attribute__((ext_vector_type(2)));
@@ -140,7 +142,65 @@ struct Q4Args {
     const float* inv_scale;     // [batch]
     float* out;                 // [batch][rows], or the slice buffer [ksplit][batch][rows]
     uint32_t batch, rows, nblocks, blocks_per_slice, ksplit;
+    // When rope_on is set (ksplit == 1, out is a fused qkv row of rope.qkv_rows = rows floats per
+    // request): the epilogue also does what qkv_split_rope_cast_kernel would do with that row.
+    uint32_t rope_on;
+    RopeArgs rope;
 };
+
+// The split + RoPE + cast (+ paged write) of one element of a request's fused qkv row, by the
+// thread that just produced it; the partner of its (even, odd) pair sits in the neighbouring
+// lane.  Same arithmetic, element for element, as qkv_split_rope_cast_kernel.  What the thread
+// needs from memory for it (its cos / sin pair, its request's page row) is fetched before the
+// matmul's main loop, so that the epilogue adds no memory round trip to the kernel's tail.
+struct Q4RopeFetch {
+    float c, s;        // rotation of this element's pair (1, 0 where none applies)
+    uint32_t page_row; // page_ids[req] * page_size + slots[req]
+};
+
+__device__ __forceinline__ Q4RopeFetch q4_rope_prefetch(const RopeArgs& p, uint32_t req, uint32_t feat) {
+    Q4RopeFetch f = {1.0f, 0.0f, 0u};
+    if (req >= p.batch || feat >= p.q_rows + p.k_rows + p.v_rows) return f;
+    const bool is_q = feat < p.q_rows;
+    const bool is_k = !is_q && feat < p.q_rows + p.k_rows;
+    const uint32_t local = is_q ? feat : (is_k ? feat - p.q_rows : feat - p.q_rows - p.k_rows);
+    if (is_q || is_k) {
+        const uint32_t d = (local & ~1u) % p.head_dim;
+        if (d < p.rotary_dim) {
+            const uint32_t ci = req * (p.rotary_dim / 2) + d / 2;
+            f.c = p.cos_table[ci];
+            f.s = p.sin_table[ci];
+        }
+    }
+    if (!is_q && (is_k ? p.k_pages : p.v_pages)) f.page_row = p.page_ids[req] * p.page_size + p.slots[req];
+    return f;
+}
+
+__device__ __forceinline__ void q4_rope_epilogue(const RopeArgs& p, const Q4RopeFetch& f, uint32_t req,
+                                                 uint32_t feat, float val) {
+    const float other = __shfl_xor(val, 1);
+    const bool odd = (feat & 1u) != 0;
+    const float2 x = odd ? make_float2(other, val) : make_float2(val, other);
+    if (feat >= p.q_rows + p.k_rows + p.v_rows) return;
+    const bool is_q = feat < p.q_rows;
+    const bool is_k = !is_q && feat < p.q_rows + p.k_rows;
+    const uint32_t local = is_q ? feat : (is_k ? feat - p.q_rows : feat - p.q_rows - p.k_rows);
+    float2 y = x;
+    if ((is_q || is_k) && (local & ~1u) % p.head_dim < p.rotary_dim) y = rope_rotate(x, f.c, f.s);
+    const float mine = odd ? y.y : y.x;
+    if (is_q) {
+        p.q[(size_t)req * p.q_rows + local] = mine;
+        return;
+    }
+    float* f32 = is_k ? p.k : p.v;
+    const uint32_t rows = is_k ? p.k_rows : p.v_rows;
+    if (f32) f32[(size_t)req * rows + local] = mine;
+    const _Float16 h = (_Float16)mine;
+    _Float16* f16 = is_k ? p.k_f16 : p.v_f16;
+    if (f16) f16[(size_t)req * rows + local] = h;
+    _Float16* pool = is_k ? p.k_pages : p.v_pages;
+    if (pool) pool[(size_t)f.page_row * rows + local] = h;
+}
 
 // (0x6400 | n) is the half 1024 + n: two nibbles -> half2 (n0 - 8, n1 - 8), exactly.
 __device__ __forceinline__ q4_half2 q4_pair(uint32_t bytes, uint32_t sel) {
@@ -177,6 +237,17 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
         for (int t = 0; t < NBT; ++t)
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[r][t][i] = 0.f;
+
+    // epilogue mapping, thread -> (weight row, batch column): consecutive threads write
+    // consecutive rows of out[b][..]
+    constexpr uint32_t ROWS = 32 * RT, COLS_PER_PASS = WAVES * 64 / ROWS, PASSES = 32 * NBT / COLS_PER_PASS;
+    const uint32_t row = threadIdx.x % ROWS, bsub = threadIdx.x / ROWS;
+    Q4RopeFetch rope_pre[PASSES];
+    if (a.rope_on) {
+#pragma unroll
+        for (uint32_t pass = 0; pass < PASSES; ++pass)
+            rope_pre[pass] = q4_rope_prefetch(a.rope, pass * COLS_PER_PASS + bsub, tile0 * 32 + row);
+    }
 
     struct Block {
         uint2 q[RT];
@@ -263,21 +334,20 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
             for (int i = 0; i < 16; ++i)
                 red[(((wave * RT + r) * NBT + t) * 16 + i) * PITCH + lane] = acc[r][t][i];
     __syncthreads();
-    // thread -> (weight row, batch column): consecutive threads write consecutive rows of out[b][..]
-    constexpr uint32_t ROWS = 32 * RT, COLS_PER_PASS = WAVES * 64 / ROWS;
-    const uint32_t row = threadIdx.x % ROWS, bsub = threadIdx.x / ROWS;
     const uint32_t r = row / 32, rr = row % 32;
     const uint32_t i = (rr / 8) * 4 + rr % 4, hf = (rr % 8) / 4;
     float* out = a.out + (size_t)slice * a.batch * a.rows;
 #pragma unroll
-    for (uint32_t pass = 0; pass < 32 * NBT / COLS_PER_PASS; ++pass) {
+    for (uint32_t pass = 0; pass < PASSES; ++pass) {
         const uint32_t b = pass * COLS_PER_PASS + bsub;
         if (b >= a.batch) continue;
         const uint32_t t = b / 32, ln = hf * 32 + b % 32;
         float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) sum += red[(((w * RT + r) * NBT + t) * 16 + i) * PITCH + ln];
-        out[(size_t)b * a.rows + tile0 * 32 + row] = sum * a.inv_scale[b];
+        const float val = sum * a.inv_scale[b];
+        out[(size_t)b * a.rows + tile0 * 32 + row] = val;
+        if (a.rope_on) q4_rope_epilogue(a.rope, rope_pre[pass], b, tile0 * 32 + row, val);  // (the lanes of a pair share b)
     }
 }
 
