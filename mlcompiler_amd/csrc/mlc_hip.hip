@@ -241,7 +241,9 @@ size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 // with this content.  The copy is ordered on the library stream, so kernels already enqueued
 // that read the previous content are not disturbed.  nullptr on failure (error recorded).
 const void* resident_blob(int kind, const void* key, const void* blob, size_t bytes) {
-    if (g.resident.size() > 1024) {  // a caller that never repeats itself: start over
+    // A caller that never repeats itself: start over -- but only while no held-back operator
+    // refers to one of the copies (their launches come later).
+    if (g.resident.size() > 1024 && !g.rows.active && !g.kv.active && !g.gemm.active) {
         if (hipStreamSynchronize(g.stream) != hipSuccess) { fail("resident: synchronize failed"); return nullptr; }
         for (auto& kv : g.resident)
             if (kv.second.dev) (void)hipFree(kv.second.dev);
