@@ -553,6 +553,22 @@ def main() -> int:
     launches = exe.lastDecodeLaunches()
     items = exe.lastDecodeWorkItems()
 
+    # ---- one launch at a time, HIP events around each (the reference's harness reports its
+    # timings this way: warm-up, >= 200 iterations, median and p10 / p90,
+    # tools/paged_flash_bench.cpp:55-76)
+    singles = []
+    exe.beginForwardPassCB()
+    for i in range(203):
+        exe.timerStart()
+        step(i % n_layers)
+        t = exe.timerStopMs()
+        if i >= 3:
+            singles.append(t * 1e3)
+    exe.flushForwardPassCB()
+    singles.sort()
+    single_us = {"median": round(singles[len(singles) // 2], 2), "p10": round(singles[len(singles) // 10], 2),
+                 "p90": round(singles[len(singles) * 9 // 10], 2), "n": len(singles)}
+
     # ---- boundary-inclusive figure: tables change every call, so each call re-plans and
     # re-uploads its metadata (what a caller that rebuilds its tables per layer would see)
     n_b = min(args.steps, 200)
@@ -647,6 +663,7 @@ def main() -> int:
             "kernels_per_step": launches,
             "work_items": items,
             "us_per_layer_with_metadata_upload": round(boundary_us, 3),
+            "single_launch_us": single_us,
             "us_per_layer_with_kv_write": round(kv_write_us, 3),
         },
         "roofline": {
