@@ -242,8 +242,10 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
     // consecutive rows of out[b][..]
     constexpr uint32_t ROWS = 32 * RT, COLS_PER_PASS = WAVES * 64 / ROWS, PASSES = 32 * NBT / COLS_PER_PASS;
     const uint32_t row = threadIdx.x % ROWS, bsub = threadIdx.x / ROWS;
-    Q4RopeFetch rope_pre[PASSES];
-    if (a.rope_on) {
+    // (fetched ahead only where a thread has one or two outputs: more would cost the loop registers)
+    constexpr bool ROPE_AHEAD = PASSES <= 2;
+    Q4RopeFetch rope_pre[ROPE_AHEAD ? PASSES : 1];
+    if (ROPE_AHEAD && a.rope_on) {
 #pragma unroll
         for (uint32_t pass = 0; pass < PASSES; ++pass)
             rope_pre[pass] = q4_rope_prefetch(a.rope, pass * COLS_PER_PASS + bsub, tile0 * 32 + row);
@@ -347,7 +349,9 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
         for (int w = 0; w < WAVES; ++w) sum += red[(((w * RT + r) * NBT + t) * 16 + i) * PITCH + ln];
         const float val = sum * a.inv_scale[b];
         out[(size_t)b * a.rows + tile0 * 32 + row] = val;
-        if (a.rope_on) q4_rope_epilogue(a.rope, rope_pre[pass], b, tile0 * 32 + row, val);  // (the lanes of a pair share b)
+        if (a.rope_on)  // (the lanes of a pair share b)
+            q4_rope_epilogue(a.rope, ROPE_AHEAD ? rope_pre[ROPE_AHEAD ? pass : 0] : q4_rope_prefetch(a.rope, b, tile0 * 32 + row),
+                             b, tile0 * 32 + row, val);
     }
 }
 
