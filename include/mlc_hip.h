@@ -265,6 +265,9 @@ long mlc_hip_fused_kv_write_launches(void);
 /* Number of Q4_0 matmuls so far that went out with the split + RoPE + cast (and KV write) of
  * their output as epilogue (for tests). */
 long mlc_hip_fused_matmul_rope_launches(void);
+/* Number of decode attention launches so far that carried the step's KV write (a pair of
+ * batched K / V scatters of every request's newest position encoded just before it). */
+long mlc_hip_kv_writes_in_decode_launches(void);
 /* Number of fused row-operator launches so far (for tests of "fuse_row_ops"). */
 long mlc_hip_row_program_launches(void);
 

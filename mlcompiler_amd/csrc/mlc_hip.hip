@@ -160,6 +160,7 @@ struct Ctx {
     } gemm;
     long gemm_rope_fused = 0;        // matmuls launched with the RoPE epilogue (for tests)
     long kv_fused = 0;               // KV writes that went out fused with a neighbour (for tests)
+    long kv_in_decode = 0;           // ... of which inside the attention launch
     long opt_fuse_rows = 1;          // 0 = every operator is launched when it is encoded
     long row_launches = 0;           // row_program_kernel launches (for tests)
     MetaSlot plan_slots[4];
@@ -791,7 +792,13 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
                               size_t kv_heads, size_t head_dim, size_t page_size_tokens,
                               int apply_causal, int sync) {
     if (!init_once()) return fail("GPU unavailable");
-    if (!settle()) return 0;
+    // A pending pair of batched K / V scatters into these pools may be this step's KV write
+    // (batched_walker.cpp:304-331): then the attention launch does it (decided below, once the
+    // tables are known to be valid); anything else pending is launched now.
+    bool carries_kv = g.opt_fuse_rows && g.kv.active && !g.kv.rope && g.kv.n == 2 && g.kv.wide && !g.rows.active &&
+                      !g.gemm.active && g.kv.pages[0] == k_pages && g.kv.pages[1] == v_pages && g.kv.batch == batch &&
+                      g.kv.row_elems == kv_heads * head_dim && g.kv.page_size == page_size_tokens;
+    if (!carries_kv && !settle()) return 0;
     if (!sync && !g.pass_open) return fail("encode: no open forward pass");  // :7090
     // metal_runtime.mm:7742-7750
     if (!q || !k_pages || !v_pages || !o) return fail("decode: null buffer");
@@ -825,6 +832,18 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
     MetaSlot& slot = g.plan_slots[p.slot];
     const char* dev = static_cast<const char*>(slot.dev);
     const float scale_log2e = (1.0f / std::sqrt(static_cast<float>(head_dim))) * 1.44269504088896340736f;
+    if (carries_kv) {
+        // only the tiled kernel writes rows, and only rows that are every request's newest
+        // visible position: then exactly one work item reads each of them, after writing it
+        carries_kv = p.fast;
+        for (size_t r = 0; carries_kv && r < batch; ++r) {
+            const uint64_t S = seq_lens[r];
+            const bool visible = !apply_causal || (uint64_t)q_positions[r] + 1 >= S;
+            carries_kv = S > 0 && visible && g.kv.slots[r] == (S - 1) % page_size_tokens &&
+                         g.kv.ids[r] == page_tables_flat[page_table_offsets[r] + (S - 1) / page_size_tokens];
+        }
+        if (!carries_kv && !settle()) return 0;
+    }
 
     g.last_launches = 0;
     g.last_items = (int)p.n_items;
@@ -846,7 +865,20 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
         a.page_size = (uint32_t)page_size_tokens;
         a.n_items = p.n_items;
         a.scale_log2e = scale_log2e;
+        a.new_k = a.new_v = nullptr;
+        a.new_ids = a.new_slots = nullptr;
+        if (carries_kv) {
+            a.new_k = static_cast<const uint4*>(g.kv.src[0]);
+            a.new_v = static_cast<const uint4*>(g.kv.src[1]);
+            a.new_ids = g.kv.d_ids;
+            a.new_slots = g.kv.d_slots;
+        }
         if (!launch_fast(head_dim, p.hpw, p.nw, p.ns, p.nbuf, a)) return fail("decode: kernel variant not built");
+        if (carries_kv) {  // (pages are not shared between requests, paged_kv.hpp:61-64: nobody else reads those rows)
+            g.kv.active = false;
+            ++g.kv_fused;
+            ++g.kv_in_decode;
+        }
         ++g.last_launches;
     } else {
         GenericArgs a;
@@ -1713,6 +1745,7 @@ int mlc_hip_last_decode_launches(void) { return g.last_launches; }
 int mlc_hip_last_decode_work_items(void) { return g.last_items; }
 long mlc_hip_fused_kv_write_launches(void) { return g.kv_fused; }
 long mlc_hip_fused_matmul_rope_launches(void) { return g.gemm_rope_fused; }
+long mlc_hip_kv_writes_in_decode_launches(void) { return g.kv_in_decode; }
 long mlc_hip_row_program_launches(void) { return g.row_launches; }
 
 int mlc_hip_set_option(const char* name, long value) {

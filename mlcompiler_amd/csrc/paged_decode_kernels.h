@@ -77,6 +77,14 @@ struct DecodeArgs {
     uint32_t page_size;         // tokens per page
     uint32_t n_items;
     float scale_log2e;          // log2(e) / sqrt(D)
+    // The step's KV write done by this launch (null: none): the new fp16 K / V row of every
+    // request, [B][Hkv][D], goes to its newest position (new_rows[r] = page id * page size +
+    // slot, which the caller has checked to be position seq_len - 1 of request r) before the
+    // item that reads that position loads anything.
+    const uint4* new_k;
+    const uint4* new_v;
+    const uint32_t* new_ids;    // [B] page ids
+    const uint32_t* new_slots;  // [B] slots in page
 };
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
@@ -213,6 +221,27 @@ __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const D
         if (wave < NW)
             for (int i = lane; i < HPW * D; i += 64) orow[i] = 0.f;
         return;
+    }
+
+    // The step's KV write, when this launch carries it: the item that ends at the request's
+    // newest position (the last split, or the only item) copies its KV head's slice of the new K
+    // and V rows into the pages and waits for the stores, so that its own tile loads below see
+    // them; no other item reads that position.  Nothing is in flight after this block, so the
+    // waits further down count the same loads as without it.
+    if (a.new_k != nullptr) {
+        const bool newest = it.part_first == kNoPartial || (it.split & 0xFFFFu) + 1u == (it.split >> 16);
+        if (newest) {
+            if (wave == 0 && lane < 2 * CPR) {
+                const bool is_v = lane >= CPR;
+                const uint32_t cc = lane % CPR;
+                const size_t row = (size_t)a.new_ids[it.req] * a.page_size + a.new_slots[it.req];
+                const uint4 val = (is_v ? a.new_v : a.new_k)[((size_t)it.req * a.kv_heads + it.kv_head) * CPR + cc];
+                uint4* dst = const_cast<uint4*>(is_v ? a.v_pages : a.k_pages);
+                dst[(row * a.kv_heads + it.kv_head) * CPR + cc] = val;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // stores complete (vmcnt 0)
+            __syncthreads();
+        }
     }
 
     // q for this wave's heads, dims c*8 .. c*8+7 (issued before the tile loads, so that waiting

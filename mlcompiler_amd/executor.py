@@ -255,6 +255,10 @@ class HipExecutor:
         """KV writes so far that went out fused with a neighbour (option "fuse_row_ops")."""
         return int(self._lib.mlc_hip_fused_kv_write_launches())
 
+    def kvWritesInDecodeLaunches(self) -> int:
+        """Decode attention launches so far that carried the step's KV write."""
+        return int(self._lib.mlc_hip_kv_writes_in_decode_launches())
+
     def fusedMatmulRopeLaunches(self) -> int:
         """Q4_0 matmuls so far launched with the split + RoPE + cast of their output as epilogue."""
         return int(self._lib.mlc_hip_fused_matmul_rope_launches())
