@@ -588,7 +588,7 @@ def main() -> int:
 
     # ---- the layer as the batched step runs it (batched_walker.cpp:304-331): write the step's
     # new K row and V row (they land on the newest position: the bytes read stay the same), then
-    # attend.  Three launches per layer.
+    # attend.  Three encode calls per layer; the attention launch carries the two scatters.
     rng = np.random.default_rng(5)
     row = c.kv_heads * c.head_dim
     new_k = rng.standard_normal((c.batch, row)).astype(np.float16)
