@@ -100,3 +100,28 @@ def test_other_rows_are_written_by_their_own_launch(exe):
         assert carried == 0
         assert np.array_equal(kp, want_k) and np.array_equal(vp, want_v)
         assert_parity(out, want_o, 64, "kv step, separate launches")
+
+
+@pytest.mark.parametrize("opts", [{"decode_tile_rows": 2}, {"decode_buffers": 1}, {"decode_buffers": 2},
+                                  {"decode_heads_per_wave": 8}, {"decode_heads_per_wave": 1},
+                                  {"decode_tile_rows": 2, "decode_target_items": 100000}],
+                         ids=lambda o: ",".join(f"{k[7:]}={v}" for k, v in o.items()))
+def test_kv_write_and_two_level_merge_in_every_kernel_variant(exe, opts):
+    """The same step through the other shapes of the tiled kernel (two tile rows per workgroup,
+    one or two staging buffers, other head groupings), with one request long enough to be cut
+    into more splits than one wave merges at once."""
+    lens = [1, 65, 700, 9000, 128]
+    case = make_case("kvstep_variants", len(lens), 32, 8, 64, 64, lens, seed=21, capacity_pages=160)
+    ids, slots = _newest(case)
+    new_k, new_v = _rows(case, 23)
+    want_k, want_v, want_o = _expect(case, ids, slots, new_k, new_v)
+    for name, value in opts.items():
+        assert exe.setOption(name, value)
+    try:
+        out, kp, vp, carried = _step(exe, case, ids, slots, new_k, new_v, 1, target=opts.get("decode_target_items", 0))
+    finally:
+        for name in opts:
+            exe.setOption(name, 1 if name == "decode_tile_rows" else 0)
+    assert carried == 1
+    assert np.array_equal(kp, want_k) and np.array_equal(vp, want_v)
+    assert_parity(out, want_o, 64, f"kv step {opts}")
