@@ -19,12 +19,16 @@ from layer_case import D, FFN, H, HID, HKV, KV_ROWS, P, Q_ROWS, QKV_ROWS, make_l
 
 
 @pytest.mark.timeout(300)
+@pytest.mark.parametrize("kv_calls", ["one_call", "reference_calls"])
 @pytest.mark.parametrize("fuse", [1, 0])
 @pytest.mark.parametrize("batch", [6, 33])
-def test_decoder_layer_matches_oracle_chain(exe, batch, fuse):
+def test_decoder_layer_matches_oracle_chain(exe, batch, fuse, kv_calls):
     """fuse = 1: the row-local operators between the matmuls run as fused launches (the default);
-    fuse = 0: every operator is launched on its own.  Same expected values either way."""
-    print(f"[layer] batch={batch} fuse_row_ops={fuse}", flush=True)
+    fuse = 0: every operator is launched on its own.  Same expected values either way.
+    kv_calls: the split + RoPE + cast + KV write as the one fused call, or as the walker's three
+    calls (encodeQkvSplitRopeCast, then the batched scatters of its fp16 K and V rows,
+    batched_walker.cpp:287-307)."""
+    print(f"[layer] batch={batch} fuse_row_ops={fuse} {kv_calls}", flush=True)
     rng = np.random.default_rng(100 + batch)
     w = make_layer_weights(200 + batch)
     w_qkv, w_o, w_gu, w_down, g_attn, g_ffn = (w[n] for n in ("w_qkv", "w_o", "w_gu", "w_down", "g_attn", "g_ffn"))
@@ -64,8 +68,10 @@ def test_decoder_layer_matches_oracle_chain(exe, batch, fuse):
     d_x, d_cos, d_sin, d_k, d_v = up(x), up(cos), up(sin), up(k_pool), up(v_pool)
     d_n, d_qkv, d_q, d_attn, d_o, d_r1 = (dev(batch * n) for n in (HID, QKV_ROWS, Q_ROWS, HID, HID, HID))
     d_gu, d_gate, d_upb, d_mix, d_down, d_out = (dev(batch * n) for n in (2 * FFN, FFN, FFN, FFN, HID, HID))
+    d_kf, d_vf = dev(batch * KV_ROWS), dev(batch * KV_ROWS)
+    d_k16, d_v16 = exe.allocateScratchBuffer(batch * KV_ROWS * 2), exe.allocateScratchBuffer(batch * KV_ROWS * 2)
     bufs = [d_x, d_cos, d_sin, d_k, d_v, d_n, d_qkv, d_q, d_attn, d_o, d_r1, d_gu, d_gate, d_upb, d_mix,
-            d_down, d_out]
+            d_down, d_out, d_kf, d_vf, d_k16, d_v16]
     tag = f"layer{batch}"
     assert exe.setOption("fuse_row_ops", fuse)
     fused_before = exe.rowProgramLaunches()
@@ -73,8 +79,14 @@ def test_decoder_layer_matches_oracle_chain(exe, batch, fuse):
         assert exe.beginForwardPassCB()
         ok = exe.encodeRmsNormBatched(d_x, g_attn, 1e-5, batch, HID, d_n)
         ok &= exe.encodeMatMulQ4_0Batched(tag + ".attn_qkv", w_qkv, d_n, batch, QKV_ROWS, HID, w_qkv.shape[1], 1, d_qkv)
-        ok &= exe.encodeQkvSplitRopeScatter(d_qkv, d_q, d_k, d_v, d_cos, d_sin, page_ids, slots, P, batch, H,
-                                            HKV, D, QKV_ROWS, Q_ROWS, KV_ROWS, KV_ROWS, D)
+        if kv_calls == "one_call":
+            ok &= exe.encodeQkvSplitRopeScatter(d_qkv, d_q, d_k, d_v, d_cos, d_sin, page_ids, slots, P, batch, H,
+                                                HKV, D, QKV_ROWS, Q_ROWS, KV_ROWS, KV_ROWS, D)
+        else:
+            ok &= exe.encodeQkvSplitRopeCast(d_qkv, d_q, d_kf, d_vf, d_k16, d_v16, d_cos, d_sin, batch, H, HKV, D,
+                                             QKV_ROWS, Q_ROWS, KV_ROWS, KV_ROWS, D)
+            ok &= exe.encodeScatterKVPagedBatched(d_k, page_ids, slots, P, HKV, D, batch, d_k16)
+            ok &= exe.encodeScatterKVPagedBatched(d_v, page_ids, slots, P, HKV, D, batch, d_v16)
         ok &= exe.encodePagedFlashAttention(d_q, d_k, d_v, d_attn, flat, off, seq, qpos, batch, H, HKV, D, P, True)
         ok &= exe.encodeMatMulQ4_0Batched(tag + ".attn_output", w_o, d_attn, batch, HID, HID, w_o.shape[1], 1, d_o)
         ok &= exe.encodeAddBatched(d_x, d_o, d_r1, batch * HID)
