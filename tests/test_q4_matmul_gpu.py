@@ -69,9 +69,10 @@ def make(rows, cols, batch, seed, pad=0, x_scale=1.0):
     return np.ascontiguousarray(q), x, q.shape[1]
 
 
-MFMA_SHAPES = [  # rows, cols, batch: TinyLlama qkv / out-proj / gate_up / down, odd batches
+MFMA_SHAPES = [  # rows, cols, batch: TinyLlama qkv / out-proj / gate_up / down, odd batches, Llama-3-8B
     (2560, 2048, 32), (2048, 2048, 64), (11264, 2048, 64), (2048, 5632, 64),
     (64, 64, 1), (128, 96, 33), (256, 2048, 7), (192, 160, 100),
+    (6144, 4096, 5), (4096, 14336, 3), (28672, 4096, 2),    # Llama-3-8B qkv / down / gate_up
 ]
 
 
