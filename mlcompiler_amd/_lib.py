@@ -4,7 +4,7 @@ from __future__ import annotations
 import ctypes as C
 import os
 
-from .build import LIB_PATH, build_all
+from .build import LIB_PATH, build_all, built_from_current_sources
 
 
 class NativeLibraryError(RuntimeError):
@@ -61,13 +61,16 @@ _lib = None
 
 
 def load(build_if_missing: bool = True) -> C.CDLL:
-    """Loads the native library (building it first only if no built file exists)."""
+    """Loads the native library.  It is built first when no built file exists or when the
+    built file does not come from the sources as they are now (a stale library would be
+    tested silently otherwise); with build_if_missing=False that is an error instead."""
     global _lib
     if _lib is not None:
         return _lib
-    if not os.path.exists(LIB_PATH):
+    if not built_from_current_sources():
         if not build_if_missing:
-            raise NativeLibraryError(f"{LIB_PATH} is missing; run mlcompiler_amd/build.py")
+            raise NativeLibraryError(f"{LIB_PATH} is missing or older than its sources; "
+                                     "run mlcompiler_amd/build.py")
         build_all()
     try:
         lib = C.CDLL(LIB_PATH)

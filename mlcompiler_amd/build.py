@@ -8,6 +8,7 @@
 """
 from __future__ import annotations
 
+import hashlib
 import os
 import shutil
 import subprocess
@@ -17,6 +18,7 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(CSRC, "libmlc_hip.so")
 EXECUTOR_LIB_PATH = os.path.join(CSRC, "libhip_executor.so")
 BENCH_LIB_PATH = os.path.join(CSRC, "libmlc_bench.so")
+STAMP_PATH = os.path.join(CSRC, "libmlc_hip.stamp")   # hash of the sources the libraries were built from
 
 # Packed FP32 instructions (v_pk_*_f32) are switched off on purpose: some of their forms have
 # produced wrong results on the target machines.  hipcc's host pass prints a harmless
@@ -26,6 +28,27 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-fno-honor-nans",
     "-Wno-inline-asm",  # the global->LDS load in paged_prefill_kernels.h names m0 as clobbered
 ]
+
+
+def source_hash() -> str:
+    """Hash over every source the native libraries are built from (and the flags)."""
+    h = hashlib.sha256(" ".join(HIPCC_FLAGS).encode())
+    files = [os.path.join(CSRC, n) for n in sorted(os.listdir(CSRC))
+             if n.endswith((".h", ".hpp", ".hip", ".cpp"))]
+    files.append(os.path.join(os.path.dirname(PKG_DIR), "include", "mlc_hip.h"))
+    for f in files:
+        h.update(os.path.basename(f).encode())
+        with open(f, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()
+
+
+def built_from_current_sources() -> bool:
+    """True when the libraries exist and were built from the sources as they are now."""
+    if not all(os.path.exists(p) for p in (LIB_PATH, EXECUTOR_LIB_PATH, BENCH_LIB_PATH, STAMP_PATH)):
+        return False
+    with open(STAMP_PATH) as fh:
+        return fh.read().strip() == source_hash()
 
 
 def hipcc() -> str:
@@ -46,6 +69,8 @@ def build_all(verbose: bool = False) -> None:
     from concurrent.futures import ThreadPoolExecutor
 
     cc = hipcc()
+    if os.path.exists(STAMP_PATH):
+        os.remove(STAMP_PATH)   # no stamp while the libraries are being replaced
     obj_dir = os.path.join(CSRC, "build")
     os.makedirs(obj_dir, exist_ok=True)
     jobs = []
@@ -63,6 +88,8 @@ def build_all(verbose: bool = False) -> None:
           "-o", EXECUTOR_LIB_PATH, "-L" + CSRC, "-lmlc_hip", "-Wl,-rpath,$ORIGIN"])
     _run([cc, *HIPCC_FLAGS, "-shared", "-x", "hip", os.path.join(CSRC, "bench_loop.cpp"),
           "-o", BENCH_LIB_PATH, "-L" + CSRC, "-lmlc_hip", "-Wl,-rpath,$ORIGIN"])
+    with open(STAMP_PATH, "w") as fh:
+        fh.write(source_hash() + "\n")
     if verbose:
         print("built", LIB_PATH, EXECUTOR_LIB_PATH, BENCH_LIB_PATH)
 

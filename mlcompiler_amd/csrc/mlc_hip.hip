@@ -817,6 +817,11 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
         if ((size_t)page_table_offsets[r] + pages > n_flat)
             return fail("decode: page table does not cover seq_len");
     }
+    {
+        const size_t qo_bytes = batch * num_heads * head_dim * 4;
+        const size_t kq = known_bytes(q), ko = known_bytes(o);
+        if ((kq && qo_bytes > kq) || (ko && qo_bytes > ko)) return fail("decode: q / o buffer too small");
+    }
     const size_t row_bytes = kv_heads * head_dim * 2;
     if (!check_pool_bounds(k_pages, page_tables_flat, page_table_offsets, seq_lens, batch,
                            page_size_tokens, row_bytes, "decode K") ||
@@ -1674,6 +1679,11 @@ int mlc_hip_paged_attn_prefill(const void* q_f16, const void* k_pages, const voi
         const size_t pages = ((size_t)seq_lens[r] + page_size_tokens - 1) / page_size_tokens;
         if ((size_t)page_table_offsets[r] + pages > n_flat)
             return fail("prefill: page table does not cover seq_len");
+    }
+    {
+        const size_t rows = batch * chunk * num_heads * head_dim;
+        const size_t kq = known_bytes(q_f16), ko = known_bytes(o);
+        if ((kq && rows * 2 > kq) || (ko && rows * 4 > ko)) return fail("prefill: q / o buffer too small");
     }
     const size_t row_bytes = kv_heads * head_dim * 2;
     if (!check_pool_bounds(k_pages, page_tables_flat, page_table_offsets, seq_lens, batch,

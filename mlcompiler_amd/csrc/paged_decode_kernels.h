@@ -239,7 +239,8 @@ __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const D
                 uint4* dst = const_cast<uint4*>(is_v ? a.v_pages : a.k_pages);
                 dst[(row * a.kv_heads + it.kv_head) * CPR + cc] = val;
             }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // stores complete (vmcnt 0)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            wait_vmcnt<0>();  // the row has left this wave before any wave of the workgroup loads it
             __syncthreads();
         }
     }
@@ -620,7 +621,11 @@ __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const D
                 st_dev(ml + lane * 2, mh);
                 st_dev(ml + lane * 2 + 1, lh);
             }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // stores complete (vmcnt 0)
+            // The partial must have reached memory before the arrival counter is bumped: the
+            // write-through stores above are complete once this wave's store counter is zero.
+            // (A workgroup-scope release alone emits no such wait on this target.)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            wait_vmcnt<0>();
         };
         // Bumps the arrival counter of slot `slot`; true for the last of `expected` arrivers, which
         // also puts the counter back to zero for the next launch.
@@ -735,7 +740,10 @@ __global__ __launch_bounds__(64 * NW * NS) void paged_decode_fast_kernel(const D
             st_dev(ml + lane * 2 + 1, lh);
         }
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // stores complete (vmcnt 0)
+    // (a workgroup-scope release alone emits no wait on this target: wait for this wave's
+    // write-through stores explicitly, so that whoever wins the ticket finds them in memory)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    wait_vmcnt<0>();
     uint32_t ticket = 0;
     uint32_t* counter = &a.counters[(size_t)it.part_first * NW + hg];
     if (lane == 0)
