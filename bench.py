@@ -474,6 +474,9 @@ def main() -> int:
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU baseline work")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--target-items", type=int, default=0)
+    ap.add_argument("--decode-kernel", type=int, default=0,
+                    help="0 = automatic (tile-balanced kernel), 1 = planned split-K items")
+    ap.add_argument("--wgs-per-cu", type=int, default=0, help="tile-balanced kernel: workgroups per CU (0 = automatic)")
     ap.add_argument("--prefill-stages", type=int, default=0, help="cfg5: LDS pipeline depth (0 = automatic)")
     ap.add_argument("--q4-ksplit", type=int, default=0, help="layer: K slices of the Q4_0 matmuls (0 = automatic)")
     ap.add_argument("--graph", action="store_true",
@@ -497,6 +500,10 @@ def main() -> int:
     exe.requireAvailable()
     if args.target_items:
         exe.setOption("decode_target_items", args.target_items)
+    if args.decode_kernel:
+        assert exe.setOption("decode_kernel", args.decode_kernel)
+    if args.wgs_per_cu:
+        assert exe.setOption("decode_wgs_per_cu", args.wgs_per_cu)
 
     case, n_layers = build_workload(args.workload)
     c = case

@@ -270,9 +270,17 @@ long mlc_hip_fused_matmul_rope_launches(void);
 long mlc_hip_kv_writes_in_decode_launches(void);
 /* Number of fused row-operator launches so far (for tests of "fuse_row_ops"). */
 long mlc_hip_row_program_launches(void);
+/* Number of times so far the decode path copied a page table to the device: the copy is
+ * reused while the table's content stays the same (for tests and benchmarks). */
+long mlc_hip_decode_table_uploads(void);
 
 /* Tunables (0 selects the automatic choice where noted):
- *   "decode_target_items"   split-K work items aimed for per launch (0 = automatic)
+ *   "decode_kernel"         0 = automatic: the tile-balanced kernel (fixed grid, work derived from
+ *                           the tables inside the kernel) wherever it applies; 1 = the planned
+ *                           kernel (host-built split-K work items); 2 = same as 0
+ *   "decode_wgs_per_cu"     workgroups per CU of the tile-balanced kernel's grid (0 = automatic)
+ *   "decode_grid_wgs"       exact grid size of the tile-balanced kernel (0 = from the above; for tests)
+ *   "decode_target_items"   planned kernel: split-K work items aimed for per launch (0 = automatic)
  *   "decode_heads_per_wave" 1, 2, 4 or 8: the most query heads one wavefront handles;
  *                           the GQA group is spread over group/that many waves (0 = automatic)
  *   "decode_tile_rows"      1 or 2: wave rows of a workgroup that share an item's tiles

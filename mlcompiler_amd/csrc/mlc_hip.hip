@@ -21,6 +21,7 @@
 #include "paged_copy_kernels.h"
 #include "paged_decode_generic.h"
 #include "paged_decode_kernels.h"
+#include "paged_decode_stream.h"
 #include "paged_prefill_kernels.h"
 #include "paged_rope_kernels.h"
 #include "walker_kernels.h"
@@ -30,6 +31,10 @@
 namespace mlc_hip {
 // Defined in paged_decode_inst.hip, one object per (head_dim, heads-per-wave).
 #define MLC_DECL(d, h) bool launch_decode_fast_##d##_##h(int, int, int, bool, const DecodeArgs&, hipStream_t);
+MLC_DECL(64, 1) MLC_DECL(64, 2) MLC_DECL(64, 4) MLC_DECL(64, 8)
+MLC_DECL(128, 1) MLC_DECL(128, 2) MLC_DECL(128, 4) MLC_DECL(128, 8)
+#undef MLC_DECL
+#define MLC_DECL(d, h) bool launch_decode_stream_##d##_##h(int, bool, const StreamArgs&, unsigned, size_t, hipStream_t);
 MLC_DECL(64, 1) MLC_DECL(64, 2) MLC_DECL(64, 4) MLC_DECL(64, 8)
 MLC_DECL(128, 1) MLC_DECL(128, 2) MLC_DECL(128, 4) MLC_DECL(128, 8)
 #undef MLC_DECL
@@ -62,6 +67,44 @@ struct MetaSlot {
     size_t cap = 0;
     hipEvent_t done = nullptr;
     bool pending = false;
+};
+
+// Scratch memory of the tile-balanced decode kernel: split-K partials (two slots per workgroup)
+// and arrival counters.  A file-scope device array, so that no entry point that uses it has to
+// allocate; every GPU the library runs on holds its own copy at its own address, which host
+// code learns from hipGetSymbolAddress (the array's name is not a device address in host code).
+// The arrival counters are zero when the module is loaded and every merge puts its counter
+// back to zero.  Launches on one GPU share the array: they must not overlap.
+constexpr size_t kScratchPartOBytes = 8u << 20;
+constexpr size_t kScratchPartMlBytes = 512u << 10;
+constexpr size_t kScratchCounterBytes = (size_t)kStreamMaxWgs * 4 * sizeof(uint32_t);
+constexpr size_t kScratchBytes = kScratchPartOBytes + kScratchPartMlBytes + kScratchCounterBytes;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+// Device copy of the flat page table (and, for batches whose per-request arrays do not fit
+// the kernel arguments, of those arrays) as the tile-balanced decode kernel reads it; uploaded
+// only when the content changes.  A ring of four slots: slot i is rewritten only after the
+// upload into slot i + 1 has completed, which is later in the stream than every launch that
+// read slot i.
+struct StreamTables {
+    struct Slot {
+        void* host = nullptr;
+        void* dev = nullptr;
+        size_t cap = 0;
+        hipEvent_t uploaded = nullptr;
+        bool has_event = false;
+    } slots[4];
+    int cur = -1;
+    std::vector<uint32_t> flat;   // the caller's flat table as last seen
+    uint64_t version = 0;         // counts the changes of `flat`
+    uint64_t uploaded = ~0ull;    // version of `flat` that slots[cur] holds
+    std::vector<uint32_t> meta;   // seq_lens | q_positions | offsets when they are uploaded too
+    size_t meta_off = 0;          // byte offset of the arrays in the slot
+    uint32_t max_page = 0;        // largest page id in flat
+    // does some page id occur in two requests' tables (then a row written for one request may be
+    // read for another)?  -1: not computed for this content
+    int shared_pages = -1;
+    std::vector<uint32_t> off;    // page_table_offsets the shared_pages answer was computed for
 };
 
 struct DecodePlan {
@@ -180,6 +223,12 @@ struct Ctx {
     int last_launches = 0;
     int last_items = 0;
     int n_cu = 256;
+    unsigned char* scratch_ptr = nullptr;   // device address of `scratch` on g.device
+    StreamTables tables;
+    long opt_decode_kernel = 0;     // 0 = automatic (tile-balanced where it applies), 1 = planned items, 2 = tile-balanced
+    long opt_wgs_per_cu = 0;        // tile-balanced kernel: workgroups per CU (0 = automatic)
+    long opt_grid_wgs = 0;          // tile-balanced kernel: exact grid size (0 = from workgroups per CU)
+    long table_uploads = 0;         // page-table uploads of the tile-balanced path (for tests)
 };
 
 Ctx g;
@@ -200,6 +249,13 @@ bool init_once() {
         return false;
     }
     g.n_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    // the device address of the scratch array on this device (see its definition)
+    void* sp = nullptr;
+    if (hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch)) != hipSuccess || !sp) {
+        g_err = "hipGetSymbolAddress(scratch) failed";
+        return false;
+    }
+    g.scratch_ptr = static_cast<unsigned char*>(sp);
     if (hipStreamCreateWithFlags(&g.stream, hipStreamNonBlocking) != hipSuccess) return false;
     if (hipEventCreate(&g.ev0) != hipSuccess || hipEventCreate(&g.ev1) != hipSuccess) return false;
     g.available = true;
@@ -515,13 +571,6 @@ int build_plan(const uint32_t* flat, size_t n_flat, const uint32_t* off, const u
         size_t total_tiles = 0;
         for (size_t r = 0; r < B; ++r) total_tiles += (limits[r] + tile - 1) / tile;
         total_tiles *= Hkv;
-        // Work items (= workgroups) aimed for: as many as are resident at once, which the
-        // 160 KiB of LDS per CU decides (at most 16 waves per CU are counted on).
-        const size_t lds_wg = (size_t)decode_lds_bytes((int)D, p.hpw, p.nw, p.ns, p.nbuf);
-        const size_t per_cu = std::max<size_t>(1, std::min<size_t>(160 * 1024 / lds_wg,
-                                                                   16 / (size_t)(p.nw * p.ns)));
-        const size_t slots = (size_t)g.n_cu * per_cu;
-        (void)slots;
         // About 8 tiles per item, but no fewer than 4 and no more than 16 items per CU
         // (measured optimum on MI355X for 35 MB .. 1.2 GB of KV per call).
         size_t target = std::min<size_t>(std::max<size_t>(total_tiles / 8, (size_t)g.n_cu * 4),
@@ -671,6 +720,164 @@ int check_pool_bounds(const void* pool, const uint32_t* flat, const uint32_t* of
         }
     }
     return 1;
+}
+
+// ---------------------------------------------------------------- tile-balanced decode
+
+// Refreshes what is remembered about the caller's page tables: their content, the largest
+// page id and whether any page id occurs twice (in one table or in two requests' tables).
+// The device copy is brought up to date by tables_upload.
+void tables_refresh(const uint32_t* flat, size_t n_flat, const uint32_t* off, size_t B) {
+    StreamTables& t = g.tables;
+    const bool same_flat = t.flat.size() == n_flat && (n_flat == 0 || std::memcmp(t.flat.data(), flat, n_flat * 4) == 0);
+    const bool same_off = t.off.size() == B + 1 && std::memcmp(t.off.data(), off, (B + 1) * 4) == 0;
+    if (same_flat && same_off && t.shared_pages >= 0) return;
+    if (!same_flat) {
+        ++t.version;
+        t.flat.assign(flat, flat + n_flat);
+        t.max_page = 0;
+        for (size_t i = 0; i < n_flat; ++i) t.max_page = std::max(t.max_page, flat[i]);
+    }
+    t.off.assign(off, off + B + 1);
+    // duplicates among the entries the requests own ([off[r], off[r+1]), a superset of what a
+    // call dereferences): generation-stamped array over the page ids
+    static thread_local std::vector<uint32_t> stamp;
+    static thread_local uint32_t generation = 0;
+    if (stamp.size() <= t.max_page) stamp.assign((size_t)t.max_page + 1, 0);
+    if (++generation == 0) {
+        std::fill(stamp.begin(), stamp.end(), 0u);
+        generation = 1;
+    }
+    t.shared_pages = 0;
+    for (size_t r = 0; r < B && !t.shared_pages; ++r) {
+        const size_t e = std::min<size_t>(off[r + 1], n_flat);
+        for (size_t i = off[r]; i < e; ++i) {
+            uint32_t& st = stamp[flat[i]];
+            if (st == generation) {
+                t.shared_pages = 1;
+                break;
+            }
+            st = generation;
+        }
+    }
+}
+
+// Makes the device copy of the flat table (and of the per-request arrays when `meta3` is
+// given: seq_lens | q_positions | offsets, B each) current.  Returns the device pointer of the
+// table in *d_flat and of the arrays in *d_meta.
+int tables_upload(const uint32_t* meta3, size_t B, const uint32_t** d_flat, const uint32_t** d_meta) {
+    StreamTables& t = g.tables;
+    const size_t n_flat = t.flat.size();
+    const size_t flat_bytes = align_up(std::max<size_t>(n_flat, 1) * 4, 16);
+    const size_t meta_bytes = meta3 ? 3 * B * 4 : 0;
+    // (the table may have changed any number of calls ago: calls that take another kernel
+    // refresh what is remembered but upload nothing)
+    bool upload = t.uploaded != t.version || t.cur < 0;
+    if (meta3) {
+        if (t.meta.size() != 3 * B || std::memcmp(t.meta.data(), meta3, meta_bytes) != 0) upload = true;
+    }
+    if (upload) {
+        const int nxt = (t.cur + 1) % 4;
+        StreamTables::Slot& after = t.slots[(nxt + 1) % 4];
+        if (after.has_event) HIP_OK(hipEventSynchronize(after.uploaded));  // nobody reads slot nxt any more
+        StreamTables::Slot& s = t.slots[nxt];
+        const size_t total = flat_bytes + meta_bytes;
+        if (total > s.cap) {
+            const size_t cap = std::max<size_t>(16384, total * 2);
+            if (s.host) HIP_OK(hipHostFree(s.host));
+            if (s.dev) HIP_OK(hipFree(s.dev));
+            s.host = s.dev = nullptr;
+            s.cap = 0;
+            HIP_OK(hipHostMalloc(&s.host, cap, hipHostMallocDefault));
+            HIP_OK(hipMalloc(&s.dev, cap));
+            s.cap = cap;
+        }
+        if (!s.uploaded) HIP_OK(hipEventCreateWithFlags(&s.uploaded, hipEventDisableTiming));
+        if (n_flat) std::memcpy(s.host, t.flat.data(), n_flat * 4);
+        if (meta3) {
+            std::memcpy(static_cast<char*>(s.host) + flat_bytes, meta3, meta_bytes);
+            t.meta.assign(meta3, meta3 + 3 * B);
+        } else {
+            t.meta.clear();
+        }
+        HIP_OK(hipMemcpyAsync(s.dev, s.host, total, hipMemcpyHostToDevice, g.stream));
+        HIP_OK(hipEventRecord(s.uploaded, g.stream));
+        s.has_event = true;
+        t.cur = nxt;
+        t.uploaded = t.version;
+        t.meta_off = flat_bytes;
+        ++g.table_uploads;
+    }
+    const char* dev = static_cast<const char*>(t.slots[t.cur].dev);
+    *d_flat = reinterpret_cast<const uint32_t*>(dev);
+    *d_meta = meta3 ? reinterpret_cast<const uint32_t*>(dev + t.meta_off) : nullptr;
+    return 1;
+}
+
+// Shape of the tile-balanced launch for (G, D): query heads per wave, waves per workgroup;
+// false when the kernel does not cover the shape.
+bool stream_variant(size_t G, size_t D, int* hpw_out, int* nw_out) {
+    if (D != 64 && D != 128) return false;
+    const long hpw_cap = g.opt_hpw_max > 0 ? g.opt_hpw_max : std::max<long>(1, (long)G / 4);
+    int hpw = 8;
+    while (hpw > 1 && (hpw > hpw_cap || (G % (size_t)hpw) != 0)) hpw >>= 1;
+    size_t nw = G / (size_t)hpw;
+    if (nw > 4 || nw == 3) {
+        hpw = 8;
+        while (hpw > 1 && (G % (size_t)hpw) != 0) hpw >>= 1;
+        nw = G / (size_t)hpw;
+    }
+    if (nw > 4 || nw == 3) return false;
+    if (stream_static_lds_bytes((int)D, (int)G) > 60 * 1024) return false;
+    *hpw_out = hpw;
+    *nw_out = (int)nw;
+    return true;
+}
+
+// Grid of the tile-balanced kernel: as many workgroups as stay resident (LDS decides), within
+// what the scratch array holds.
+unsigned stream_grid(size_t G, size_t D, size_t dyn_lds) {
+    const size_t lds = (size_t)stream_static_lds_bytes((int)D, (int)G) + dyn_lds;
+    size_t per_cu = std::max<size_t>(1, std::min<size_t>(160 * 1024 / lds, 3));
+    if (g.opt_wgs_per_cu > 0) per_cu = (size_t)g.opt_wgs_per_cu;
+    size_t W = (size_t)g.n_cu * per_cu;
+    if (g.opt_grid_wgs > 0) W = (size_t)g.opt_grid_wgs;
+    W = std::min<size_t>(W, kStreamMaxWgs);
+    W = std::min<size_t>(W, kScratchPartOBytes / (2 * G * D * 4));
+    W = std::min<size_t>(W, kScratchPartMlBytes / (2 * G * 2 * 4));
+    return (unsigned)std::max<size_t>(W, 1);
+}
+
+bool launch_stream_variant(size_t D, int hpw, int nw, const StreamArgs& a, unsigned n_wg, size_t dyn_lds) {
+    const bool pv16 = g.opt_pv_fp16 != 0;
+#define MLC_CASE(d, h) \
+    if (D == d && hpw == h) return launch_decode_stream_##d##_##h(nw, pv16, a, n_wg, dyn_lds, g.stream);
+    MLC_CASE(64, 1) MLC_CASE(64, 2) MLC_CASE(64, 4) MLC_CASE(64, 8)
+    MLC_CASE(128, 1) MLC_CASE(128, 2) MLC_CASE(128, 4) MLC_CASE(128, 8)
+#undef MLC_CASE
+    return false;
+}
+
+void stream_fill_common(StreamArgs& a, const void* q, const void* k_pages, const void* v_pages, void* o,
+                        size_t B, size_t H, size_t Hkv, size_t D, size_t P, int causal) {
+    a.q = static_cast<const float*>(q);
+    a.k_pages = static_cast<const uint4*>(k_pages);
+    a.v_pages = static_cast<const uint4*>(v_pages);
+    a.o = static_cast<float*>(o);
+    a.part_o = reinterpret_cast<float*>(g.scratch_ptr);
+    a.part_ml = reinterpret_cast<float*>(g.scratch_ptr + kScratchPartOBytes);
+    a.counters = reinterpret_cast<uint32_t*>(g.scratch_ptr + kScratchPartOBytes + kScratchPartMlBytes);
+    a.batch = (uint32_t)B;
+    a.num_heads = (uint32_t)H;
+    a.kv_heads = (uint32_t)Hkv;
+    a.page_size = (uint32_t)P;
+    a.causal = causal ? 1u : 0u;
+    a.capacity_pages = 0;
+    a.meta = nullptr;
+    a.meta_stride = 0;
+    a.scale_log2e = (1.0f / std::sqrt(static_cast<float>(D))) * 1.44269504088896340736f;
+    a.new_k = a.new_v = nullptr;
+    a.new_ids = a.new_slots = nullptr;
 }
 
 }  // namespace
@@ -823,24 +1030,58 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
         if ((kq && qo_bytes > kq) || (ko && qo_bytes > ko)) return fail("decode: q / o buffer too small");
     }
     const size_t row_bytes = kv_heads * head_dim * 2;
-    if (!check_pool_bounds(k_pages, page_tables_flat, page_table_offsets, seq_lens, batch,
-                           page_size_tokens, row_bytes, "decode K") ||
-        !check_pool_bounds(v_pages, page_tables_flat, page_table_offsets, seq_lens, batch,
-                           page_size_tokens, row_bytes, "decode V"))
-        return 0;
-
+    // What is remembered about the tables (content, largest page id, repeated page ids) is
+    // refreshed only when they changed; the walker passes the same tables for every layer of a
+    // step (compiler/runtime/batched_walker.cpp:316-325).
+    tables_refresh(page_tables_flat, n_flat, page_table_offsets, batch);
+    {
+        // pools this library allocated: no page id of the table may lie beyond them.  The largest
+        // id of the whole table decides at once; only if that one is too large (it may sit in a
+        // part of the table no request uses) the pages in use are checked one by one.
+        const size_t page_bytes = page_size_tokens * row_bytes;
+        const size_t kk = known_bytes(k_pages), kv = known_bytes(v_pages);
+        const size_t need = n_flat ? ((size_t)g.tables.max_page + 1) * page_bytes : 0;
+        if (((kk && need > kk) || (kv && need > kv)) &&
+            (!check_pool_bounds(k_pages, page_tables_flat, page_table_offsets, seq_lens, batch,
+                                page_size_tokens, row_bytes, "decode K") ||
+             !check_pool_bounds(v_pages, page_tables_flat, page_table_offsets, seq_lens, batch,
+                                page_size_tokens, row_bytes, "decode V")))
+            return 0;
+    }
     const bool aligned = aligned16(q) && aligned16(k_pages) && aligned16(v_pages) && aligned16(o);
-    if (!build_plan(page_tables_flat, n_flat, page_table_offsets, seq_lens, q_positions, batch,
-                    num_heads, kv_heads, head_dim, page_size_tokens, apply_causal ? 1 : 0, aligned))
-        return 0;
-    const DecodePlan& p = g.plan;
-    MetaSlot& slot = g.plan_slots[p.slot];
-    const char* dev = static_cast<const char*>(slot.dev);
-    const float scale_log2e = (1.0f / std::sqrt(static_cast<float>(head_dim))) * 1.44269504088896340736f;
+    const size_t G = num_heads / kv_heads;
+    const size_t tile = (head_dim == 64) ? 64 : 32;
+
+    // ---- which kernel: the tile-balanced one wherever it applies
+    int s_hpw = 0, s_nw = 0;
+    bool use_stream = g.opt_decode_kernel != 1 && !g.opt_force_generic && aligned &&
+                      (page_size_tokens % tile) == 0 && batch <= kStreamMaxBatch &&
+                      stream_variant(G, head_dim, &s_hpw, &s_nw);
+    uint64_t total_tiles = 0;
+    if (use_stream) {
+        for (size_t r = 0; r < batch; ++r) {
+            uint64_t lim = seq_lens[r];
+            if (apply_causal && (uint64_t)q_positions[r] + 1 < lim) lim = (uint64_t)q_positions[r] + 1;  // :2286
+            total_tiles += (lim + tile - 1) / tile;
+        }
+        total_tiles *= kv_heads;
+        if (total_tiles >= 0x7FFFFFFFull) use_stream = false;
+    }
+    const DecodePlan* plan = nullptr;
+    if (!use_stream) {
+        if (!build_plan(page_tables_flat, n_flat, page_table_offsets, seq_lens, q_positions, batch,
+                        num_heads, kv_heads, head_dim, page_size_tokens, apply_causal ? 1 : 0, aligned))
+            return 0;
+        plan = &g.plan;
+    }
+
     if (carries_kv) {
-        // only the tiled kernel writes rows, and only rows that are every request's newest
-        // visible position: then exactly one work item reads each of them, after writing it
-        carries_kv = p.fast;
+        // Only the tiled kernels write rows, and only rows that are every request's newest
+        // visible position: then exactly one workgroup reads each of them, after writing it.
+        // That also needs every page to belong to one request (and to appear once in its
+        // table): with a repeated page id another workgroup could read the row while it is
+        // being written, and the separate launches are the ones that give the order of the calls.
+        carries_kv = (use_stream || plan->fast) && g.tables.shared_pages == 0;
         for (size_t r = 0; carries_kv && r < batch; ++r) {
             const uint64_t S = seq_lens[r];
             const bool visible = !apply_causal || (uint64_t)q_positions[r] + 1 >= S;
@@ -851,9 +1092,67 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
     }
 
     g.last_launches = 0;
+    if (use_stream) {
+        // per-request arrays: inside the kernel arguments when they fit, else uploaded with the table
+        const bool embed = batch <= kStreamEmbBatch;
+        static thread_local std::vector<uint32_t> meta3;
+        if (!embed) {
+            meta3.resize(3 * batch);
+            std::memcpy(meta3.data(), seq_lens, batch * 4);
+            std::memcpy(meta3.data() + batch, q_positions, batch * 4);
+            std::memcpy(meta3.data() + 2 * batch, page_table_offsets, batch * 4);
+        }
+        const uint32_t* d_flat = nullptr;
+        const uint32_t* d_meta = nullptr;
+        if (!tables_upload(embed ? nullptr : meta3.data(), batch, &d_flat, &d_meta)) return 0;
+        const size_t dyn_lds = stream_dynamic_lds_bytes(batch);
+        const unsigned n_wg = stream_grid(G, head_dim, dyn_lds);
+        StreamArgs a;
+        stream_fill_common(a, q, k_pages, v_pages, o, batch, num_heads, kv_heads, head_dim, page_size_tokens,
+                           apply_causal);
+        a.pt_flat = d_flat;
+        {
+            // pools this library allocated: the kernel clamps page ids below their size (the host
+            // checks above already refuse such tables; the clamp keeps a stale or overwritten
+            // table from turning into a stray access)
+            const size_t page_bytes = page_size_tokens * row_bytes;
+            const size_t kk = known_bytes(k_pages), kv = known_bytes(v_pages);
+            size_t pages = std::min(kk ? kk / page_bytes : SIZE_MAX, kv ? kv / page_bytes : SIZE_MAX);
+            if (pages != SIZE_MAX) a.capacity_pages = (uint32_t)std::min<size_t>(pages, 0xFFFFFFFFu);
+        }
+        if (embed) {
+            std::memcpy(a.emb, seq_lens, batch * 4);
+            std::memcpy(a.emb + kStreamEmbBatch, q_positions, batch * 4);
+            std::memcpy(a.emb + 2 * kStreamEmbBatch, page_table_offsets, batch * 4);
+        } else {
+            a.meta = d_meta;
+            a.meta_stride = (uint32_t)batch;
+        }
+        if (carries_kv) {
+            a.new_k = static_cast<const uint4*>(g.kv.src[0]);
+            a.new_v = static_cast<const uint4*>(g.kv.src[1]);
+            a.new_ids = g.kv.d_ids;
+            a.new_slots = g.kv.d_slots;
+        }
+        if (!launch_stream_variant(head_dim, s_hpw, s_nw, a, n_wg, dyn_lds))
+            return fail("decode: kernel variant not built");
+        g.last_items = (int)std::min<uint64_t>(n_wg, total_tiles);
+        if (carries_kv) {
+            g.kv.active = false;
+            ++g.kv_fused;
+            ++g.kv_in_decode;
+        }
+        ++g.last_launches;
+        return finish(sync);
+    }
+
+    const DecodePlan& p = *plan;
+    MetaSlot& slot = g.plan_slots[p.slot];
+    const char* dev = static_cast<const char*>(slot.dev);
+    const float scale_log2e = (1.0f / std::sqrt(static_cast<float>(head_dim))) * 1.44269504088896340736f;
     g.last_items = (int)p.n_items;
     if (p.fast) {
-        if (p.n_part && !ensure_partials(p.n_part, num_heads / kv_heads, head_dim, (size_t)p.nw))
+        if (p.n_part && !ensure_partials(p.n_part, G, head_dim, (size_t)p.nw))
             return 0;
         DecodeArgs a;
         a.q = static_cast<const float*>(q);
@@ -879,7 +1178,7 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
             a.new_slots = g.kv.d_slots;
         }
         if (!launch_fast(head_dim, p.hpw, p.nw, p.ns, p.nbuf, a)) return fail("decode: kernel variant not built");
-        if (carries_kv) {  // (pages are not shared between requests, paged_kv.hpp:61-64: nobody else reads those rows)
+        if (carries_kv) {
             g.kv.active = false;
             ++g.kv_fused;
             ++g.kv_in_decode;
@@ -1757,6 +2056,7 @@ long mlc_hip_fused_kv_write_launches(void) { return g.kv_fused; }
 long mlc_hip_fused_matmul_rope_launches(void) { return g.gemm_rope_fused; }
 long mlc_hip_kv_writes_in_decode_launches(void) { return g.kv_in_decode; }
 long mlc_hip_row_program_launches(void) { return g.row_launches; }
+long mlc_hip_decode_table_uploads(void) { return g.table_uploads; }
 
 int mlc_hip_set_option(const char* name, long value) {
     if (!name) return 0;
@@ -1764,6 +2064,21 @@ int mlc_hip_set_option(const char* name, long value) {
     if (!std::strcmp(name, "fuse_row_ops")) { g.opt_fuse_rows = value ? 1 : 0; return 1; }
     if (!std::strcmp(name, "decode_target_items")) { g.opt_target_items = value; return 1; }
     if (!std::strcmp(name, "decode_force_generic")) { g.opt_force_generic = value; return 1; }
+    if (!std::strcmp(name, "decode_kernel")) {
+        if (value < 0 || value > 2) return 0;
+        g.opt_decode_kernel = value;
+        return 1;
+    }
+    if (!std::strcmp(name, "decode_grid_wgs")) {
+        if (value < 0 || value > (long)kStreamMaxWgs) return 0;
+        g.opt_grid_wgs = value;
+        return 1;
+    }
+    if (!std::strcmp(name, "decode_wgs_per_cu")) {
+        if (value < 0 || value > 8) return 0;
+        g.opt_wgs_per_cu = value;
+        return 1;
+    }
     if (!std::strcmp(name, "decode_pv_fp16")) { g.opt_pv_fp16 = value ? 1 : 0; return 1; }
     if (!std::strcmp(name, "q4_force_generic")) { g.opt_q4_force_generic = value ? 1 : 0; return 1; }
     if (!std::strcmp(name, "q4_ksplit")) {

@@ -11,8 +11,9 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("c", list(load_attention_cases()), ids=lambda c: f"H{c['H']}kv{c['Hkv']}D{c['D']}S{c['S']}")
-@pytest.mark.parametrize("generic", [0, 1], ids=["fast", "generic"])
-def test_decode_matches_golden_reference_outputs(exe, c, generic):
+@pytest.mark.parametrize("kernel", ["balanced", "planned", "generic"])
+def test_decode_matches_golden_reference_outputs(exe, c, kernel):
+    generic = 1 if kernel == "generic" else 0
     P, S = c["P"], c["S"]
     pool_pages = c["k"].size // (P * c["Hkv"] * c["D"])
     case = DecodeCase(name="golden", batch=1, num_heads=c["H"], kv_heads=c["Hkv"], head_dim=c["D"],
@@ -21,14 +22,16 @@ def test_decode_matches_golden_reference_outputs(exe, c, generic):
                       page_tables_flat=c["pt"].astype(np.uint32),
                       page_table_offsets=np.array([0, c["pt"].size], np.uint32), apply_causal=True,
                       q=c["q"].reshape(1, c["H"], c["D"]), k_pages=c["k"], v_pages=c["v"])
-    print(f"[golden] H={c['H']}/{c['Hkv']} D={c['D']} S={S} P={P} generic={generic}", flush=True)
+    print(f"[golden] H={c['H']}/{c['Hkv']} D={c['D']} S={S} P={P} kernel={kernel}", flush=True)
     assert exe.setOption("decode_force_generic", generic)
+    assert exe.setOption("decode_kernel", 1 if kernel == "planned" else 0)
     dev = DeviceCase(exe, case)
     try:
         got = dev.run(sync=True)
     finally:
         dev.free()
         exe.setOption("decode_force_generic", 0)
+        exe.setOption("decode_kernel", 0)
     assert_parity(got.reshape(1, c["H"], c["D"]), c["o"].reshape(1, c["H"], c["D"]), c["D"], "golden")
 
 

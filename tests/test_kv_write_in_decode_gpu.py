@@ -22,12 +22,14 @@ def _newest(case):
     return ids, (last % case.page_size).astype(np.uint32)
 
 
-def _step(exe, case, ids, slots, new_k, new_v, fuse, *, only_k=False, target=0):
+def _step(exe, case, ids, slots, new_k, new_v, fuse, *, only_k=False, target=0, kernel="balanced"):
     """scatter K, scatter V, attention in one open pass -> (output, K pool, V pool, launches that carried the write)"""
     dev = DeviceCase(exe, case)
     nk, nv = (exe.allocateScratchBuffer(a.nbytes) for a in (new_k, new_v))
     assert exe.uploadToBuffer(nk, new_k) and exe.uploadToBuffer(nv, new_v)
-    assert exe.setOption("fuse_row_ops", fuse) and exe.setOption("decode_target_items", target)
+    split = "decode_target_items" if kernel == "planned" else "decode_grid_wgs"
+    assert exe.setOption("decode_kernel", 1 if kernel == "planned" else 0)
+    assert exe.setOption("fuse_row_ops", fuse) and exe.setOption(split, target)
     before = exe.kvWritesInDecodeLaunches()
     c = case
     try:
@@ -45,7 +47,8 @@ def _step(exe, case, ids, slots, new_k, new_v, fuse, *, only_k=False, target=0):
         assert exe.downloadFromBuffer(dev.k_buf, kp) and exe.downloadFromBuffer(dev.v_buf, vp)
     finally:
         exe.setOption("fuse_row_ops", 1)
-        exe.setOption("decode_target_items", 0)
+        exe.setOption(split, 0)
+        exe.setOption("decode_kernel", 0)
         dev.free()
         exe.releaseScratchBuffer(nk)
         exe.releaseScratchBuffer(nv)
@@ -67,8 +70,11 @@ def _rows(case, seed):
 
 
 @pytest.mark.parametrize("shape", [(8, 2, 64), (32, 4, 64), (32, 8, 128), (8, 8, 64)], ids=["g4d64", "g8d64", "g4d128", "mha"])
-@pytest.mark.parametrize("target", [0, 100000, 1], ids=["auto", "many_splits", "no_splits"])
-def test_attention_launch_carries_the_kv_write(exe, shape, target):
+@pytest.mark.parametrize("kernel,target", [("planned", 0), ("planned", 100000), ("planned", 1),
+                                           ("balanced", 0), ("balanced", 2048), ("balanced", 1), ("balanced", 5)],
+                         ids=["planned_auto", "planned_many_splits", "planned_no_splits", "balanced_auto",
+                              "balanced_many_splits", "balanced_one_workgroup", "balanced_five_workgroups"])
+def test_attention_launch_carries_the_kv_write(exe, shape, kernel, target):
     h, hkv, d = shape
     lens = [1, 64, 65, 130, 700, 2000, 63, 128]     # newest position at page starts, page ends, mid-page
     case = make_case("kvstep", len(lens), h, hkv, d, 64, lens, seed=3 + d, capacity_pages=64)
@@ -76,8 +82,8 @@ def test_attention_launch_carries_the_kv_write(exe, shape, target):
     new_k, new_v = _rows(case, 17)
     want_k, want_v, want_o = _expect(case, ids, slots, new_k, new_v)
     print(f"[case] kv write in decode {shape} target={target}", flush=True)
-    plain = _step(exe, case, ids, slots, new_k, new_v, 0, target=target)
-    fused = _step(exe, case, ids, slots, new_k, new_v, 1, target=target)
+    plain = _step(exe, case, ids, slots, new_k, new_v, 0, target=target, kernel=kernel)
+    fused = _step(exe, case, ids, slots, new_k, new_v, 1, target=target, kernel=kernel)
     assert plain[3] == 0 and fused[3] == 1
     for got in (plain, fused):
         assert np.array_equal(got[1], want_k) and np.array_equal(got[2], want_v)
@@ -85,7 +91,8 @@ def test_attention_launch_carries_the_kv_write(exe, shape, target):
     assert np.array_equal(plain[0], fused[0])      # the same kernel did the arithmetic
 
 
-def test_other_rows_are_written_by_their_own_launch(exe):
+@pytest.mark.parametrize("kernel", ["balanced", "planned"])
+def test_other_rows_are_written_by_their_own_launch(exe, kernel):
     case = make_case("kvstep_other", 4, 8, 2, 64, 64, [70, 200, 64, 129], seed=9, capacity_pages=16)
     ids, slots = _newest(case)
     new_k, new_v = _rows(case, 5)
@@ -96,7 +103,7 @@ def test_other_rows_are_written_by_their_own_launch(exe):
     case_b = replace(case, q_positions=np.array([69, 199, 10, 128], np.uint32))
     for c, sl, only_k in ((case, slots_a, False), (case_b, slots, False), (case, slots, True)):
         want_k, want_v, want_o = _expect(c, ids, sl, new_k, new_v, only_k)
-        out, kp, vp, carried = _step(exe, c, ids, sl, new_k, new_v, 1, only_k=only_k)
+        out, kp, vp, carried = _step(exe, c, ids, sl, new_k, new_v, 1, only_k=only_k, kernel=kernel)
         assert carried == 0
         assert np.array_equal(kp, want_k) and np.array_equal(vp, want_v)
         assert_parity(out, want_o, 64, "kv step, separate launches")
@@ -118,10 +125,35 @@ def test_kv_write_and_two_level_merge_in_every_kernel_variant(exe, opts):
     for name, value in opts.items():
         assert exe.setOption(name, value)
     try:
-        out, kp, vp, carried = _step(exe, case, ids, slots, new_k, new_v, 1, target=opts.get("decode_target_items", 0))
+        out, kp, vp, carried = _step(exe, case, ids, slots, new_k, new_v, 1, target=opts.get("decode_target_items", 0),
+                                     kernel="planned")
     finally:
         for name in opts:
             exe.setOption(name, 1 if name == "decode_tile_rows" else 0)
     assert carried == 1
     assert np.array_equal(kp, want_k) and np.array_equal(vp, want_v)
     assert_parity(out, want_o, 64, f"kv step {opts}")
+
+
+@pytest.mark.parametrize("kernel", ["balanced", "planned"])
+def test_a_shared_page_keeps_the_launches_apart(exe, kernel):
+    """Two requests whose tables name the same physical page (the reference's allocator never
+    does that, the interface does not forbid it): the row written for one request is then also
+    read for the other, so the attention launch must not take the write; the three launches run
+    one after the other and give what the calls in their order give."""
+    case = make_case("kvstep_shared", 3, 8, 2, 64, 64, [130, 100, 70], seed=31, capacity_pages=16)
+    flat = case.page_tables_flat.copy()
+    off = case.page_table_offsets
+    flat[off[1] + 1] = flat[off[0] + 2]       # request 1's last page is request 0's last page
+    case = replace(case, page_tables_flat=flat)
+    ids, slots = _newest(case)
+    new_k, new_v = _rows(case, 41)
+    want_k, want_v, want_o = _expect(case, ids, slots, new_k, new_v)
+    out, kp, vp, carried = _step(exe, case, ids, slots, new_k, new_v, 1, kernel=kernel)
+    assert carried == 0
+    assert np.array_equal(kp, want_k) and np.array_equal(vp, want_v)
+    assert_parity(out, want_o, 64, "kv step, shared page")
+    # the same tables without the repeated page: the attention launch takes the write again
+    case2 = make_case("kvstep_unshared", 3, 8, 2, 64, 64, [130, 100, 70], seed=31, capacity_pages=16)
+    ids2, slots2 = _newest(case2)
+    assert _step(exe, case2, ids2, slots2, new_k, new_v, 1, kernel=kernel)[3] == 1

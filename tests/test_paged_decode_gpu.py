@@ -10,6 +10,20 @@ from paged_cases import (DeviceCase, assert_parity, baseline_config, make_case, 
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(params=["balanced", "planned"], autouse=True)
+def decode_kernel(exe, request):
+    """Every test runs on both tiled decode kernels: the tile-balanced one (fixed grid, work
+    derived from the tables in the kernel; the default) and the planned one (host-built items)."""
+    assert exe.setOption("decode_kernel", 1 if request.param == "planned" else 0)
+    yield request.param
+    exe.setOption("decode_kernel", 0)
+
+
+# how each kernel's split of the work is varied: items aimed for / exact grid size
+def _split_option(kernel):
+    return "decode_target_items" if kernel == "planned" else "decode_grid_wgs"
+
+
 def _check(exe, case, sync=True):
     print(f"[case] {case.name} B={case.batch} H={case.num_heads}/{case.kv_heads} D={case.head_dim} "
           f"P={case.page_size} causal={case.apply_causal}", flush=True)
@@ -78,6 +92,18 @@ def test_other_shapes(exe, head_dim, page):
     _check(exe, case)
 
 
+@pytest.mark.parametrize("batch", [65, 70, 300, 1000])
+def test_large_batches(exe, batch):
+    # more requests than one wavefront has lanes (two-level search over the tile prefix), and
+    # more than travel inside the kernel arguments (per-request arrays uploaded with the table);
+    # many requests of one tile or none, so that a workgroup's range holds many pairs
+    rng = np.random.default_rng(batch)
+    lens = rng.integers(0, 200, batch)
+    lens[rng.random(batch) < 0.2] = 0
+    lens[3] = 1500
+    _check(exe, make_case(f"b{batch}", batch, 8, 2, 64, 64, lens, seed=batch))
+
+
 def test_edge_lengths(exe):
     # empty request, single token, exactly one page, page + 1, one tile + 1
     case = make_case("edges", 6, 32, 4, 64, 64, [0, 1, 64, 65, 63, 129])
@@ -133,13 +159,14 @@ def test_page_permutation_invariance(exe):
     assert np.array_equal(got_a, got_b)
 
 
-def test_split_k_targets_agree(exe):
-    # the same batch planned as 1 item per (request, kv head) and as many small items
+def test_split_k_targets_agree(exe, decode_kernel):
+    # the same batch as one piece of work, as a few, and as many small pieces
     case = baseline_config(2, batch=6)
     want = oracle_decode(case)
     outs = []
-    for target in (1, 64, 100000):
-        assert exe.setOption("decode_target_items", target)
+    opt = _split_option(decode_kernel)
+    for target in ((1, 64, 100000) if decode_kernel == "planned" else (1, 7, 2048)):
+        assert exe.setOption(opt, target)
         dev = DeviceCase(exe, case)
         try:
             outs.append(dev.run())
@@ -147,7 +174,7 @@ def test_split_k_targets_agree(exe):
         finally:
             dev.free()
         assert_parity(outs[-1], want, 64, f"target={target}")
-    exe.setOption("decode_target_items", 0)
+    exe.setOption(opt, 0)
     # splits differ only by rounding (fp32 sums in another order, fp16 softmax weights)
     assert np.max(np.abs(outs[0] - outs[2])) < 3e-4, np.max(np.abs(outs[0] - outs[2]))
 
@@ -155,7 +182,7 @@ def test_split_k_targets_agree(exe):
 @pytest.mark.parametrize("shape", [(32, 8, 128, [8192 + 17, 3001]), (32, 4, 64, [5000, 1100, 70]),
                                    (8, 8, 64, [16384 + 1])],
                          ids=["d128", "d64", "mha"])
-def test_many_splits_merge_in_two_levels(exe, shape):
+def test_many_splits_merge_in_two_levels(exe, shape, decode_kernel):
     """Few long requests: each (request, KV head) is cut into far more than the 16 partials one
     wave merges at once, so groups of partials are merged first and the groups' results after
     them (also with a last group of one partial).  Planned automatically, with one tile per item,
@@ -166,18 +193,20 @@ def test_many_splits_merge_in_two_levels(exe, shape):
     want = oracle_decode(case)
     dev = DeviceCase(exe, case)
     outs = {}
+    opt = _split_option(decode_kernel)
+    big = 1000000 if decode_kernel == "planned" else 2048   # balanced: up to 2048 partials of one pair
     try:
-        for target in (0, 1000000, 1):
-            assert exe.setOption("decode_target_items", target)
+        for target in (0, big, 1):
+            assert exe.setOption(opt, target)
             for rep in range(2):
                 got = dev.run()
                 print("target", target, "items", exe.lastDecodeWorkItems(), flush=True)
                 assert_parity(got, want, dim, f"target={target} rep={rep}")
             outs[target] = got
     finally:
-        exe.setOption("decode_target_items", 0)
+        exe.setOption(opt, 0)
         dev.free()
-    assert np.max(np.abs(outs[1000000] - outs[1])) < 1e-3
+    assert np.max(np.abs(outs[big] - outs[1])) < 1e-3
 
 
 def test_generic_kernel_agrees_with_fast(exe):
@@ -206,6 +235,20 @@ def test_plan_cache_across_layers_and_steps(exe):
     c3 = baseline_config(2, batch=4, seed=2)
     _check(exe, c3)
     _check(exe, c1)
+
+
+def test_kernels_alternate_on_changing_tables(exe):
+    """The device copy of the page table belongs to the tile-balanced kernel; calls that take
+    the planned kernel in between must not make it look current when it is not."""
+    a = make_case("alt_a", 3, 8, 2, 64, 64, [300, 70, 129], capacity_pages=16, seed=61)
+    b = make_case("alt_b", 3, 8, 2, 64, 64, [300, 70, 129], capacity_pages=16, seed=62)   # other page ids
+    assert not np.array_equal(a.page_tables_flat, b.page_tables_flat)
+    try:
+        for case, kernel in ((a, 0), (b, 1), (b, 0), (a, 1), (a, 0)):
+            assert exe.setOption("decode_kernel", kernel)
+            _check(exe, case)
+    finally:
+        exe.setOption("decode_kernel", 0)
 
 
 def test_stress_online_rescale(exe):
@@ -272,7 +315,7 @@ def test_bad_arguments_are_rejected(exe):
 
 
 @pytest.mark.timeout(600)
-def test_baseline_config4_full_size(exe):
+def test_baseline_config4_full_size(exe, decode_kernel):
     """Llama-3-8B shape at its full size (batch 64, 16384-page pool, 1.16 GB of KV per call).
     The oracle is too slow for all of it, so: (1) four sampled requests are checked against the
     oracle on the same pool, (2) a second run with a different split-K plan must agree with the
@@ -285,11 +328,11 @@ def test_baseline_config4_full_size(exe):
     try:
         got = dev.run(sync=True)
         items_auto = exe.lastDecodeWorkItems()
-        assert exe.setOption("decode_target_items", 1536)
+        assert exe.setOption(_split_option(decode_kernel), 1536)
         again = dev.run(sync=True)
         assert exe.lastDecodeWorkItems() != items_auto
     finally:
-        exe.setOption("decode_target_items", 0)
+        exe.setOption(_split_option(decode_kernel), 0)
         dev.free()
     assert np.all(np.isfinite(got))
     # the softmax weights are rounded to fp16 (relative 2^-11) against the running maximum of
