@@ -477,6 +477,9 @@ def main() -> int:
     ap.add_argument("--decode-kernel", type=int, default=0,
                     help="0 = automatic (tile-balanced kernel), 1 = planned split-K items")
     ap.add_argument("--wgs-per-cu", type=int, default=0, help="tile-balanced kernel: workgroups per CU (0 = automatic)")
+    ap.add_argument("--stages", type=int, default=0, help="tile-balanced kernel: LDS stages (0 = automatic)")
+    ap.add_argument("--opt", action="append", default=[], metavar="NAME=VALUE",
+                    help="library tunable (mlc_hip_set_option), may be repeated")
     ap.add_argument("--prefill-stages", type=int, default=0, help="cfg5: LDS pipeline depth (0 = automatic)")
     ap.add_argument("--q4-ksplit", type=int, default=0, help="layer: K slices of the Q4_0 matmuls (0 = automatic)")
     ap.add_argument("--graph", action="store_true",
@@ -504,6 +507,11 @@ def main() -> int:
         assert exe.setOption("decode_kernel", args.decode_kernel)
     if args.wgs_per_cu:
         assert exe.setOption("decode_wgs_per_cu", args.wgs_per_cu)
+    if args.stages:
+        assert exe.setOption("decode_stages", args.stages)
+    for kv in args.opt:
+        name, value = kv.split("=")
+        assert exe.setOption(name, int(value)), f"unknown option {kv}"
 
     case, n_layers = build_workload(args.workload)
     c = case

@@ -279,6 +279,8 @@ long mlc_hip_decode_table_uploads(void);
  *                           the tables inside the kernel) wherever it applies; 1 = the planned
  *                           kernel (host-built split-K work items); 2 = same as 0
  *   "decode_wgs_per_cu"     workgroups per CU of the tile-balanced kernel's grid (0 = automatic)
+ *   "decode_stages"         2, 3 or 4 K/V tiles staged in LDS per workgroup of the tile-balanced kernel
+ *                           (0 = automatic: 2; batches above 64 requests take 3 at most)
  *   "decode_grid_wgs"       exact grid size of the tile-balanced kernel (0 = from the above; for tests)
  *   "decode_target_items"   planned kernel: split-K work items aimed for per launch (0 = automatic)
  *   "decode_heads_per_wave" 1, 2, 4 or 8: the most query heads one wavefront handles;

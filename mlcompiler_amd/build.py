@@ -30,6 +30,10 @@ HIPCC_FLAGS = [
 ]
 
 
+# extra compiler flags for experiments (for example -DMLC_STREAM_PROBE: time stamps per workgroup)
+HIPCC_FLAGS += os.environ.get("MLC_HIPCC_EXTRA", "").split()
+
+
 def source_hash() -> str:
     """Hash over every source the native libraries are built from (and the flags)."""
     h = hashlib.sha256(" ".join(HIPCC_FLAGS).encode())

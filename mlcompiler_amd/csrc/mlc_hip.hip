@@ -34,7 +34,7 @@ namespace mlc_hip {
 MLC_DECL(64, 1) MLC_DECL(64, 2) MLC_DECL(64, 4) MLC_DECL(64, 8)
 MLC_DECL(128, 1) MLC_DECL(128, 2) MLC_DECL(128, 4) MLC_DECL(128, 8)
 #undef MLC_DECL
-#define MLC_DECL(d, h) bool launch_decode_stream_##d##_##h(int, bool, const StreamArgs&, unsigned, size_t, hipStream_t);
+#define MLC_DECL(d, h) bool launch_decode_stream_##d##_##h(int, int, bool, const StreamArgs&, unsigned, size_t, hipStream_t);
 MLC_DECL(64, 1) MLC_DECL(64, 2) MLC_DECL(64, 4) MLC_DECL(64, 8)
 MLC_DECL(128, 1) MLC_DECL(128, 2) MLC_DECL(128, 4) MLC_DECL(128, 8)
 #undef MLC_DECL
@@ -227,6 +227,7 @@ struct Ctx {
     StreamTables tables;
     long opt_decode_kernel = 0;     // 0 = automatic (tile-balanced where it applies), 1 = planned items, 2 = tile-balanced
     long opt_wgs_per_cu = 0;        // tile-balanced kernel: workgroups per CU (0 = automatic)
+    long opt_stream_stages = 0;     // tile-balanced kernel: LDS stages per workgroup (0 = automatic)
     long opt_grid_wgs = 0;          // tile-balanced kernel: exact grid size (0 = from workgroups per CU)
     long table_uploads = 0;         // page-table uploads of the tile-balanced path (for tests)
 };
@@ -828,17 +829,28 @@ bool stream_variant(size_t G, size_t D, int* hpw_out, int* nw_out) {
         nw = G / (size_t)hpw;
     }
     if (nw > 4 || nw == 3) return false;
-    if (stream_static_lds_bytes((int)D, (int)G) > 60 * 1024) return false;
     *hpw_out = hpw;
     *nw_out = (int)nw;
     return true;
 }
 
+// LDS stages of the tile-balanced kernel.  Two by default: swept over 2..4 stages and 2..5
+// workgroups per CU on MI355X, two stages and two workgroups per CU were fastest at 38 MB and at
+// 1.2 GB of KV per launch (deeper stages only delay the first tile of every workgroup: the
+// kernel's steady state is bound by VALU issue, not by loads in flight).  Batches above 64
+// requests keep their per-request figures in LDS as well and take three stages at most.
+int stream_stages(size_t batch) {
+    const int most = batch <= 64 ? 4 : 3;
+    int nbuf = 2;
+    if (g.opt_stream_stages > 0) nbuf = (int)std::min<long>(g.opt_stream_stages, most);
+    return nbuf;
+}
+
 // Grid of the tile-balanced kernel: as many workgroups as stay resident (LDS decides), within
 // what the scratch array holds.
-unsigned stream_grid(size_t G, size_t D, size_t dyn_lds) {
-    const size_t lds = (size_t)stream_static_lds_bytes((int)D, (int)G) + dyn_lds;
-    size_t per_cu = std::max<size_t>(1, std::min<size_t>(160 * 1024 / lds, 3));
+unsigned stream_grid(size_t G, size_t D, int nbuf, size_t dyn_lds) {
+    const size_t lds = (size_t)stream_static_lds_bytes(nbuf) + dyn_lds;
+    size_t per_cu = std::max<size_t>(1, std::min<size_t>(160 * 1024 / lds, 2));
     if (g.opt_wgs_per_cu > 0) per_cu = (size_t)g.opt_wgs_per_cu;
     size_t W = (size_t)g.n_cu * per_cu;
     if (g.opt_grid_wgs > 0) W = (size_t)g.opt_grid_wgs;
@@ -848,10 +860,11 @@ unsigned stream_grid(size_t G, size_t D, size_t dyn_lds) {
     return (unsigned)std::max<size_t>(W, 1);
 }
 
-bool launch_stream_variant(size_t D, int hpw, int nw, const StreamArgs& a, unsigned n_wg, size_t dyn_lds) {
+bool launch_stream_variant(size_t D, int hpw, int nw, int nbuf, const StreamArgs& a, unsigned n_wg, size_t dyn_lds,
+                           hipStream_t stream) {
     const bool pv16 = g.opt_pv_fp16 != 0;
 #define MLC_CASE(d, h) \
-    if (D == d && hpw == h) return launch_decode_stream_##d##_##h(nw, pv16, a, n_wg, dyn_lds, g.stream);
+    if (D == d && hpw == h) return launch_decode_stream_##d##_##h(nw, nbuf, pv16, a, n_wg, dyn_lds, stream);
     MLC_CASE(64, 1) MLC_CASE(64, 2) MLC_CASE(64, 4) MLC_CASE(64, 8)
     MLC_CASE(128, 1) MLC_CASE(128, 2) MLC_CASE(128, 4) MLC_CASE(128, 8)
 #undef MLC_CASE
@@ -1105,8 +1118,9 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
         const uint32_t* d_flat = nullptr;
         const uint32_t* d_meta = nullptr;
         if (!tables_upload(embed ? nullptr : meta3.data(), batch, &d_flat, &d_meta)) return 0;
-        const size_t dyn_lds = stream_dynamic_lds_bytes(batch);
-        const unsigned n_wg = stream_grid(G, head_dim, dyn_lds);
+        const size_t dyn_lds = batch <= 64 ? 0 : stream_dynamic_lds_bytes(batch);
+        const int nbuf = stream_stages(batch);
+        const unsigned n_wg = stream_grid(G, head_dim, nbuf, dyn_lds);
         StreamArgs a;
         stream_fill_common(a, q, k_pages, v_pages, o, batch, num_heads, kv_heads, head_dim, page_size_tokens,
                            apply_causal);
@@ -1134,7 +1148,7 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
             a.new_ids = g.kv.d_ids;
             a.new_slots = g.kv.d_slots;
         }
-        if (!launch_stream_variant(head_dim, s_hpw, s_nw, a, n_wg, dyn_lds))
+        if (!launch_stream_variant(head_dim, s_hpw, s_nw, nbuf, a, n_wg, dyn_lds, g.stream))
             return fail("decode: kernel variant not built");
         g.last_items = (int)std::min<uint64_t>(n_wg, total_tiles);
         if (carries_kv) {
@@ -2058,6 +2072,16 @@ long mlc_hip_kv_writes_in_decode_launches(void) { return g.kv_in_decode; }
 long mlc_hip_row_program_launches(void) { return g.row_launches; }
 long mlc_hip_decode_table_uploads(void) { return g.table_uploads; }
 
+#ifdef MLC_STREAM_PROBE
+// timing probe build only: the per-workgroup time stamps of the last tile-balanced launch
+int mlc_hip_debug_probe(uint64_t* dst, size_t n_wg) {
+    if (!init_once()) return 0;
+    HIP_OK(hipStreamSynchronize(g.stream));
+    HIP_OK(hipMemcpy(dst, g.scratch_ptr + kScratchPartOBytes + 65536 * 4, n_wg * 64, hipMemcpyDeviceToHost));
+    return 1;
+}
+#endif
+
 int mlc_hip_set_option(const char* name, long value) {
     if (!name) return 0;
     if (g.inited && g.available && !settle()) return 0;
@@ -2067,6 +2091,11 @@ int mlc_hip_set_option(const char* name, long value) {
     if (!std::strcmp(name, "decode_kernel")) {
         if (value < 0 || value > 2) return 0;
         g.opt_decode_kernel = value;
+        return 1;
+    }
+    if (!std::strcmp(name, "decode_stages")) {
+        if (value != 0 && (value < 2 || value > 4)) return 0;
+        g.opt_stream_stages = value;
         return 1;
     }
     if (!std::strcmp(name, "decode_grid_wgs")) {

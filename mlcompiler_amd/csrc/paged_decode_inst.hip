@@ -50,27 +50,37 @@ bool MLC_CAT(MLC_D, MLC_HPW)(int nw, int ns, int nbuf, bool pv16, const DecodeAr
 }
 
 namespace {
+template <int NW, bool SMALL, int NBUF>
+void launch_stream_pv(bool pv16, const StreamArgs& a, unsigned n_wg, size_t dyn_lds, hipStream_t stream) {
+    const dim3 grid(n_wg), block(64 * NW);
+    if (pv16)
+        hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, true, SMALL, NBUF>), grid, block, dyn_lds, stream, a);
+    else
+        hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, false, SMALL, NBUF>), grid, block, dyn_lds, stream, a);
+}
 template <int NW>
-bool launch_stream(bool pv16, const StreamArgs& a, unsigned n_wg, size_t dyn_lds, hipStream_t stream) {
-    if constexpr (stream_static_lds_bytes(MLC_D, MLC_HPW * NW) <= 60 * 1024) {
-        const dim3 grid(n_wg), block(64 * NW);
-        if (pv16)
-            hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, true>), grid, block, dyn_lds, stream, a);
-        else
-            hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, false>), grid, block, dyn_lds, stream, a);
-        return true;
+bool launch_stream(int nbuf, bool pv16, const StreamArgs& a, unsigned n_wg, size_t dyn_lds, hipStream_t stream) {
+    // at most 64 requests: the variant that keeps the per-request figures in registers; larger
+    // batches keep them in dynamic LDS, next to two or three stages
+    if (a.batch <= 64) {
+        if (nbuf == 2) launch_stream_pv<NW, true, 2>(pv16, a, n_wg, 0, stream);
+        else if (nbuf == 3) launch_stream_pv<NW, true, 3>(pv16, a, n_wg, 0, stream);
+        else launch_stream_pv<NW, true, 4>(pv16, a, n_wg, 0, stream);
     } else {
-        return false;
+        if (nbuf == 2) launch_stream_pv<NW, false, 2>(pv16, a, n_wg, dyn_lds, stream);
+        else launch_stream_pv<NW, false, 3>(pv16, a, n_wg, dyn_lds, stream);
     }
+    return true;
 }
 }  // namespace
 
-// Tile-balanced kernel: nw = waves over the GQA group, n_wg = grid size; false for an unbuilt combination.
-bool MLC_SCAT(MLC_D, MLC_HPW)(int nw, bool pv16, const StreamArgs& a, unsigned n_wg, size_t dyn_lds, hipStream_t stream) {
+// Tile-balanced kernel: nw = waves over the GQA group, nbuf = LDS stages (large batches: at most 3),
+// n_wg = grid size; false for an unbuilt combination.
+bool MLC_SCAT(MLC_D, MLC_HPW)(int nw, int nbuf, bool pv16, const StreamArgs& a, unsigned n_wg, size_t dyn_lds, hipStream_t stream) {
     switch (nw) {
-        case 1: return launch_stream<1>(pv16, a, n_wg, dyn_lds, stream);
-        case 2: return launch_stream<2>(pv16, a, n_wg, dyn_lds, stream);
-        case 4: return launch_stream<4>(pv16, a, n_wg, dyn_lds, stream);
+        case 1: return launch_stream<1>(nbuf, pv16, a, n_wg, dyn_lds, stream);
+        case 2: return launch_stream<2>(nbuf, pv16, a, n_wg, dyn_lds, stream);
+        case 4: return launch_stream<4>(nbuf, pv16, a, n_wg, dyn_lds, stream);
         default: return false;
     }
 }

@@ -6,8 +6,9 @@
 //
 //   * The KV tiles of the whole batch are numbered in the order
 //     [request][kv head][tile of the request]; with T tiles and W workgroups, workgroup w
-//     takes tiles [w*T/W, (w+1)*T/W): every workgroup gets the same number of tiles (+-1)
-//     whatever the context lengths are, and the grid size does not depend on the tables.
+//     takes T/W consecutive tiles (the first T%W workgroups one more): every workgroup gets
+//     the same number of tiles (+-1) whatever the context lengths are, and the grid size does
+//     not depend on the tables.
 //   * A workgroup walks its range as one stream: tile k+1 is in flight while tile k is
 //     consumed, also across the boundary between two (request, kv head) pairs; the running
 //     softmax state is kept across the tiles of a pair and finalised when the pair (or the
@@ -59,15 +60,63 @@ struct StreamArgs {
     uint32_t emb[3 * kStreamEmbBatch];
 };
 
-constexpr int stream_static_lds_bytes(int D, int G) {
-    const int rpi = 64 / (D / 8);
-    return 2 * 2 * (8 * rpi * D * 2) + G * D * rpi * 4;  // two staging buffers (K, V tiles) + epilogue sums
-}
+// LDS of one workgroup: NBUF stages of one K tile and one V tile (8 KiB each)
+constexpr int stream_static_lds_bytes(int NBUF) { return NBUF * 2 * 8192; }
 // dynamic LDS: tile prefix [B + 1], visible lengths [B], page-table offsets [B]
 inline size_t stream_dynamic_lds_bytes(size_t batch) { return (3 * batch + 1) * 4; }
 
-template <int D, int HPW, int NW, bool PV16>
+#ifdef MLC_STREAM_PROBE
+#define MLC_PROBE(i)                                                                                   \
+    do {                                                                                               \
+        if (threadIdx.x == 0)                                                                          \
+            reinterpret_cast<uint64_t*>(a.part_ml + 65536)[blockIdx.x * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); \
+    } while (0)
+#else
+#define MLC_PROBE(i)
+#endif
+
+// 16-byte global -> LDS load that bypasses the register file: lane i's 16 bytes land at LDS byte
+// address lds_base + 16*i (lds_base wave-uniform).  Issued as inline assembly on purpose: the
+// compiler then does not know of the load, so it neither waits for all loads in flight before
+// LDS reads of another stage nor needs one array per stage; the ordering is explicit instead
+// (sd_wait_vmcnt, sd_barrier).
+__device__ __forceinline__ void sd_g2lds16(const void* g, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(lds_base), "v"(g)
+                 : "memory", "m0");
+}
+__device__ __forceinline__ uint32_t sd_lds_addr(const void* p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
+}
+// s_waitcnt vmcnt(N), other counters untouched; also a compiler barrier for memory accesses
+// (the LDS reads behind it depend on loads the compiler does not know about).
+template <int N>
+__device__ __forceinline__ void sd_wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+// Workgroup barrier that orders LDS traffic only (global -> LDS loads stay in flight across it).
+__device__ __forceinline__ void sd_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// exclusive-to-inclusive prefix sum over the 64 lanes in six DPP steps (no LDS traffic)
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t x) {
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x111, 0xF, 0xF, true);   // row_shr:1
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x112, 0xF, 0xF, true);   // row_shr:2
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x114, 0xF, 0xF, true);   // row_shr:4
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x118, 0xF, 0xF, true);   // row_shr:8
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x142, 0xA, 0xF, false);  // row_bcast:15 -> rows 1, 3
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x143, 0xC, 0xF, false);  // row_bcast:31 -> rows 2, 3
+    return x;
+}
+
+// SMALL: at most 64 requests; lane r of every wave holds request r's figures in registers and
+// nothing goes through LDS.  Otherwise they are kept in (dynamic) LDS.
+// NBUF: tiles staged in LDS per workgroup; tile k + NBUF - 1 is requested while tile k is consumed.
+template <int D, int HPW, int NW, bool PV16, bool SMALL, int NBUF>
 __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const StreamArgs a) {
+    static_assert(NBUF >= 2 && NBUF <= 4, "2 to 4 stages");
     static_assert(D == 64 || D == 128, "head_dim 64 and 128");
     static_assert(NW == 1 || NW == 2 || NW == 4, "waves per GQA group");
     constexpr int CPR = D / 8;         // 16-byte chunks per row
@@ -77,18 +126,26 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     constexpr int HPK = D / 64;        // epilogue registers per head
     constexpr int G = HPW * NW;        // query heads per KV head
     constexpr int TILE_BYTES = TT * D * 2;  // one tensor, one KV head: 8 KiB
-    // Separate arrays: reads of the buffer being consumed do not alias the global -> LDS loads
-    // in flight into the other one, and the epilogue has memory of its own because tile loads
-    // stay in flight across it.
-    __shared__ __attribute__((aligned(16))) unsigned char stage0[2 * TILE_BYTES];
-    __shared__ __attribute__((aligned(16))) unsigned char stage1[2 * TILE_BYTES];
-    __shared__ __attribute__((aligned(16))) float s_epi[NW * RPI * HPW * D];
+    constexpr int LPW = 16 / NW;            // tile-load instructions per wave and tile (8 K + 8 V in all)
+    constexpr int STAGE_BYTES = 2 * TILE_BYTES;
+    __shared__ __attribute__((aligned(16))) unsigned char stages[NBUF * STAGE_BYTES];
     extern __shared__ uint32_t s_meta[];
     const uint32_t B = a.batch;
     uint32_t* s_start = s_meta;            // [B + 1] tiles of the requests before r (one KV head)
     uint32_t* s_lim = s_meta + B + 1;      // [B] visible tokens
     uint32_t* s_off = s_lim + B;           // [B] offset of the request's page ids
 
+    MLC_PROBE(0);
+    // Everything the prologue needs from the kernel arguments is requested now, in one go: left
+    // to the compiler, each would be fetched where it is first used, one memory round trip after
+    // the other on the way to the first tile load.
+    {
+        const uint64_t p0 = (uint64_t)a.q, p1 = (uint64_t)a.k_pages, p2 = (uint64_t)a.v_pages, p3 = (uint64_t)a.pt_flat,
+                       p4 = (uint64_t)a.new_k;
+        asm volatile("" ::"s"(a.batch), "s"(a.num_heads), "s"(a.kv_heads), "s"(a.page_size), "s"(a.causal),
+                     "s"(a.capacity_pages), "s"(a.scale_log2e), "s"(p0), "s"(p1), "s"(p2), "s"(p3), "s"(p4),
+                     "s"(gridDim.x));
+    }
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const int lane = threadIdx.x % 64;
     const int hg = wave;  // head group of this wave
@@ -99,55 +156,92 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     const uint32_t Hkv = a.kv_heads;
     const uint32_t row_u4 = Hkv * CPR;  // 16-byte chunks per token row (all KV heads)
 
-    // ---- the per-request arrays -> LDS: visible length, page-table offset, tile prefix
-    if (wave == 0) {
-        const uint32_t* meta = a.meta ? a.meta : a.emb;
-        const uint32_t stride = a.meta ? a.meta_stride : kStreamEmbBatch;
-        uint32_t carry = 0;
-        for (uint32_t b0 = 0; b0 < B; b0 += 64) {
-            const uint32_t i = b0 + lane;
-            uint32_t seq = 0, qp = 0, off = 0;
-            if (i < B) {
-                seq = meta[i];
-                qp = meta[stride + i];
-                off = meta[2 * stride + i];
-            }
-            const uint32_t lim = (a.causal && qp < seq) ? qp + 1u : seq;  // metal_runtime.mm:2286
-            const uint32_t tiles = (lim + TT - 1) / TT;
-            uint32_t x = tiles;
-#pragma unroll
-            for (int d = 1; d < 64; d <<= 1) {
-                const uint32_t y = __shfl_up(x, d);
-                if (lane >= d) x += y;
-            }
-            if (i < B) {
-                s_start[i] = carry + x - tiles;
-                s_lim[i] = lim;
-                s_off[i] = off;
-            }
-            carry += __shfl(x, 63);
+    // ---- the per-request arrays: visible length, page-table offset, tile prefix
+    uint32_t v_start = 0, v_tiles = 0, v_lim = 0, v_off = 0;  // SMALL: request `lane`
+    uint32_t tiles_head;                                       // tiles of all requests (one KV head)
+    if constexpr (SMALL) {
+        // The arrays inside the kernel arguments are read before anything else is known (their
+        // address is the argument segment's, no pointer has to be fetched first); lanes past
+        // the batch read other arguments and are masked.
+        uint32_t seq = a.emb[lane], qp = a.emb[kStreamEmbBatch + lane], off = a.emb[2 * kStreamEmbBatch + lane];
+        if (a.meta != nullptr && (uint32_t)lane < B) {
+            seq = a.meta[lane];
+            qp = a.meta[a.meta_stride + lane];
+            off = a.meta[2 * a.meta_stride + lane];
         }
-        if (lane == 0) s_start[B] = carry;
+        uint32_t lim = (a.causal && qp < seq) ? qp + 1u : seq;  // metal_runtime.mm:2286
+        lim = (uint32_t)lane < B ? lim : 0u;
+        v_lim = lim;
+        v_off = off;
+        v_tiles = (lim + TT - 1) / TT;
+        const uint32_t incl = wave_inclusive_scan(v_tiles);
+        v_start = incl - v_tiles;
+        tiles_head = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+    } else {
+        if (wave == 0) {
+            const uint32_t* meta = a.meta ? a.meta : a.emb;
+            const uint32_t stride = a.meta ? a.meta_stride : kStreamEmbBatch;
+            uint32_t carry = 0;
+            for (uint32_t b0 = 0; b0 < B; b0 += 64) {
+                const uint32_t i = b0 + lane;
+                uint32_t seq = 0, qp = 0, off = 0;
+                if (i < B) {
+                    seq = meta[i];
+                    qp = meta[stride + i];
+                    off = meta[2 * stride + i];
+                }
+                const uint32_t lim = (a.causal && qp < seq) ? qp + 1u : seq;  // metal_runtime.mm:2286
+                const uint32_t tiles = (lim + TT - 1) / TT;
+                const uint32_t x = wave_inclusive_scan(tiles);
+                if (i < B) {
+                    s_start[i] = carry + x - tiles;
+                    s_lim[i] = lim;
+                    s_off[i] = off;
+                }
+                carry += (uint32_t)__builtin_amdgcn_readlane((int)x, 63);
+            }
+            if (lane == 0) s_start[B] = carry;
+        }
+        __syncthreads();
+        tiles_head = s_start[B];
     }
-    __syncthreads();
+    MLC_PROBE(1);
+    auto req_start = [&](uint32_t r) {
+        if constexpr (SMALL) return (uint32_t)__builtin_amdgcn_readlane((int)v_start, (int)r);
+        else return (uint32_t)__builtin_amdgcn_readfirstlane(s_start[r]);
+    };
+    auto req_tiles = [&](uint32_t r) {
+        if constexpr (SMALL) return (uint32_t)__builtin_amdgcn_readlane((int)v_tiles, (int)r);
+        else return (uint32_t)__builtin_amdgcn_readfirstlane(s_start[r + 1] - s_start[r]);
+    };
+    auto req_lim = [&](uint32_t r) {
+        if constexpr (SMALL) return (uint32_t)__builtin_amdgcn_readlane((int)v_lim, (int)r);
+        else return (uint32_t)__builtin_amdgcn_readfirstlane(s_lim[r]);
+    };
+    auto req_off = [&](uint32_t r) {
+        if constexpr (SMALL) return (uint32_t)__builtin_amdgcn_readlane((int)v_off, (int)r);
+        else return (uint32_t)__builtin_amdgcn_readfirstlane(s_off[r]);
+    };
 
     // ---- requests without visible tokens are in nobody's range: their rows are zero
     // (metal_runtime.mm:2254-2257)
     for (uint32_t rr = blockIdx.x; rr < B; rr += gridDim.x) {
-        if (s_lim[rr] == 0) {
+        if (req_lim(rr) == 0) {
             float* orow = a.o + (size_t)rr * a.num_heads * D;
             for (uint32_t i = threadIdx.x; i < a.num_heads * D; i += 64 * NW) orow[i] = 0.f;
         }
     }
 
-    const uint32_t tiles_head = s_start[B];
     const uint32_t T = tiles_head * Hkv;                       // the host keeps this below 2^31
     const uint32_t W = gridDim.x < T ? gridDim.x : T;          // every workgroup below W has work
     const uint32_t w = blockIdx.x;
     if (w >= W) return;
-    const uint32_t g0 = (uint32_t)(((uint64_t)w * T) / W);
-    const uint32_t g1 = (uint32_t)(((uint64_t)(w + 1) * T) / W);
-    const uint32_t n = g1 - g0;  // >= 1
+    // T = W * tq + trem: the first trem workgroups take tq + 1 tiles, the others tq
+    const uint32_t tq = __builtin_amdgcn_readfirstlane(T / W), trem = T - tq * W;
+    auto range_start = [&](uint32_t wg) { return wg * tq + (wg < trem ? wg : trem); };
+    const uint32_t g0 = range_start(w);
+    const uint32_t n = tq + (w < trem ? 1u : 0u);  // >= 1
+    const uint32_t g1 = g0 + n;
 
     // Position in the tile stream: request, KV head, tile of the request, and the request's
     // figures.  All wave-uniform (kept in scalar registers).
@@ -155,26 +249,31 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         uint32_t r, kvh, t, tiles, lim, off;
     };
     auto load_request = [&](Cursor& cu) {
-        cu.tiles = __builtin_amdgcn_readfirstlane(s_start[cu.r + 1] - s_start[cu.r]);
-        cu.lim = __builtin_amdgcn_readfirstlane(s_lim[cu.r]);
-        cu.off = __builtin_amdgcn_readfirstlane(s_off[cu.r]);
+        cu.tiles = req_tiles(cu.r);
+        cu.lim = req_lim(cu.r);
+        cu.off = req_off(cu.r);
     };
-    // largest r with s_start[r] <= key (key < tiles_head): 64-ary search, two levels
+    // largest r with start[r] <= key (key < tiles_head)
     auto find_request = [&](uint32_t key) {
-        uint32_t base = 0;
-        if (B > 64) {
-            const uint32_t idx = (uint32_t)lane * 64u;
+        if constexpr (SMALL) {
+            // lanes past the batch hold the total, which is above any key
+            return (uint32_t)__builtin_popcountll(__ballot(v_start <= key)) - 1u;
+        } else {
+            uint32_t base = 0;
+            if (B > 64) {  // 64-ary search, two levels
+                const uint32_t idx = (uint32_t)lane * 64u;
+                const uint32_t v = idx < B ? s_start[idx] : 0xFFFFFFFFu;
+                base = (uint32_t)(__builtin_popcountll(__ballot(v <= key)) - 1) * 64u;
+            }
+            const uint32_t idx = base + (uint32_t)lane;
             const uint32_t v = idx < B ? s_start[idx] : 0xFFFFFFFFu;
-            base = (uint32_t)(__builtin_popcountll(__ballot(v <= key)) - 1) * 64u;
+            return (uint32_t)__builtin_amdgcn_readfirstlane(base + (uint32_t)__builtin_popcountll(__ballot(v <= key)) - 1u);
         }
-        const uint32_t idx = base + (uint32_t)lane;
-        const uint32_t v = idx < B ? s_start[idx] : 0xFFFFFFFFu;
-        return (uint32_t)__builtin_amdgcn_readfirstlane(base + (uint32_t)__builtin_popcountll(__ballot(v <= key)) - 1u);
     };
     auto seek = [&](Cursor& cu, uint32_t g) {
         cu.r = find_request(g / Hkv);
         load_request(cu);
-        const uint32_t rem = g - __builtin_amdgcn_readfirstlane(s_start[cu.r]) * Hkv;
+        const uint32_t rem = g - req_start(cu.r) * Hkv;
         cu.kvh = __builtin_amdgcn_readfirstlane(rem / cu.tiles);
         cu.t = rem - cu.kvh * cu.tiles;
     };
@@ -186,7 +285,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         cu.kvh = 0;
         do {
             ++cu.r;
-        } while (__builtin_amdgcn_readfirstlane(s_start[cu.r + 1] - s_start[cu.r]) == 0);
+        } while (req_tiles(cu.r) == 0);
         load_request(cu);
     };
     const uint32_t tpp = a.page_size / TT;  // tiles per page (page size is a multiple of the tile)
@@ -204,9 +303,14 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         const uint32_t t = pv_win + (uint32_t)lane;
         pv = 0;
         if (t < cu.tiles) pv = a.pt_flat[cu.off + t / tpp];
+        // The ids are waited for here, inside whatever branch fetches them: left pending, the
+        // compiler would wait at every later join of the control flow, and as it does not know
+        // of the tile loads, that wait would be for all of them.
+        asm volatile("" : "+v"(pv));
     };
     auto pages_ready = [&](const Cursor& cu) { return pv_req == cu.r && (cu.t & ~63u) == pv_win; };
     fetch_pages(ci);
+    MLC_PROBE(2);
 
     // ---- the step's KV write: this workgroup owns the last tile of every pair that ends in
     // its range, so it writes those pairs' slices of the new rows, waits for the stores, and
@@ -241,8 +345,8 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        wait_vmcnt<0>();  // the rows have left this wave before any wave of the workgroup loads them
-        __syncthreads();
+        sd_wait_vmcnt<0>();  // the rows have left this wave before any wave of the workgroup loads them
+        sd_barrier();
     }
 
     // q of this wave's heads, dims c*8 .. c*8+7, scaled
@@ -263,7 +367,8 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     // This wave's share of the global -> LDS loads of the tile under `cu`.  Load instruction j
     // of a tensor brings row group j ^ g(c) to lane (r, c), at LDS offset j*1024 + lane*16; rows
     // past the visible end are clamped onto the last visible row (in bounds, masked out later).
-    auto issue_tile = [&](const Cursor& cu, unsigned char* stage) {
+    const uint32_t stages_lds = sd_lds_addr(stages);
+    auto issue_tile = [&](const Cursor& cu, uint32_t slot) {
         uint32_t page_id = (uint32_t)__builtin_amdgcn_readlane((int)pv, (int)(cu.t & 63u));
         if (a.capacity_pages && page_id >= a.capacity_pages) page_id = a.capacity_pages - 1u;
         const uint32_t tile_start = cu.t * TT;
@@ -277,15 +382,28 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
             const int tensor = (NW == 1) ? p : (NW == 2 ? hg : hg / 2);
             const int j0 = (NW == 4) ? (hg % 2) * 4 : 0;
             const uint4* base = (tensor ? a.v_pages : a.k_pages) + row0;
-            unsigned char* dst = stage + tensor * TILE_BYTES;
+            const uint32_t dst = stages_lds + slot * STAGE_BYTES + tensor * TILE_BYTES;
 #pragma unroll
             for (int jj = 0; jj < JN; ++jj) {
                 const int j = j0 + jj;
                 uint32_t tr = (uint32_t)((j ^ gsw) * RPI + r_l);
                 tr = tr < last ? tr : last;
-                g2lds16(base + (size_t)tr * row_u4, dst + j * 1024);
+#ifndef MLC_NO_LOADS
+                sd_g2lds16(base + (size_t)tr * row_u4, dst + j * 1024);
+#else
+                asm volatile("" ::"v"(base + (size_t)tr * row_u4), "s"(dst + j * 1024));
+#endif
             }
         }
+    };
+    // waits until this wave's loads of the oldest tile in flight have landed, given how many
+    // tiles were issued after it (loads return in order; other loads issued in between only
+    // make the wait longer, never shorter)
+    auto wait_tile = [&](uint32_t younger) {
+        if (younger == 0) sd_wait_vmcnt<0>();
+        else if (younger == 1) sd_wait_vmcnt<LPW>();
+        else if (younger == 2) sd_wait_vmcnt<(NBUF > 2 ? 2 * LPW : 0)>();
+        else sd_wait_vmcnt<(NBUF > 3 ? 3 * LPW : 0)>();
     };
 
     float acc[HPW][8];
@@ -302,7 +420,8 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     reset_state();
 
     // ---- one tile: QK, softmax update, PV (the arithmetic of paged_decode_fast_kernel)
-    auto consume_tile = [&](const unsigned char* cur, uint32_t t, uint32_t lim) {
+    auto consume_tile = [&](uint32_t slot, uint32_t t, uint32_t lim) {
+        const unsigned char* cur = stages + (size_t)slot * STAGE_BYTES;
         const uint32_t tile_start = t * TT;
         const uint4* kl = reinterpret_cast<const uint4*>(cur) + lane;
         const uint4* vl = kl + TILE_BYTES / 16;
@@ -440,8 +559,13 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     // the output (the whole pair was ours) or a partial, whose last arriver merges.
     // seg_first: global index of the first tile this workgroup consumed for the pair.
     auto finalize = [&](const Cursor& cu, uint32_t seg_first, uint32_t seg_end) {
-        float* s_acc = s_epi + (size_t)wave * (RPI * HPW * D);
+        // Bring the rows of lanes (the tokens a lane row owns) onto one reference and sum over
+        // them by reduce-scatter across the lane bits above the chunk index: every step halves the
+        // values a lane keeps (v_permlane32_swap / v_permlane16_swap hand the other half to the
+        // partner, the last step of head_dim 64 goes over lane ^ 8).  Lane (r, c) ends up with
+        // dims c*8 + r*HPK + kk (kk < HPK) of every head, summed over all tokens of the wave.
         float m_all[HPW], l_all[HPW];
+        float o_un[OPL];
 #pragma unroll
         for (int h = 0; h < HPW; ++h) {
             float m = m_ref[h];
@@ -451,45 +575,54 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
             const float wgt = fast_exp2(m_ref[h] - m);
             // with CPR == 16 every token's weight sits in two lanes (c and c^8): count it once
             l_all[h] = wave_sum((CPR == 16 && (c & 8)) ? 0.f : l_sum[h] * wgt);
-            float4* dst = reinterpret_cast<float4*>(&s_acc[((r_l * HPW + h) * CPR + c) * 8]);
-            dst[0] = make_float4(acc[h][0] * wgt, acc[h][1] * wgt, acc[h][2] * wgt, acc[h][3] * wgt);
-            dst[1] = make_float4(acc[h][4] * wgt, acc[h][5] * wgt, acc[h][6] * wgt, acc[h][7] * wgt);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        float o_un[OPL];
+            float v4[4], v2[2];
 #pragma unroll
-        for (int k = 0; k < OPL; ++k) {
-            const int idx = k * 64 + lane;
-            float sum = 0.f;
+            for (int i = 0; i < 4; ++i) {  // lane bit 5: keep dims i (lower half) or i + 4 (upper half)
+                const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[h][i] * wgt),
+                                                                 __float_as_uint(acc[h][i + 4] * wgt), false, false);
+                v4[i] = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+            }
 #pragma unroll
-            for (int rr = 0; rr < RPI; ++rr) sum += s_acc[rr * HPW * D + idx];
-            o_un[k] = sum;
+            for (int i = 0; i < 2; ++i) {  // lane bit 4
+                const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(v4[i]), __float_as_uint(v4[i + 2]),
+                                                                 false, false);
+                v2[i] = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+            }
+            if constexpr (CPR == 8) {      // lane bit 3 (head_dim 64: eight rows of lanes)
+                const bool up = (lane & 8) != 0;
+                const float send = up ? v2[0] : v2[1];
+                const float keep = up ? v2[1] : v2[0];
+                o_un[h] = keep + dpp_f<kDppRowRor8>(send);
+            } else {
+                o_un[h * 2] = v2[0];
+                o_un[h * 2 + 1] = v2[1];
+            }
         }
-        // (the next pair's sums are written to the same memory: reads above come first)
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
+        // element (head k / HPK, dim) of output register k of this lane
+        const int dim0 = c * 8 + r_l * HPK;
 
         const uint32_t head0 = cu.kvh * G + hg * HPW;
         float* orow = a.o + ((size_t)cu.r * a.num_heads + head0) * D;
-        const uint32_t ps = __builtin_amdgcn_readfirstlane(s_start[cu.r]) * Hkv + cu.kvh * cu.tiles;  // pair's first tile
+        const uint32_t ps = req_start(cu.r) * Hkv + cu.kvh * cu.tiles;  // pair's first tile
         const uint32_t pe = ps + cu.tiles;
         if (seg_first == ps && seg_end == pe) {
 #pragma unroll
             for (int k = 0; k < OPL; ++k) {
                 const float l = l_all[k / HPK];
                 const float inv = l > 0.f ? 1.0f / l : 0.f;
-                orow[k * 64 + lane] = o_un[k] * inv;
+                orow[(k / HPK) * D + dim0 + (k % HPK)] = o_un[k] * inv;
             }
             return;
         }
-        // workgroup of tile g: the largest w with w*T/W <= g
-        auto wg_of = [&](uint32_t g) { return (uint32_t)((((uint64_t)g + 1u) * W - 1u) / T); };
+        // workgroup that holds tile g
+        const uint32_t thr = trem * (tq + 1u);
+        auto wg_of = [&](uint32_t g) {
+            return (uint32_t)__builtin_amdgcn_readfirstlane(g < thr ? g / (tq + 1u) : trem + (g - thr) / tq);
+        };
         const uint32_t w_lo = wg_of(ps), w_hi = wg_of(pe - 1u);
         const uint32_t n_splits = w_hi - w_lo + 1u;
         // A workgroup's first pair uses slot 2w, a later (so: its last) pair slot 2w + 1.
-        const uint32_t g0_lo = (uint32_t)(((uint64_t)w_lo * T) / W);
+        const uint32_t g0_lo = range_start(w_lo);
         const uint32_t slot_first = 2u * w_lo + (g0_lo == ps ? 0u : 1u);
         const uint32_t my_slot = (ps <= g0) ? 2u * w : 2u * w + 1u;
         {
@@ -511,7 +644,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         // The partial must have reached memory before the arrival counter is bumped: the
         // write-through stores are complete once this wave's memory counter is zero.
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        wait_vmcnt<0>();
+        sd_wait_vmcnt<0>();
         uint32_t ticket = 0;
         uint32_t* counter = &a.counters[(size_t)w_lo * NW + hg];
         if (lane == 0) ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -579,45 +712,64 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         for (int k = 0; k < OPL; ++k) {
             const float l = l_run[k / HPK];
             const float inv = l > 0.f ? 1.0f / l : 0.f;
-            orow[k * 64 + lane] = acc_o[k] * inv;
+            orow[(k / HPK) * D + dim0 + (k % HPK)] = acc_o[k] * inv;
         }
     };
 
-    // ---- the stream: tiles 0 and 1 of the range go out together, then one tile per step
+    // ---- the stream: the first NBUF tiles of the range go out together, then one tile per step
+    // into the stage the step before has left
     load_q(cc);
-    issue_tile(ci, stage0);
-    if (n > 1) {
-        advance(ci);
-        if (!pages_ready(ci)) fetch_pages(ci);
-        issue_tile(ci, stage1);
+    uint32_t issued = 1;
+    issue_tile(ci, 0);
+#pragma unroll
+    for (int i = 1; i < NBUF; ++i) {
+        if (issued < n) {
+            advance(ci);
+            if (!pages_ready(ci)) fetch_pages(ci);
+            issue_tile(ci, (uint32_t)i);
+            ++issued;
+        }
     }
     uint32_t seg_first = g0;  // first tile consumed for the pair under cc
-    auto do_step = [&](uint32_t k, unsigned char* cur, unsigned char* nxt) {
-        wait_vmcnt<0>();   // own loads of tile k (and the page ids fetched with them) have landed
-        __syncthreads();   // everyone's have; everyone left tile k-1, whose buffer is free
-        if (k >= 1 && k + 1 < n) {
+    bool drain = false;       // stores are in flight: they do not complete in order with loads
+    uint32_t slot = 0;        // stage of tile k
+    for (uint32_t k = 0; k < n; ++k) {
+        // this wave's loads of tile k have landed ...
+        if (drain) sd_wait_vmcnt<0>(); else wait_tile(issued - k - 1u);
+        drain = false;
+        sd_barrier();   // ... and everyone's; everyone has left tile k-1, whose stage is free
+        if (k == 0) MLC_PROBE(3);
+        if (k >= 1 && issued < n) {
             advance(ci);
-            if (!pages_ready(ci)) {  // rare (a new request, or 64 tiles on): fetched on demand
-                fetch_pages(ci);
-            }
-            issue_tile(ci, nxt);
+            if (!pages_ready(ci)) fetch_pages(ci);  // another request, or 64 tiles on
+            issue_tile(ci, slot == 0 ? (uint32_t)(NBUF - 1) : slot - 1u);
+            ++issued;
         }
-        consume_tile(cur, cc.t, cc.lim);
+#ifndef MLC_NO_COMPUTE
+        consume_tile(slot, cc.t, cc.lim);
+#endif
         const bool pair_done = cc.t + 1u == cc.tiles;
+        if (k + 1 == n) MLC_PROBE(4);
         if (pair_done || k + 1 == n) {
             finalize(cc, seg_first, g0 + k + 1u);
             reset_state();
             seg_first = g0 + k + 1u;
+            drain = true;
         }
         if (k + 1 < n) {
             advance(cc);
             if (pair_done) load_q(cc);
         }
-    };
-    for (uint32_t k = 0; k < n; k += 2) {
-        do_step(k, stage0, stage1);
-        if (k + 1 < n) do_step(k + 1, stage1, stage0);
+        slot = slot + 1u == (uint32_t)NBUF ? 0u : slot + 1u;
     }
+    MLC_PROBE(5);
+#ifdef MLC_STREAM_PROBE
+    if (threadIdx.x == 0) {
+        reinterpret_cast<uint64_t*>(a.part_ml + 65536)[blockIdx.x * 8 + 6] = n;
+        const uint64_t hw = __builtin_amdgcn_s_getreg((31 << 11) | 4), xcc = __builtin_amdgcn_s_getreg((31 << 11) | 20);
+        reinterpret_cast<uint64_t*>(a.part_ml + 65536)[blockIdx.x * 8 + 7] = hw | (xcc << 32);
+    }
+#endif
 }
 
 }  // namespace mlc_hip
