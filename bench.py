@@ -9,8 +9,14 @@ independent per-layer K/V pools so the working set (~0.8 GB touched) does not
 sit in the 256 MB Infinity Cache.
 
 Prints ONE JSON line: the KV-read GB/s of the whole job, the roofline of the
-decode kernel measured with HIP events on the kernel's stream, and the CPU
-baseline timed on this host's cores in the same run.
+decode kernel measured with HIP events on the kernel's stream (with a plain
+streaming read of the same bytes beside it), and the CPU baseline timed on
+this host's cores in the same run.  The default run adds config.per_config:
+configurations 1, 3 (with its KV write), 4 and 5 (chunked prefill), each with
+its own time, rate, roofline fraction and bounded CPU baseline.
+--workload cfg1|cfg3|cfg4|cfg5 print one of those as a line of its own,
+--workload refbench the reference's own micro-benchmark grid, --workload
+layer|step a whole decoder layer / decode step.
 """
 from __future__ import annotations
 
@@ -61,7 +67,16 @@ def bench_copy(args) -> int:
     return 0
 
 
-def bench_prefill(args) -> int:
+def prefill_traffic():
+    """HBM bytes per launch of the prefill kernel at configuration 5 (profiles/traffic.json)."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as fh:
+            return json.load(fh).get("prefill", {}).get("cfg5", {}).get("hbm_bytes_per_launch")
+    except (OSError, ValueError):
+        return None
+
+
+def bench_prefill(args) -> dict:
     """Chunked prefill (benchmark configuration 5): B=8, 256-row fp16 query chunk after 3840
     cached tokens, 32q/8kv heads, head_dim 128.  Reports TFLOP/s on the exact causal FLOPs."""
     import ctypes as C
@@ -113,8 +128,7 @@ def bench_prefill(args) -> int:
                    "flop_per_step": flops, "kv_bytes_per_step": kv_bytes},
         "roofline": {"bound": "mfma", "achieved": round(ach, 2), "peak": MFMA_F16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(ach / MFMA_F16_PEAK_TFLOPS, 4),
-                     # rocprofv3 FETCH_SIZE x2.0 + WRITE_SIZE x1.0 (copy-kernel calibration)
-                     "traffic": 184_800_000 if not (args.prefill_stages) else None,
+                     "traffic": prefill_traffic() if not args.prefill_stages else None,
                      "us_per_launch": round(ev_ms / steps * 1e3, 2)},
     }
     if not args.no_cpu:
@@ -141,8 +155,7 @@ def bench_prefill(args) -> int:
                                   "sample": f"{rows} of {Cc} chunk rows of request 0 (all heads), {dt:.2f} s"}
         result["parity_vs_cpu_baseline"] = {"min_cosine": round(rep["min_cosine"], 7),
                                             "max_abs": float(f"{rep['max_abs']:.3e}")}
-    print(json.dumps(result))
-    return 0
+    return result
 
 
 def bench_layer(args) -> int:
@@ -447,8 +460,9 @@ def cpu_baseline(case, budget_s: float):
             break
     sample = f"{len(outs)} of {c.batch} requests of the same batch, {done_bytes} KV bytes, {spent:.2f} s"
     # all host cores, OpenMP over (request, head): reported beside the 1-thread figure
-    n = os.cpu_count() or 1
-    n = min(n, 16)
+    # (the oracle's OpenMP loop is given at most 16 threads: the share of the host a one-GPU
+    # box has; the host's own count is reported beside it)
+    n = min(os.cpu_count() or 1, 16)
     t0 = time.perf_counter()
     po.paged_attention_executor(c.q, c.k_pages, c.v_pages, c.page_tables_flat,
                                 c.page_table_offsets, c.seq_lens, c.q_positions, c.batch,
@@ -460,8 +474,278 @@ def cpu_baseline(case, budget_s: float):
         "cores": 1,
         "kind": kind,
         "sample": sample,
-        "all_cores": {"value": round(case.kv_bytes / t_all / 1e9, 4), "cores": n, "kind": "port"},
+        "all_cores": {"value": round(case.kv_bytes / t_all / 1e9, 4), "cores": n, "kind": "port",
+                      "host_cores": os.cpu_count()},
     }, outs
+
+
+def load_traffic(workload: str, kernel: str, work_items: int):
+    """HBM bytes per launch of the decode kernel as profiled with rocprofv3 (FETCH_SIZE and
+    WRITE_SIZE, scaled by the copy-kernel calibration), from profiles/traffic.json.  The figure
+    belongs to one kernel variant and one split of the work: None when this run's differ."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as fh:
+            table = json.load(fh)
+    except (OSError, ValueError):
+        return None
+    e = table.get("decode", {}).get(workload)
+    if not e or e.get("kernel") != kernel or e.get("work_items") != work_items:
+        return None
+    return e.get("hbm_bytes_per_launch")
+
+
+def run_decode(args, name: str, steps: int, warmup: int, cpu_budget: float, full: bool) -> dict:
+    """Times one decode configuration through the C ABI and frees its buffers again.
+    full: also the one-launch-at-a-time distribution, the changing-tables loop, the fp32-weight
+    variant and the streaming-read ceiling (the headline configuration's extras)."""
+    import ctypes as C
+
+    from mlcompiler_amd import HipExecutor
+    from mlcompiler_amd.build import BENCH_LIB_PATH
+    exe = HipExecutor.Instance()
+    case, n_layers = build_workload(name)
+    c = case
+    pool_bytes = c.k_pages.nbytes
+    q_buf = exe.allocateScratchBuffer(c.q.nbytes)
+    o_buf = exe.allocateScratchBuffer(c.q.nbytes)
+    assert exe.uploadToBuffer(q_buf, c.q)
+    k_bufs, v_bufs = [], []
+    for _ in range(n_layers):
+        kb = exe.allocateScratchBuffer(pool_bytes)
+        vb = exe.allocateScratchBuffer(pool_bytes)
+        assert kb and vb, "out of device memory"
+        assert exe.uploadToBuffer(kb, c.k_pages) and exe.uploadToBuffer(vb, c.v_pages)
+        k_bufs.append(kb)
+        v_bufs.append(vb)
+
+    bl = C.CDLL(BENCH_LIB_PATH)   # native loop around the C ABI (no Python between launches)
+    u32p = C.POINTER(C.c_uint32)
+    meta = [np.ascontiguousarray(x, np.uint32) for x in
+            (c.page_tables_flat, c.page_table_offsets, c.seq_lens, c.q_positions)]
+    kp = (C.c_void_p * n_layers)(*k_bufs)
+    vp = (C.c_void_p * n_layers)(*v_bufs)
+
+    def native_loop(n: int):
+        ms, wall_s = C.c_float(), C.c_double()
+        ok = bl.mlc_bench_decode_loop(
+            C.c_void_p(q_buf), kp, vp, C.c_size_t(n_layers), C.c_void_p(o_buf),
+            meta[0].ctypes.data_as(u32p), C.c_size_t(meta[0].size), meta[1].ctypes.data_as(u32p),
+            meta[2].ctypes.data_as(u32p), meta[3].ctypes.data_as(u32p), C.c_size_t(c.batch),
+            C.c_size_t(c.num_heads), C.c_size_t(c.kv_heads), C.c_size_t(c.head_dim),
+            C.c_size_t(c.page_size), C.c_int(int(c.apply_causal)), C.c_size_t(n),
+            C.byref(ms), C.byref(wall_s))
+        if not ok:
+            raise RuntimeError("decode loop failed: " + exe.lastError())
+        return ms.value, wall_s.value
+
+    def step(layer: int, flat=None, pos=None, causal=None) -> None:
+        ok = exe.encodePagedFlashAttention(q_buf, k_bufs[layer], v_bufs[layer], o_buf,
+                                           c.page_tables_flat if flat is None else flat,
+                                           c.page_table_offsets, c.seq_lens,
+                                           c.q_positions if pos is None else pos, c.batch, c.num_heads,
+                                           c.kv_heads, c.head_dim, c.page_size,
+                                           c.apply_causal if causal is None else causal)
+        if not ok:
+            raise RuntimeError("encodePagedFlashAttention failed: " + exe.lastError())
+
+    # set-up: one untimed pass over every pool (the first launch that touches a pool pays for its
+    # address translations), then the --warmup steps
+    native_loop(n_layers)
+    if warmup:
+        native_loop(warmup)
+
+    # ---- timed region: exactly `steps` steps, device idle on both sides (the loop starts on an
+    # idle stream and returns after the stream has drained); HIP events bracket the same region
+    # on the kernels' stream.
+    ev_ms, wall = native_loop(steps)
+    r = {"case": c, "n_layers": n_layers, "steps": steps, "ev_us": ev_ms / steps * 1e3, "wall_us": wall / steps * 1e6,
+         "launches": exe.lastDecodeLaunches(), "items": exe.lastDecodeWorkItems(), "kernel": exe.lastDecodeKernel()}
+
+    if full:
+        # ---- one launch at a time, HIP events around each (the reference's harness reports its
+        # timings this way: warm-up, >= 200 iterations, median and p10 / p90,
+        # tools/paged_flash_bench.cpp:55-76)
+        singles = []
+        exe.beginForwardPassCB()
+        for i in range(203):
+            exe.timerStart()
+            step(i % n_layers)
+            t = exe.timerStopMs()
+            if i >= 3:
+                singles.append(t * 1e3)
+        exe.flushForwardPassCB()
+        singles.sort()
+        r["single_us"] = {"median": round(singles[len(singles) // 2], 2), "p10": round(singles[len(singles) // 10], 2),
+                          "p90": round(singles[len(singles) * 9 // 10], 2), "n": len(singles)}
+
+        # ---- boundary-inclusive figures: what a caller sees whose tables change with every call.
+        # (a) the per-request arrays change (one query position alternates); (b) the page table's
+        # content changes too (two page ids of one request trade places: same bytes read), so
+        # the device copy of the table is refreshed by every call.
+        n_b = min(steps, 200)
+        for key, swap_pages in (("tables_change_us", False), ("page_table_changes_us", True)):
+            pos = c.q_positions.copy()
+            flat2 = c.page_tables_flat.copy()
+            big = int(np.argmax(c.seq_lens))
+            o0 = int(c.page_table_offsets[big])
+            if int(c.page_table_offsets[big + 1]) - o0 >= 2:
+                flat2[o0], flat2[o0 + 1] = flat2[o0 + 1], flat2[o0]
+            exe.beginForwardPassCB()
+            exe.timerStart()
+            tb = time.perf_counter()
+            for i in range(n_b):
+                pos2 = pos.copy()
+                pos2[0] = pos[0] - (i % 2)
+                step(i % n_layers, flat=(flat2 if (swap_pages and i % 2) else None), pos=pos2, causal=False)
+            ev = exe.timerStopMs()
+            assert exe.flushForwardPassCB()
+            r[key] = {"wall": round((time.perf_counter() - tb) / n_b * 1e6, 3), "events": round(ev / n_b * 1e3, 3)}
+
+        # ---- fp32 softmax weights for P.V (decode_pv_fp16 = 0: meets the reference's 1e-5 gate)
+        assert exe.setOption("decode_pv_fp16", 0)
+        native_loop(n_layers)
+        ev32, _ = native_loop(steps)
+        assert exe.setOption("decode_pv_fp16", 1)
+        r["pv_fp32_us"] = ev32 / steps * 1e3
+
+        # ---- a plain streaming read of the same number of bytes from the same pools
+        each = min(c.kv_bytes // 2 // 16 * 16, pool_bytes)
+        ms_r = C.c_float()
+        bl.mlc_bench_read_loop(kp, vp, C.c_size_t(n_layers), C.c_size_t(each), C.c_size_t(n_layers), C.byref(ms_r))
+        assert bl.mlc_bench_read_loop(kp, vp, C.c_size_t(n_layers), C.c_size_t(each), C.c_size_t(steps), C.byref(ms_r))
+        r["stream_read"] = {"bytes": 2 * each, "us_per_launch": ms_r.value / steps * 1e3}
+
+    # ---- the layer as the batched step runs it (batched_walker.cpp:304-331): write the step's
+    # new K row and V row (they land on the newest position: the bytes read stay the same), then
+    # attend.  Three encode calls per layer; the attention launch carries the two scatters.
+    rng = np.random.default_rng(5)
+    row = c.kv_heads * c.head_dim
+    new_k = rng.standard_normal((c.batch, row)).astype(np.float16)
+    new_v = rng.standard_normal((c.batch, row)).astype(np.float16)
+    nk_buf, nv_buf = exe.allocateScratchBuffer(new_k.nbytes), exe.allocateScratchBuffer(new_v.nbytes)
+    assert exe.uploadToBuffer(nk_buf, new_k) and exe.uploadToBuffer(nv_buf, new_v)
+    last = np.maximum(c.seq_lens.astype(np.int64) - 1, 0)
+    ids = np.array([c.page_tables_flat[c.page_table_offsets[i] + last[i] // c.page_size] if c.seq_lens[i] else 0
+                    for i in range(c.batch)], np.uint32)
+    slots = (last % c.page_size).astype(np.uint32)
+    n_w = max(1, min(steps, 500))
+    ms_w, wall_w = C.c_float(), C.c_double()
+    ok = bl.mlc_bench_decode_step_loop(
+        C.c_void_p(q_buf), kp, vp, C.c_size_t(n_layers), C.c_void_p(o_buf), C.c_void_p(nk_buf), C.c_void_p(nv_buf),
+        ids.ctypes.data_as(u32p), slots.ctypes.data_as(u32p),
+        meta[0].ctypes.data_as(u32p), C.c_size_t(meta[0].size), meta[1].ctypes.data_as(u32p),
+        meta[2].ctypes.data_as(u32p), meta[3].ctypes.data_as(u32p), C.c_size_t(c.batch),
+        C.c_size_t(c.num_heads), C.c_size_t(c.kv_heads), C.c_size_t(c.head_dim), C.c_size_t(c.page_size),
+        C.c_size_t(n_w), C.byref(ms_w), C.byref(wall_w))
+    if not ok:
+        raise RuntimeError("decode step loop failed: " + exe.lastError())
+    r["kv_write_us"] = ms_w.value / n_w * 1e3
+    r["kv_write_steps"] = n_w
+    # the pools now hold the new rows at the newest positions: the parity check below uses them
+    for attr, new in (("k_pages", new_k), ("v_pages", new_v)):
+        p2 = getattr(c, attr).copy().view(np.uint16).reshape(-1, c.page_size, row)
+        for i in range(c.batch):
+            if c.seq_lens[i]:
+                p2[ids[i], slots[i]] = new[i].view(np.uint16)
+        setattr(c, attr, p2.reshape(-1))
+
+    out = np.empty(c.q.shape, np.float32)
+    exe.beginForwardPassCB()
+    step(0)
+    exe.flushForwardPassCB()
+    exe.downloadFromBuffer(o_buf, out)
+    for b in [q_buf, o_buf, nk_buf, nv_buf] + k_bufs + v_bufs:
+        exe.releaseScratchBuffer(b)
+
+    if not args.no_cpu:
+        cpu, outs = cpu_baseline(case, cpu_budget)
+        from oracle import paged_oracle as po
+        worst_cos, worst_abs = 1.0, 0.0
+        for i, o in outs.items():
+            rep = po.per_head_report(out[i], o, c.head_dim)
+            worst_cos = min(worst_cos, rep["min_cosine"])
+            worst_abs = max(worst_abs, rep["max_abs"])
+        r["cpu"] = cpu
+        r["parity"] = {"min_cosine": round(worst_cos, 7), "max_abs": float(f"{worst_abs:.3e}"),
+                       "requests_checked": len(outs)}
+    return r
+
+
+def workload_text(c, n_layers) -> str:
+    return (f"{c.name}: batched paged decode attention, batch {c.batch}, "
+            f"{c.num_heads}q/{c.kv_heads}kv heads, head_dim {c.head_dim}, "
+            f"contexts {int(c.seq_lens.min())}..{int(c.seq_lens.max())} "
+            f"(sum {int(c.seq_lens.sum())}), {c.page_size}-token fp16 pages permuted in a "
+            f"{c.capacity_pages}-page pool, {n_layers} layer pools rotated")
+
+
+def per_config_entry(name: str, r: dict) -> dict:
+    """One decode configuration as an entry of config.per_config: every figure can be recomputed
+    from kv_bytes_per_step and the microseconds beside it."""
+    c = r["case"]
+    with_write = name == "cfg3"   # the step of configuration 3 is scatter K, scatter V, attention
+    us = r["kv_write_us"] if with_write else r["ev_us"]
+    e = {"workload": workload_text(c, r["n_layers"]),
+         "step": "scatter K row, scatter V row, attention (one launch: the attention kernel carries the write)"
+                 if with_write else "attention",
+         "steps": r["kv_write_steps"] if with_write else r["steps"],
+         "kv_bytes_per_step": c.kv_bytes, "us_per_step": round(us, 3),
+         "GBs": round(c.kv_bytes / us / 1e3, 1), "frac_of_hbm_peak": round(c.kv_bytes / us / 1e3 / HBM_PEAK_GBS, 4),
+         "us_attention_only": round(r["ev_us"], 3), "kernel": r["kernel"], "work_items": r["items"],
+         "traffic": load_traffic(name, r["kernel"], r["items"])}
+    if "cpu" in r:
+        e["cpu_baseline"] = r["cpu"]
+        e["parity_vs_cpu_baseline"] = r["parity"]
+    return e
+
+
+def bench_refbench(args) -> int:
+    """The reference's own micro-benchmark grid (tools/paged_flash_bench.cpp:29-34, 206-226):
+    32 query heads, 4 KV heads, head_dim 64, one 64-token page per request, batch 1, 2, 4, 8;
+    3 warm-up calls, then 200 synchronous runPagedFlashAttention calls timed one by one on the
+    host clock (as the reference's harness does, :55-76), median / p10 / p90 in microseconds; beside
+    it the same calls timed with a HIP event pair on the stream."""
+    from mlcompiler_amd import HipExecutor
+    from paged_cases import DeviceCase, make_case
+    exe = HipExecutor.Instance()
+    exe.requireAvailable()
+    rows = []
+    for b in (1, 2, 4, 8):
+        case = make_case(f"refbench_b{b}", b, 32, 4, 64, 64, [64] * b, capacity_pages=b, permute=False, seed=42,
+                         dist="uniform")
+        d = DeviceCase(exe, case)
+        host, dev = [], []
+        a = (d.q_buf, d.k_buf, d.v_buf, d.o_buf, case.page_tables_flat, case.page_table_offsets, case.seq_lens,
+             case.q_positions, case.batch, case.num_heads, case.kv_heads, case.head_dim, case.page_size,
+             case.apply_causal)
+        for i in range(203):
+            t0 = time.perf_counter()
+            assert exe.runPagedFlashAttention(*a), exe.lastError()
+            t = (time.perf_counter() - t0) * 1e6
+            if i >= 3:
+                host.append(t)
+        exe.beginForwardPassCB()
+        for i in range(203):
+            exe.timerStart()
+            assert exe.encodePagedFlashAttention(*a), exe.lastError()
+            t = exe.timerStopMs() * 1e3
+            if i >= 3:
+                dev.append(t)
+        exe.flushForwardPassCB()
+        d.free()
+        host.sort()
+        dev.sort()
+        pick = lambda v: {"median": round(v[len(v) // 2], 2), "p10": round(v[len(v) // 10], 2),
+                          "p90": round(v[len(v) * 9 // 10], 2)}
+        rows.append({"batch": b, "host_sync_call_us": pick(host), "stream_event_us": pick(dev), "n": len(host)})
+    print(json.dumps({"metric": "paged flash attention micro-benchmark of the reference (median us per call)",
+                      "value": rows[-1]["host_sync_call_us"]["median"], "unit": "us", "n_gpus": 1, "steps": 200,
+                      "warmup": 3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+                      "dtype": "f32 (fp16 K/V storage, fp32 q, accumulate and output)", "data": "synthetic",
+                      "config": {"workload": "tools/paged_flash_bench.cpp grid: 32q/4kv heads, head_dim 64, one "
+                                             "64-token page per request, batch 1/2/4/8, uniform(-0.5, 0.5) inputs",
+                                 "rows": rows}}))
+    return 0
 
 
 def main() -> int:
@@ -469,7 +753,11 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=100)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "layer", "step", "copy"])
+    ap.add_argument("--workload", default="cfg2",
+                    choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "layer", "step", "copy", "refbench"])
+    ap.add_argument("--per-config", type=int, default=-1,
+                    help="1: add config.per_config (configurations 1, 3, 4 and 5, each with its own bounded CPU "
+                         "baseline) to the line; default: only for the default workload")
     ap.add_argument("--copy-mib", type=int, default=32, help="size of the calibration copy")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU baseline work")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -492,9 +780,12 @@ def main() -> int:
         return 2
 
     if args.workload == "cfg5":
-        return bench_prefill(args)
+        print(json.dumps(bench_prefill(args)))
+        return 0
     if args.workload == "copy":
         return bench_copy(args)
+    if args.workload == "refbench":
+        return bench_refbench(args)
     if args.workload in ("layer", "step"):
         return bench_layer(args)
 
@@ -513,146 +804,18 @@ def main() -> int:
         name, value = kv.split("=")
         assert exe.setOption(name, int(value)), f"unknown option {kv}"
 
-    case, n_layers = build_workload(args.workload)
-    c = case
-    pool_bytes = c.k_pages.nbytes
-    q_buf = exe.allocateScratchBuffer(c.q.nbytes)
-    o_buf = exe.allocateScratchBuffer(c.q.nbytes)
-    assert exe.uploadToBuffer(q_buf, c.q)
-    k_bufs, v_bufs = [], []
-    for _ in range(n_layers):
-        kb = exe.allocateScratchBuffer(pool_bytes)
-        vb = exe.allocateScratchBuffer(pool_bytes)
-        assert kb and vb, "out of device memory"
-        assert exe.uploadToBuffer(kb, c.k_pages) and exe.uploadToBuffer(vb, c.v_pages)
-        k_bufs.append(kb)
-        v_bufs.append(vb)
-
-    import ctypes as C
-    from mlcompiler_amd.build import BENCH_LIB_PATH
-    bl = C.CDLL(BENCH_LIB_PATH)   # native loop around the C ABI (no Python between launches)
-    u32p = C.POINTER(C.c_uint32)
-    meta = [np.ascontiguousarray(x, np.uint32) for x in
-            (c.page_tables_flat, c.page_table_offsets, c.seq_lens, c.q_positions)]
-    kp = (C.c_void_p * n_layers)(*k_bufs)
-    vp = (C.c_void_p * n_layers)(*v_bufs)
-
-    def native_loop(steps: int):
-        ms, wall_s = C.c_float(), C.c_double()
-        ok = bl.mlc_bench_decode_loop(
-            C.c_void_p(q_buf), kp, vp, C.c_size_t(n_layers), C.c_void_p(o_buf),
-            meta[0].ctypes.data_as(u32p), C.c_size_t(meta[0].size), meta[1].ctypes.data_as(u32p),
-            meta[2].ctypes.data_as(u32p), meta[3].ctypes.data_as(u32p), C.c_size_t(c.batch),
-            C.c_size_t(c.num_heads), C.c_size_t(c.kv_heads), C.c_size_t(c.head_dim),
-            C.c_size_t(c.page_size), C.c_int(int(c.apply_causal)), C.c_size_t(steps),
-            C.byref(ms), C.byref(wall_s))
-        if not ok:
-            raise RuntimeError("decode loop failed: " + exe.lastError())
-        return ms.value, wall_s.value
-
-    def step(layer: int) -> None:
-        ok = exe.encodePagedFlashAttention(q_buf, k_bufs[layer], v_bufs[layer], o_buf,
-                                           c.page_tables_flat, c.page_table_offsets, c.seq_lens,
-                                           c.q_positions, c.batch, c.num_heads, c.kv_heads,
-                                           c.head_dim, c.page_size, c.apply_causal)
-        if not ok:
-            raise RuntimeError("encodePagedFlashAttention failed: " + exe.lastError())
-
-    if args.warmup:
-        native_loop(args.warmup)
-
-    # ---- timed region: exactly --steps steps, device idle on both sides (the loop starts
-    # on an idle stream and returns after the stream has drained); HIP events bracket the
-    # same region on the kernels' stream.
-    ev_ms, wall = native_loop(args.steps)
-    launches = exe.lastDecodeLaunches()
-    items = exe.lastDecodeWorkItems()
-
-    # ---- one launch at a time, HIP events around each (the reference's harness reports its
-    # timings this way: warm-up, >= 200 iterations, median and p10 / p90,
-    # tools/paged_flash_bench.cpp:55-76)
-    singles = []
-    exe.beginForwardPassCB()
-    for i in range(203):
-        exe.timerStart()
-        step(i % n_layers)
-        t = exe.timerStopMs()
-        if i >= 3:
-            singles.append(t * 1e3)
-    exe.flushForwardPassCB()
-    singles.sort()
-    single_us = {"median": round(singles[len(singles) // 2], 2), "p10": round(singles[len(singles) // 10], 2),
-                 "p90": round(singles[len(singles) * 9 // 10], 2), "n": len(singles)}
-
-    # ---- boundary-inclusive figure: tables change every call, so each call re-plans and
-    # re-uploads its metadata (what a caller that rebuilds its tables per layer would see)
-    n_b = min(args.steps, 200)
-    pos = c.q_positions.copy()
-    exe.beginForwardPassCB()
-    tb = time.perf_counter()
-    for i in range(n_b):
-        pos2 = pos.copy()
-        pos2[0] = pos[0] - (i % 2)  # alternate one q position (non-causal effect: none on bytes)
-        ok = exe.encodePagedFlashAttention(q_buf, k_bufs[i % n_layers], v_bufs[i % n_layers], o_buf,
-                                           c.page_tables_flat, c.page_table_offsets, c.seq_lens,
-                                           pos2, c.batch, c.num_heads, c.kv_heads, c.head_dim,
-                                           c.page_size, False)
-        assert ok, exe.lastError()
-    assert exe.flushForwardPassCB()
-    boundary_us = (time.perf_counter() - tb) / n_b * 1e6
-
-    # ---- the layer as the batched step runs it (batched_walker.cpp:304-331): write the step's
-    # new K row and V row (they land on the newest position: the bytes read stay the same), then
-    # attend.  Three encode calls per layer; the attention launch carries the two scatters.
-    rng = np.random.default_rng(5)
-    row = c.kv_heads * c.head_dim
-    new_k = rng.standard_normal((c.batch, row)).astype(np.float16)
-    new_v = rng.standard_normal((c.batch, row)).astype(np.float16)
-    nk_buf, nv_buf = exe.allocateScratchBuffer(new_k.nbytes), exe.allocateScratchBuffer(new_v.nbytes)
-    assert exe.uploadToBuffer(nk_buf, new_k) and exe.uploadToBuffer(nv_buf, new_v)
-    last = np.maximum(c.seq_lens.astype(np.int64) - 1, 0)
-    ids = np.array([c.page_tables_flat[c.page_table_offsets[r] + last[r] // c.page_size] if c.seq_lens[r] else 0
-                    for r in range(c.batch)], np.uint32)
-    slots = (last % c.page_size).astype(np.uint32)
-    n_w = max(1, min(args.steps, 500))
-    ms_w, wall_w = C.c_float(), C.c_double()
-    ok = bl.mlc_bench_decode_step_loop(
-        C.c_void_p(q_buf), kp, vp, C.c_size_t(n_layers), C.c_void_p(o_buf), C.c_void_p(nk_buf), C.c_void_p(nv_buf),
-        ids.ctypes.data_as(u32p), slots.ctypes.data_as(u32p),
-        meta[0].ctypes.data_as(u32p), C.c_size_t(meta[0].size), meta[1].ctypes.data_as(u32p),
-        meta[2].ctypes.data_as(u32p), meta[3].ctypes.data_as(u32p), C.c_size_t(c.batch),
-        C.c_size_t(c.num_heads), C.c_size_t(c.kv_heads), C.c_size_t(c.head_dim), C.c_size_t(c.page_size),
-        C.c_size_t(n_w), C.byref(ms_w), C.byref(wall_w))
-    if not ok:
-        raise RuntimeError("decode step loop failed: " + exe.lastError())
-    kv_write_us = wall_w.value / n_w * 1e6
-    # the pools now hold the new rows at the newest positions: the parity check below uses them
-    kv_after = {}
-    for name, pool, new in (("k", c.k_pages, new_k), ("v", c.v_pages, new_v)):
-        p2 = pool.copy().view(np.uint16).reshape(-1, c.page_size, row)
-        for r in range(c.batch):
-            if c.seq_lens[r]:
-                p2[ids[r], slots[r]] = new[r].view(np.uint16)
-        kv_after[name] = p2.reshape(-1)
-    c.k_pages, c.v_pages = kv_after["k"], kv_after["v"]
-
-    out = np.empty(c.q.shape, np.float32)
-    exe.beginForwardPassCB()
-    step(0)
-    exe.flushForwardPassCB()
-    exe.downloadFromBuffer(o_buf, out)
-
+    per_config = args.per_config == 1 or (args.per_config < 0 and args.workload == "cfg2" and not args.no_cpu)
+    r = run_decode(args, args.workload, args.steps, args.warmup, args.cpu_budget, full=True)
+    c = r["case"]
     kv_bytes = c.kv_bytes
-    ms_per_step = wall / args.steps * 1e3
-    value = kv_bytes / (wall / args.steps) / 1e9
-    ev_us = ev_ms / args.steps * 1e3
-    achieved = kv_bytes / (ev_ms / args.steps * 1e-3) / 1e9
-
-    # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs),
-    # scaled by the copy-kernel calibration (x2.0 / x1.0); valid for the default planner only.
-    measured_traffic = {"cfg2": 44_220_000, "cfg3": 142_580_000, "cfg4": 1_203_400_000}
-    traffic = measured_traffic.get(args.workload) if not args.target_items else None
-
+    # `value` and `ms_per_step` come from the HIP-event time of the timed region (device time of
+    # exactly --steps steps, gaps between launches included).  The host clock around the same
+    # region adds the one-off latency of the first launch and of the final synchronisation
+    # (about 40 us): at --steps 20 that is a tenth of the region, so it is reported beside it
+    # (wall_us_per_step) instead of being folded into the rate.
+    ev_us = r["ev_us"]
+    value = kv_bytes / ev_us / 1e3
+    sr = r["stream_read"]
     result = {
         "metric": "decode attn KV-read GB/s (% of HBM peak) & us/layer, TinyLlama shape B=32",
         "value": round(value, 2),
@@ -660,51 +823,64 @@ def main() -> int:
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 6),
+        "ms_per_step": round(ev_us / 1e3, 6),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32 (fp16 K/V storage, fp32 q, accumulate and output)",
+        "dtype": "f32 accumulate and output (fp16 K/V storage, fp32 q; softmax weights rounded to fp16 for P.V, "
+                 "option decode_pv_fp16: us_per_layer_pv_fp32 is the time with fp32 weights)",
         "data": "synthetic",
         "config": {
-            "workload": f"{c.name}: batched paged decode attention, batch {c.batch}, "
-                        f"{c.num_heads}q/{c.kv_heads}kv heads, head_dim {c.head_dim}, "
-                        f"contexts {int(c.seq_lens.min())}..{int(c.seq_lens.max())} "
-                        f"(sum {int(c.seq_lens.sum())}), {c.page_size}-token fp16 pages permuted in a "
-                        f"{c.capacity_pages}-page pool, {n_layers} layer pools rotated",
+            "workload": workload_text(c, r["n_layers"]),
             "kv_bytes_per_step": kv_bytes,
-            "us_per_layer": round(ms_per_step * 1e3, 3),
+            "us_per_layer": round(ev_us, 3),
+            "wall_us_per_step": round(r["wall_us"], 3),
+            "setup_steps_before_warmup": r["n_layers"],
             "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
-            "kernels_per_step": launches,
-            "work_items": items,
-            "us_per_layer_with_metadata_upload": round(boundary_us, 3),
-            "single_launch_us": single_us,
-            "us_per_layer_with_kv_write": round(kv_write_us, 3),
+            "kernels_per_step": r["launches"],
+            "kernel": r["kernel"],
+            "work_items": r["items"],
+            "us_per_layer_pv_fp32": round(r["pv_fp32_us"], 3),
+            "us_per_layer_tables_change": r["tables_change_us"],
+            "us_per_layer_page_table_changes": r["page_table_changes_us"],
+            "single_launch_us": r["single_us"],
+            "us_per_layer_with_kv_write": round(r["kv_write_us"], 3),
+            "host_cores": os.cpu_count(),
         },
         "roofline": {
             "bound": "hbm",
-            "achieved": round(achieved, 2),
+            "achieved": round(value, 2),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": traffic,
+            "frac": round(value / HBM_PEAK_GBS, 4),
+            "traffic": load_traffic(args.workload, r["kernel"], r["items"]),
+            "traffic_source": "profiles/traffic.json (rocprofv3 FETCH_SIZE / WRITE_SIZE of this kernel variant and "
+                              "work split; null when this run's differ from the profiled ones)",
             "us_per_launch": round(ev_us, 3),
-            "note": "HIP events around the timed region on the library stream / steps: one step = "
+            "stream_read_ceiling": {"bytes": sr["bytes"], "us_per_launch": round(sr["us_per_launch"], 3),
+                                    "GBs": round(sr["bytes"] / sr["us_per_launch"] / 1e3, 1),
+                                    "frac": round(sr["bytes"] / sr["us_per_launch"] / 1e3 / HBM_PEAK_GBS, 4),
+                                    "note": "a kernel that only reads the same number of bytes contiguously from "
+                                            "the same pools, same run, same timing"},
+            "note": "HIP events around the timed region on the library stream / steps: one step = one "
                     "decode kernel (split requests are merged inside it by the last workgroup to arrive)",
         },
     }
-    if not args.no_cpu:
-        cpu, outs = cpu_baseline(case, args.cpu_budget)
-        result["cpu_baseline"] = cpu
-        from oracle import paged_oracle as po
-        worst_cos, worst_abs = 1.0, 0.0
-        for r, o in outs.items():
-            rep = po.per_head_report(out[r], o, c.head_dim)
-            worst_cos = min(worst_cos, rep["min_cosine"])
-            worst_abs = max(worst_abs, rep["max_abs"])
-        result["parity_vs_cpu_baseline"] = {"min_cosine": round(worst_cos, 7),
-                                            "max_abs": float(f"{worst_abs:.3e}"),
-                                            "requests_checked": len(outs)}
+    if "cpu" in r:
+        result["cpu_baseline"] = r["cpu"]
+        result["parity_vs_cpu_baseline"] = r["parity"]
+    if per_config:
+        pc = {}
+        for name, st in (("cfg1", min(args.steps, 2000)), ("cfg3", min(args.steps, 500)), ("cfg4", min(args.steps, 100))):
+            sub = run_decode(args, name, st, min(args.warmup, st), 4.0, full=False)
+            pc[name] = per_config_entry(name, sub)
+        p5 = bench_prefill(args)
+        pc["cfg5"] = {"workload": p5["config"]["workload"], "steps": p5["steps"],
+                      "flop_per_step": p5["config"]["flop_per_step"],
+                      "us_per_step": p5["roofline"]["us_per_launch"], "TFLOPs": p5["roofline"]["achieved"],
+                      "frac_of_mfma_f16_peak": p5["roofline"]["frac"], "traffic": p5["roofline"]["traffic"],
+                      **{k: p5[k] for k in ("cpu_baseline", "parity_vs_cpu_baseline") if k in p5}}
+        result["config"]["per_config"] = pc
     print(json.dumps(result))
     return 0
 

@@ -259,6 +259,10 @@ float mlc_hip_timer_stop(void);
  * number of split-K work items it planned (for benchmarks and tests). */
 int mlc_hip_last_decode_launches(void);
 int mlc_hip_last_decode_work_items(void);
+/* Name of the kernel variant the last decode call launched, with its template arguments, e.g.
+ * "stream<64,2,4,pv16,regs,2>" (head_dim, query heads per wave, waves per group, softmax-weight
+ * type, where the per-request figures live, LDS stages), "planned<...>" or "generic". */
+const char* mlc_hip_last_decode_kernel(void);
 /* Number of KV writes so far that went out fused with a neighbour: a batched K scatter with its
  * V twin, or split + RoPE + cast with the scatters of its fp16 rows (for tests). */
 long mlc_hip_fused_kv_write_launches(void);

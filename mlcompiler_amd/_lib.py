@@ -50,6 +50,7 @@ SIGNATURES = {
     "mlc_hip_timer_stop": (C.c_float, []),
     "mlc_hip_last_decode_launches": (C.c_int, []),
     "mlc_hip_last_decode_work_items": (C.c_int, []),
+    "mlc_hip_last_decode_kernel": (C.c_char_p, []),
     "mlc_hip_row_program_launches": (C.c_long, []),
     "mlc_hip_decode_table_uploads": (C.c_long, []),
     "mlc_hip_fused_kv_write_launches": (C.c_long, []),

@@ -20,7 +20,43 @@ __global__ __launch_bounds__(256) void mlc_bench_copy_kernel(const uint4* __rest
         dst[i] = src[i];
 }
 
+// Plain streaming read: every thread loads 16-byte units with a grid stride and folds them into
+// one word that is stored only if it has a value it never has.  The same number of bytes as a
+// decode launch, read contiguously with nothing else to do: the practical ceiling of the memory
+// system for a launch of that size, quoted beside the decode kernel.
+__global__ __launch_bounds__(256) void mlc_bench_read_kernel(const uint4* __restrict__ a, const uint4* __restrict__ b,
+                                                             size_t n_each, uint32_t* sink) {
+    uint32_t acc = 0;
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n_each; i += stride) {
+        const uint4 x = a[i], y = b[i];
+        acc ^= x.x ^ x.y ^ x.z ^ x.w ^ y.x ^ y.y ^ y.z ^ y.w;
+    }
+    if (acc == 0x9E3779B9u && sink) sink[0] = acc;
+}
+
 extern "C" {
+
+// `steps` launches of the streaming-read kernel, launch i reading the first bytes_each bytes of
+// K pool and V pool i % n_layers (device buffers of at least that size) on the library's stream;
+// reports the HIP-event time of the region in milliseconds.
+int mlc_bench_read_loop(void* const* k_pools, void* const* v_pools, size_t n_layers, size_t bytes_each,
+                        size_t steps, float* event_ms) {
+    hipStream_t stream = static_cast<hipStream_t>(mlc_hip_stream());
+    if (!stream || !k_pools || !v_pools || !n_layers) return 0;
+    const size_t n = bytes_each / 16;
+    const size_t want = (n + 255) / 256;
+    const unsigned grid = (unsigned)(want < 256 * 8 ? (want ? want : 1) : 256 * 8);
+    if (!mlc_hip_timer_start()) return 0;
+    for (size_t i = 0; i < steps; ++i)
+        hipLaunchKernelGGL(mlc_bench_read_kernel, dim3(grid), dim3(256), 0, stream,
+                           static_cast<const uint4*>(k_pools[i % n_layers]),
+                           static_cast<const uint4*>(v_pools[i % n_layers]), n, static_cast<uint32_t*>(nullptr));
+    const float ms = mlc_hip_timer_stop();
+    if (ms < 0.f) return 0;
+    if (event_ms) *event_ms = ms;
+    return 1;
+}
 
 // Enqueues `steps` decode-attention layer calls (encode variant, one open pass), layer i
 // reading K/V pool i % n_layers, and reports the HIP-event time of the whole region

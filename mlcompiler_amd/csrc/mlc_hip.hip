@@ -222,6 +222,7 @@ struct Ctx {
     long opt_pv_fp16 = 1;                                      // softmax weights rounded to fp16 for P.V
     int last_launches = 0;
     int last_items = 0;
+    char last_kernel[96] = "";   // kernel variant of the last decode launch (for benchmarks)
     int n_cu = 256;
     unsigned char* scratch_ptr = nullptr;   // device address of `scratch` on g.device
     StreamTables tables;
@@ -1151,6 +1152,8 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
         if (!launch_stream_variant(head_dim, s_hpw, s_nw, nbuf, a, n_wg, dyn_lds, g.stream))
             return fail("decode: kernel variant not built");
         g.last_items = (int)std::min<uint64_t>(n_wg, total_tiles);
+        std::snprintf(g.last_kernel, sizeof g.last_kernel, "stream<%zu,%d,%d,%s,%s,%d>", head_dim, s_hpw, s_nw,
+                      g.opt_pv_fp16 ? "pv16" : "pv32", batch <= 64 ? "regs" : "lds", nbuf);
         if (carries_kv) {
             g.kv.active = false;
             ++g.kv_fused;
@@ -1192,6 +1195,8 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
             a.new_slots = g.kv.d_slots;
         }
         if (!launch_fast(head_dim, p.hpw, p.nw, p.ns, p.nbuf, a)) return fail("decode: kernel variant not built");
+        std::snprintf(g.last_kernel, sizeof g.last_kernel, "planned<%zu,%d,%d,%d,%d,%s>", head_dim, p.hpw, p.nw, p.ns,
+                      p.nbuf, g.opt_pv_fp16 ? "pv16" : "pv32");
         if (carries_kv) {
             g.kv.active = false;
             ++g.kv_fused;
@@ -1214,6 +1219,7 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
         a.scale_log2e = scale_log2e;
         hipLaunchKernelGGL(paged_decode_generic_kernel, dim3((unsigned)(batch * num_heads)),
                            dim3(64), 0, g.stream, a);
+        std::snprintf(g.last_kernel, sizeof g.last_kernel, "generic");
         ++g.last_launches;
     }
     if (!slot_mark(slot)) return 0;
@@ -2066,6 +2072,7 @@ float mlc_hip_timer_stop(void) {
 
 int mlc_hip_last_decode_launches(void) { return g.last_launches; }
 int mlc_hip_last_decode_work_items(void) { return g.last_items; }
+const char* mlc_hip_last_decode_kernel(void) { return g.last_kernel; }
 long mlc_hip_fused_kv_write_launches(void) { return g.kv_fused; }
 long mlc_hip_fused_matmul_rope_launches(void) { return g.gemm_rope_fused; }
 long mlc_hip_kv_writes_in_decode_launches(void) { return g.kv_in_decode; }
@@ -2077,7 +2084,7 @@ long mlc_hip_decode_table_uploads(void) { return g.table_uploads; }
 int mlc_hip_debug_probe(uint64_t* dst, size_t n_wg) {
     if (!init_once()) return 0;
     HIP_OK(hipStreamSynchronize(g.stream));
-    HIP_OK(hipMemcpy(dst, g.scratch_ptr + kScratchPartOBytes + 65536 * 4, n_wg * 64, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(dst, g.scratch_ptr + kScratchPartOBytes + 65536 * 4, n_wg * 256, hipMemcpyDeviceToHost));
     return 1;
 }
 #endif

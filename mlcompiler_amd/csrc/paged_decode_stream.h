@@ -69,7 +69,7 @@ inline size_t stream_dynamic_lds_bytes(size_t batch) { return (3 * batch + 1) * 
 #define MLC_PROBE(i)                                                                                   \
     do {                                                                                               \
         if (threadIdx.x == 0)                                                                          \
-            reinterpret_cast<uint64_t*>(a.part_ml + 65536)[blockIdx.x * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); \
+            reinterpret_cast<uint64_t*>(a.part_ml + 65536)[blockIdx.x * 32 + (i)] = __builtin_amdgcn_s_memrealtime(); \
     } while (0)
 #else
 #define MLC_PROBE(i)
@@ -645,11 +645,14 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         // write-through stores are complete once this wave's memory counter is zero.
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         sd_wait_vmcnt<0>();
+        MLC_PROBE(26);
         uint32_t ticket = 0;
         uint32_t* counter = &a.counters[(size_t)w_lo * NW + hg];
         if (lane == 0) ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         ticket = __shfl(ticket, 0);
+        MLC_PROBE(27);
         if (ticket != n_splits - 1u) return;
+        MLC_PROBE(28);
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
         if (lane == 0)  // ready for the next launch
             __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -735,9 +738,11 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     uint32_t slot = 0;        // stage of tile k
     for (uint32_t k = 0; k < n; ++k) {
         // this wave's loads of tile k have landed ...
+        if (k < 6) MLC_PROBE(8 + 3 * k);
         if (drain) sd_wait_vmcnt<0>(); else wait_tile(issued - k - 1u);
         drain = false;
         sd_barrier();   // ... and everyone's; everyone has left tile k-1, whose stage is free
+        if (k < 6) MLC_PROBE(9 + 3 * k);
         if (k == 0) MLC_PROBE(3);
         if (k >= 1 && issued < n) {
             advance(ci);
@@ -749,6 +754,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         consume_tile(slot, cc.t, cc.lim);
 #endif
         const bool pair_done = cc.t + 1u == cc.tiles;
+        if (k < 6) MLC_PROBE(10 + 3 * k);
         if (k + 1 == n) MLC_PROBE(4);
         if (pair_done || k + 1 == n) {
             finalize(cc, seg_first, g0 + k + 1u);
@@ -765,9 +771,9 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     MLC_PROBE(5);
 #ifdef MLC_STREAM_PROBE
     if (threadIdx.x == 0) {
-        reinterpret_cast<uint64_t*>(a.part_ml + 65536)[blockIdx.x * 8 + 6] = n;
+        reinterpret_cast<uint64_t*>(a.part_ml + 65536)[blockIdx.x * 32 + 6] = n;
         const uint64_t hw = __builtin_amdgcn_s_getreg((31 << 11) | 4), xcc = __builtin_amdgcn_s_getreg((31 << 11) | 20);
-        reinterpret_cast<uint64_t*>(a.part_ml + 65536)[blockIdx.x * 8 + 7] = hw | (xcc << 32);
+        reinterpret_cast<uint64_t*>(a.part_ml + 65536)[blockIdx.x * 32 + 7] = hw | (xcc << 32);
     }
 #endif
 }

@@ -251,6 +251,9 @@ class HipExecutor:
     def lastDecodeWorkItems(self) -> int:
         return int(self._lib.mlc_hip_last_decode_work_items())
 
+    def lastDecodeKernel(self) -> str:
+        return (self._lib.mlc_hip_last_decode_kernel() or b"").decode()
+
     def fusedKvWriteLaunches(self) -> int:
         """KV writes so far that went out fused with a neighbour (option "fuse_row_ops")."""
         return int(self._lib.mlc_hip_fused_kv_write_launches())
