@@ -245,6 +245,32 @@ int mlc_hip_paged_attn_prefill(const void* q_f16, const void* k_pages, const voi
                                size_t batch, size_t chunk, size_t num_heads, size_t kv_heads,
                                size_t head_dim, size_t page_size_tokens, int sync);
 
+/* Decode attention for callers that cannot allocate (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same result as mlc_hip_paged_attn_decode (same kernel), but the call itself allocates no device
+ * or pinned memory and creates no stream or event: the kernel's scratch memory (split-K partial results and
+ * arrival counters, 8.5 MiB) is a static device array that every GPU the library runs on holds
+ * until the process ends; seq_lens, q_positions and page_table_offsets (HOST arrays, as above)
+ * travel inside the kernel arguments; the flat page table is read where the caller keeps it:
+ *   page_tables_flat_device  DEVICE pointer to n_page_tables_flat uint32 page ids (4-byte aligned)
+ *   stream                   hipStream_t to launch on; NULL = the library's stream
+ * Limits, refused with an error otherwise: batch <= 256; head_dim 64 or 128; GQA ratio 1, 2, 4, 8,
+ * 16 or 32; page size a multiple of 64 (head_dim 64) or 32 (head_dim 128) tokens; q, o and the
+ * pools 16-byte aligned.  mlc_hip_available() must have returned 1 before (set-up creates the
+ * library's stream and looks up the scratch array's device address).  The call returns when the
+ * kernel is enqueued (no synchronisation).  Every decode launch of this library on one GPU
+ * uses the same scratch array: launches must not overlap (two streams without an ordering
+ * between them race).  The page ids cannot be checked on the host; for pools obtained from
+ * mlc_hip_alloc the kernel clamps them below the pool's size. */
+int mlc_hip_paged_attn_decode_noalloc(const void* q, const void* k_pages, const void* v_pages, void* o,
+                                      const uint32_t* page_tables_flat_device, size_t n_page_tables_flat,
+                                      const uint32_t* page_table_offsets,
+                                      const uint32_t* seq_lens,
+                                      const uint32_t* q_positions,
+                                      size_t batch, size_t num_heads, size_t kv_heads,
+                                      size_t head_dim, size_t page_size_tokens, int apply_causal,
+                                      void* stream);
+
 /* ---- measurement helpers (no reference counterpart) ------------------------
  * The library's stream as a hipStream_t, for callers that need to order their
  * own work or events with it. */

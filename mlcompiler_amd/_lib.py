@@ -30,6 +30,8 @@ SIGNATURES = {
     "mlc_hip_has_open_pass": (C.c_int, []),
     "mlc_hip_paged_attn_decode": (C.c_int, [_vp, _vp, _vp, _vp, _u32p, _sz, _u32p, _u32p, _u32p,
                                             _sz, _sz, _sz, _sz, _sz, C.c_int, C.c_int]),
+    "mlc_hip_paged_attn_decode_noalloc": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _sz, _u32p, _u32p, _u32p,
+                                                    _sz, _sz, _sz, _sz, _sz, C.c_int, _vp]),
     "mlc_hip_scatter_kv_paged_batched_f16": (C.c_int, [_vp, _u32p, _u32p, _sz, _sz, _sz, _sz, _vp,
                                                        C.c_int]),
     "mlc_hip_scatter_kv_paged": (C.c_int, [_vp, _u32p, _sz, _sz, _sz, _sz, _sz, _sz, _vp, _sz]),

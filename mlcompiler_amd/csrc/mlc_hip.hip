@@ -1226,6 +1226,79 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
     return finish(sync);
 }
 
+int mlc_hip_paged_attn_decode_noalloc(const void* q, const void* k_pages, const void* v_pages, void* o,
+                                      const uint32_t* page_tables_flat_device, size_t n_flat,
+                                      const uint32_t* page_table_offsets, const uint32_t* seq_lens,
+                                      const uint32_t* q_positions, size_t batch, size_t num_heads,
+                                      size_t kv_heads, size_t head_dim, size_t page_size_tokens,
+                                      int apply_causal, void* stream) {
+    // Nothing here allocates device or pinned memory: no hipMalloc / hipFree / hipHostMalloc, no
+    // event or stream creation (only the text of an error message, on a refusal, takes host heap).
+    // The kernel's scratch memory (split-K partials, arrival counters) is
+    // the file-scope device array whose address init_once() looked up; the per-request arrays travel
+    // inside the kernel arguments and the page table stays where the caller keeps it.
+    if (!g.inited || !g.available) return fail("decode (no allocation): call mlc_hip_available() once at set-up");
+    if (!settle()) return 0;  // operators held back by earlier encode calls are launched (kernel launches only)
+    if (!q || !k_pages || !v_pages || !o) return fail("decode: null buffer");  // metal_runtime.mm:7742-7750
+    if (batch == 0 || num_heads == 0 || head_dim == 0 || page_size_tokens == 0) return fail("decode: zero dimension");
+    if (kv_heads == 0 || (num_heads % kv_heads) != 0) return fail("decode: heads % kv_heads != 0");
+    if (!page_table_offsets || !seq_lens || !q_positions) return fail("decode: null metadata");
+    if (n_flat && !page_tables_flat_device) return fail("decode: null page table");
+    if (n_flat < page_table_offsets[batch]) return fail("decode: page table shorter than offsets");
+    if (batch > kStreamEmbBatch) return fail("decode (no allocation): more than 256 requests");
+    const size_t G = num_heads / kv_heads;
+    const size_t tile = (head_dim == 64) ? 64 : 32;
+    int hpw = 0, nw = 0;
+    if (!stream_variant(G, head_dim, &hpw, &nw) || (page_size_tokens % tile) != 0)
+        return fail("decode (no allocation): head_dim must be 64 or 128, the GQA ratio 1, 2, 4, 8, 16 or 32, "
+                    "the page size a multiple of 64 (head_dim 64) or 32 (head_dim 128) tokens");
+    if (!aligned16(q) || !aligned16(k_pages) || !aligned16(v_pages) || !aligned16(o) ||
+        (reinterpret_cast<uintptr_t>(page_tables_flat_device) & 3u))
+        return fail("decode (no allocation): buffers must be 16-byte aligned");
+    uint64_t total_tiles = 0;
+    for (size_t r = 0; r < batch; ++r) {
+        const size_t pages = ((size_t)seq_lens[r] + page_size_tokens - 1) / page_size_tokens;
+        if ((size_t)page_table_offsets[r] + pages > n_flat) return fail("decode: page table does not cover seq_len");
+        uint64_t lim = seq_lens[r];
+        if (apply_causal && (uint64_t)q_positions[r] + 1 < lim) lim = (uint64_t)q_positions[r] + 1;  // :2286
+        total_tiles += (lim + tile - 1) / tile;
+    }
+    total_tiles *= kv_heads;
+    if (total_tiles >= 0x7FFFFFFFull) return fail("decode (no allocation): too many KV tiles");
+    {
+        const size_t qo_bytes = batch * num_heads * head_dim * 4;
+        const size_t kq = known_bytes(q), ko = known_bytes(o), kt = known_bytes(page_tables_flat_device);
+        if ((kq && qo_bytes > kq) || (ko && qo_bytes > ko)) return fail("decode: q / o buffer too small");
+        if (kt && n_flat * 4 > kt) return fail("decode: page table buffer too small");
+    }
+    const int nbuf = stream_stages(batch);
+    const size_t dyn_lds = batch <= 64 ? 0 : stream_dynamic_lds_bytes(batch);
+    const unsigned n_wg = stream_grid(G, head_dim, nbuf, dyn_lds);
+    StreamArgs a;
+    stream_fill_common(a, q, k_pages, v_pages, o, batch, num_heads, kv_heads, head_dim, page_size_tokens, apply_causal);
+    a.pt_flat = page_tables_flat_device;
+    {
+        // the page ids are on the device and cannot be checked here: pools this library allocated
+        // are protected by the kernel's clamp of the ids to their size
+        const size_t page_bytes = page_size_tokens * kv_heads * head_dim * 2;
+        const size_t kk = known_bytes(k_pages), kv = known_bytes(v_pages);
+        const size_t pages = std::min(kk ? kk / page_bytes : SIZE_MAX, kv ? kv / page_bytes : SIZE_MAX);
+        if (pages != SIZE_MAX) a.capacity_pages = (uint32_t)std::min<size_t>(pages, 0xFFFFFFFFu);
+    }
+    std::memcpy(a.emb, seq_lens, batch * 4);
+    std::memcpy(a.emb + kStreamEmbBatch, q_positions, batch * 4);
+    std::memcpy(a.emb + 2 * kStreamEmbBatch, page_table_offsets, batch * 4);
+    hipStream_t st = stream ? static_cast<hipStream_t>(stream) : g.stream;
+    if (!launch_stream_variant(head_dim, hpw, nw, nbuf, a, n_wg, dyn_lds, st))
+        return fail("decode: kernel variant not built");
+    HIP_OK(hipGetLastError());
+    g.last_items = (int)std::min<uint64_t>(n_wg, total_tiles);
+    std::snprintf(g.last_kernel, sizeof g.last_kernel, "stream<%zu,%d,%d,%s,%s,%d>", head_dim, hpw, nw,
+                  g.opt_pv_fp16 ? "pv16" : "pv32", batch <= 64 ? "regs" : "lds", nbuf);
+    g.last_launches = 1;
+    return 1;
+}
+
 int mlc_hip_scatter_kv_paged_batched_f16(void* page_storage, const uint32_t* page_ids,
                                          const uint32_t* slots_in_page, size_t page_size_tokens,
                                          size_t n_kv_heads, size_t head_dim, size_t batch,
