@@ -254,6 +254,10 @@ class HipExecutor:
     def lastDecodeKernel(self) -> str:
         return (self._lib.mlc_hip_last_decode_kernel() or b"").decode()
 
+    def tableUploads(self) -> int:
+        """Times so far the decode path copied a page table to the device."""
+        return int(self._lib.mlc_hip_decode_table_uploads())
+
     def fusedKvWriteLaunches(self) -> int:
         """KV writes so far that went out fused with a neighbour (option "fuse_row_ops")."""
         return int(self._lib.mlc_hip_fused_kv_write_launches())

@@ -154,3 +154,21 @@ def test_prefill_baseline_config5_sampled(exe):
             want = oracle(sub)
             rep = po.per_head_report(got[r, i], want[0, 0], 128)
             assert rep["min_cosine"] >= MIN_COSINE and rep["max_abs"] <= MAX_ABS, (r, i, rep)
+
+
+def test_prefill_baseline_config5_every_row_of_one_request(exe):
+    """Configuration 5 at full size, all 256 chunk rows x 32 heads of one request against the
+    oracle (the sampled test above covers two requests at nine rows each)."""
+    w = make_prefill(8, 256, 32, 8, 128, 64, [3840] * 8, seed=55)
+    got = run_gpu(exe, w)
+    r = 3
+    sub = dict(w)
+    sub.update(B=1)
+    sub["q"] = np.ascontiguousarray(w["q"].reshape(8, 256 * 32 * 128)[r])
+    sub["flat"] = w["flat"][w["off"][r]:w["off"][r + 1]]
+    sub["off"] = np.array([0, sub["flat"].size], np.uint32)
+    sub["seq"], sub["q_start"] = w["seq"][r:r + 1], w["q_start"][r:r + 1]
+    want = oracle(sub)
+    rep = po.per_head_report(got[r], want[0], 128)
+    print("[prefill] config 5, request 3, 256 rows:", rep, flush=True)
+    assert rep["min_cosine"] >= MIN_COSINE and rep["max_abs"] <= MAX_ABS, rep
