@@ -432,9 +432,19 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
             const half8_t kh = __builtin_bit_cast(half8_t, kq);
 #pragma unroll
             for (int h = 0; h < HPW; ++h) {
-                float s = qv[h][0] * (float)kh[0];
+#ifdef MLC_QK_DOT2
+                const uint32_t* kw = reinterpret_cast<const uint32_t*>(&kq);
+                float s = 0.f;
 #pragma unroll
-                for (int i = 1; i < 8; ++i) s = fmaf(qv[h][i], (float)kh[i], s);
+                for (int i = 0; i < 4; ++i) {
+                    const half2_t qq = {(_Float16)qv[h][2 * i], (_Float16)qv[h][2 * i + 1]};
+                    s = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, kw[i]), qq, s, false);
+                }
+#else
+                float s = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) s = fmaf(qv[h][i], (float)kh[i], s);  // v_fma_mix_f32 throughout
+#endif
                 part[h][j] = s;
             }
         }
@@ -555,17 +565,24 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         }
     };
 
-    // ---- end of a pair's tiles inside this range: sum over the rows of lanes, then either
-    // the output (the whole pair was ours) or a partial, whose last arriver merges.
-    // seg_first: global index of the first tile this workgroup consumed for the pair.
-    auto finalize = [&](const Cursor& cu, uint32_t seg_first, uint32_t seg_end) {
-        // Bring the rows of lanes (the tokens a lane row owns) onto one reference and sum over
-        // them by reduce-scatter across the lane bits above the chunk index: every step halves the
-        // values a lane keeps (v_permlane32_swap / v_permlane16_swap hand the other half to the
-        // partner, the last step of head_dim 64 goes over lane ^ 8).  Lane (r, c) ends up with
-        // dims c*8 + r*HPK + kk (kk < HPK) of every head, summed over all tokens of the wave.
-        float m_all[HPW], l_all[HPW];
-        float o_un[OPL];
+    // ---- end of a pair's tiles inside this range.  The rows of lanes are summed; a pair that
+    // lay inside the range is written to O at once.  A pair cut by range boundaries becomes a
+    // partial, and nothing about a partial touches memory before the range has ended: a range's
+    // first pair that ends in mid-range is kept in registers (at most one per workgroup: a later
+    // pair that ends inside the range also started inside it), so that the stream never stops for
+    // the round trips of a publication.  At the end of the range the workgroup stores its
+    // partials (one or two), waits for them once, takes the arrival tickets together and merges
+    // where it arrived last.
+    struct PairOut {
+        uint32_t w_lo, n_splits, slot_first, my_slot;
+        float* orow;
+    };
+    // Brings the rows of lanes (the tokens a lane row owns) onto one reference and sums over
+    // them by reduce-scatter across the lane bits above the chunk index: every step halves the
+    // values a lane keeps (v_permlane32_swap / v_permlane16_swap hand the other half to the
+    // partner, the last step of head_dim 64 goes over lane ^ 8).  Lane (r, c) ends up with
+    // dims c*8 + r*HPK + kk (kk < HPK) of every head, summed over all tokens of the wave.
+    auto reduce_rows = [&](float (&o_un)[OPL], float (&m_all)[HPW], float (&l_all)[HPW]) {
 #pragma unroll
         for (int h = 0; h < HPW; ++h) {
             float m = m_ref[h];
@@ -574,7 +591,11 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
             m_all[h] = m;
             const float wgt = fast_exp2(m_ref[h] - m);
             // with CPR == 16 every token's weight sits in two lanes (c and c^8): count it once
-            l_all[h] = wave_sum((CPR == 16 && (c & 8)) ? 0.f : l_sum[h] * wgt);
+            // (one lane's sum for the whole wave: with the product fused into the first addition the
+            // lanes' sums can differ in the last bit, and the partial's l must not depend on the
+            // lane it is read from)
+            l_all[h] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(
+                int, wave_sum((CPR == 16 && (c & 8)) ? 0.f : l_sum[h] * wgt))));
             float v4[4], v2[2];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {  // lane bit 5: keep dims i (lower half) or i + 4 (upper half)
@@ -598,68 +619,60 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
                 o_un[h * 2 + 1] = v2[1];
             }
         }
-        // element (head k / HPK, dim) of output register k of this lane
-        const int dim0 = c * 8 + r_l * HPK;
-
-        const uint32_t head0 = cu.kvh * G + hg * HPW;
-        float* orow = a.o + ((size_t)cu.r * a.num_heads + head0) * D;
-        const uint32_t ps = req_start(cu.r) * Hkv + cu.kvh * cu.tiles;  // pair's first tile
-        const uint32_t pe = ps + cu.tiles;
-        if (seg_first == ps && seg_end == pe) {
+    };
+    // element (head k / HPK, dim) of output register k of this lane
+    const int dim0 = c * 8 + r_l * HPK;
+    // workgroup that holds tile g
+    const uint32_t thr = trem * (tq + 1u);
+    auto wg_of = [&](uint32_t g) {
+        return (uint32_t)__builtin_amdgcn_readfirstlane(g < thr ? g / (tq + 1u) : trem + (g - thr) / tq);
+    };
+    auto out_row = [&](const Cursor& cu) {
+        return a.o + ((size_t)cu.r * a.num_heads + cu.kvh * G + hg * HPW) * D;
+    };
+    // who shares the pair [ps, pe) and where its partials go.  A workgroup's first pair uses
+    // slot 2w, a later (so: its last) pair slot 2w + 1.
+    auto pair_out = [&](const Cursor& cu, uint32_t ps, uint32_t pe) {
+        PairOut po;
+        po.w_lo = wg_of(ps);
+        po.n_splits = wg_of(pe - 1u) - po.w_lo + 1u;
+        po.slot_first = 2u * po.w_lo + (range_start(po.w_lo) == ps ? 0u : 1u);
+        po.my_slot = (ps <= g0) ? 2u * w : 2u * w + 1u;
+        po.orow = out_row(cu);
+        return po;
+    };
+    auto store_direct = [&](float* orow, const float (&o_un)[OPL], const float (&l_all)[HPW]) {
 #pragma unroll
-            for (int k = 0; k < OPL; ++k) {
-                const float l = l_all[k / HPK];
-                const float inv = l > 0.f ? 1.0f / l : 0.f;
-                orow[(k / HPK) * D + dim0 + (k % HPK)] = o_un[k] * inv;
-            }
-            return;
+        for (int k = 0; k < OPL; ++k) {
+            const float l = l_all[k / HPK];
+            const float inv = l > 0.f ? 1.0f / l : 0.f;
+            orow[(k / HPK) * D + dim0 + (k % HPK)] = o_un[k] * inv;
         }
-        // workgroup that holds tile g
-        const uint32_t thr = trem * (tq + 1u);
-        auto wg_of = [&](uint32_t g) {
-            return (uint32_t)__builtin_amdgcn_readfirstlane(g < thr ? g / (tq + 1u) : trem + (g - thr) / tq);
-        };
-        const uint32_t w_lo = wg_of(ps), w_hi = wg_of(pe - 1u);
-        const uint32_t n_splits = w_hi - w_lo + 1u;
-        // A workgroup's first pair uses slot 2w, a later (so: its last) pair slot 2w + 1.
-        const uint32_t g0_lo = range_start(w_lo);
-        const uint32_t slot_first = 2u * w_lo + (g0_lo == ps ? 0u : 1u);
-        const uint32_t my_slot = (ps <= g0) ? 2u * w : 2u * w + 1u;
-        {
-            float* po = a.part_o + ((size_t)my_slot * G + hg * HPW) * D;
-            float* ml = a.part_ml + ((size_t)my_slot * G + hg * HPW) * 2;
+    };
+    auto store_partial = [&](uint32_t my_slot, const float (&o_un)[OPL], const float (&m_all)[HPW],
+                             const float (&l_all)[HPW]) {
+        float* po = a.part_o + ((size_t)my_slot * G + hg * HPW) * D;
+        float* ml = a.part_ml + ((size_t)my_slot * G + hg * HPW) * 2;
 #pragma unroll
-            for (int k = 0; k < OPL; ++k) st_dev(po + k * 64 + lane, o_un[k]);
-            if (lane < HPW) {
-                float mh = m_all[0], lh = l_all[0];
+        for (int k = 0; k < OPL; ++k) st_dev(po + k * 64 + lane, o_un[k]);
+        if (lane < HPW) {
+            float mh = m_all[0], lh = l_all[0];
 #pragma unroll
-                for (int hh = 1; hh < HPW; ++hh) {
-                    mh = (lane == hh) ? m_all[hh] : mh;
-                    lh = (lane == hh) ? l_all[hh] : lh;
-                }
-                st_dev(ml + lane * 2, mh);
-                st_dev(ml + lane * 2 + 1, lh);
+            for (int hh = 1; hh < HPW; ++hh) {
+                mh = (lane == hh) ? m_all[hh] : mh;
+                lh = (lane == hh) ? l_all[hh] : lh;
             }
+            st_dev(ml + lane * 2, mh);
+            st_dev(ml + lane * 2 + 1, lh);
         }
-        // The partial must have reached memory before the arrival counter is bumped: the
-        // write-through stores are complete once this wave's memory counter is zero.
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        sd_wait_vmcnt<0>();
-        MLC_PROBE(26);
-        uint32_t ticket = 0;
-        uint32_t* counter = &a.counters[(size_t)w_lo * NW + hg];
-        if (lane == 0) ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        ticket = __shfl(ticket, 0);
-        MLC_PROBE(27);
-        if (ticket != n_splits - 1u) return;
-        MLC_PROBE(28);
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-        if (lane == 0)  // ready for the next launch
-            __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-
-        // Merge, 64 partials at a time: lane s holds the (m, l) of partial s for every head; the
-        // partial outputs are loaded eight at a time, all issued before any is consumed.
-        auto slot_of = [&](uint32_t i) { return i == 0 ? slot_first : 2u * (w_lo + i); };
+    };
+    // Merge of a pair's partials by the wave that arrived last, in the order of their slots (so
+    // the result does not depend on who arrived last).  64 partials at a time: lane s holds the
+    // (m, l) of partial s for every head; the partial outputs are loaded eight at a time, the
+    // first eight (nearly always: all) together with the (m, l) pairs, before anything is
+    // consumed: one memory round trip.
+    auto merge = [&](const PairOut& po) {
+        auto slot_of = [&](uint32_t i) { return i == 0 ? po.slot_first : 2u * (po.w_lo + i); };
         float acc_o[OPL], m_run[HPW], l_run[HPW];
 #pragma unroll
         for (int k = 0; k < OPL; ++k) acc_o[k] = 0.f;
@@ -668,40 +681,49 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
             m_run[h] = kNegBig;
             l_run[h] = 0.f;
         }
-        for (uint32_t s0 = 0; s0 < n_splits; s0 += 64) {
-            const uint32_t cnt = min(64u, n_splits - s0);
-            float wgt[HPW];
-            {
-                const size_t my = slot_of(s0 + (uint32_t)lane);
-                const float* ml = a.part_ml + (my * G + hg * HPW) * 2;
-#pragma unroll
-                for (int h = 0; h < HPW; ++h) {
-                    float ms = kNegBig, ls = 0.f;
-                    if ((uint32_t)lane < cnt) {
-                        ms = ld_dev(ml + h * 2);
-                        ls = ld_dev(ml + h * 2 + 1);
-                    }
-                    const float m_new = max_nn(m_run[h], wave_max(ms));
-                    const float keep = fast_exp2(m_run[h] - m_new);
-                    wgt[h] = fast_exp2(ms - m_new);  // lanes >= cnt: exp2(-1e30 - m) = 0
-                    l_run[h] = l_run[h] * keep + wave_sum(wgt[h] * ls);
-                    m_run[h] = m_new;
-#pragma unroll
-                    for (int kk = 0; kk < HPK; ++kk) acc_o[h * HPK + kk] *= keep;
-                }
-            }
-            constexpr int UNR = 8;
-            for (uint32_t u0 = 0; u0 < cnt; u0 += UNR) {
-                float pvv[UNR][OPL];
+        constexpr int UNR = 8;
+        for (uint32_t s0 = 0; s0 < po.n_splits; s0 += 64) {
+            const uint32_t cnt = min(64u, po.n_splits - s0);
+            float pvv[UNR][OPL];
+            auto load_outputs = [&](uint32_t u0) {
 #pragma unroll
                 for (int u = 0; u < UNR; ++u) {
-                    const float* po = a.part_o + ((size_t)slot_of(s0 + u0 + u) * G + hg * HPW) * D;
+                    const float* src = a.part_o + ((size_t)slot_of(s0 + u0 + u) * G + hg * HPW) * D;
 #pragma unroll
                     for (int k = 0; k < OPL; ++k) {
                         pvv[u][k] = 0.f;
-                        if (u0 + u < cnt) pvv[u][k] = ld_dev(po + k * 64 + lane);
+                        if (u0 + u < cnt) pvv[u][k] = ld_dev(src + k * 64 + lane);
                     }
                 }
+            };
+            load_outputs(0);
+            float ms[HPW], ls[HPW];
+            {
+                const float* ml = a.part_ml + ((size_t)slot_of(s0 + (uint32_t)lane) * G + hg * HPW) * 2;
+#pragma unroll
+                for (int h = 0; h < HPW; ++h) {
+                    ms[h] = kNegBig;
+                    ls[h] = 0.f;
+                    if ((uint32_t)lane < cnt) {
+                        ms[h] = ld_dev(ml + h * 2);
+                        ls[h] = ld_dev(ml + h * 2 + 1);
+                    }
+                }
+            }
+            float wgt[HPW];
+#pragma unroll
+            for (int h = 0; h < HPW; ++h) {
+                const float m_new = max_nn(m_run[h], wave_max(ms[h]));
+                const float keep = fast_exp2(m_run[h] - m_new);
+                wgt[h] = fast_exp2(ms[h] - m_new);  // lanes >= cnt: exp2(-1e30 - m) = 0
+                l_run[h] = l_run[h] * keep + __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(
+                                                 int, wave_sum(wgt[h] * ls[h]))));
+                m_run[h] = m_new;
+#pragma unroll
+                for (int kk = 0; kk < HPK; ++kk) acc_o[h * HPK + kk] *= keep;
+            }
+            for (uint32_t u0 = 0; u0 < cnt; u0 += UNR) {
+                if (u0) load_outputs(u0);
 #pragma unroll
                 for (int u = 0; u < UNR; ++u) {
                     if (u0 + u < cnt) {
@@ -711,12 +733,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
                 }
             }
         }
-#pragma unroll
-        for (int k = 0; k < OPL; ++k) {
-            const float l = l_run[k / HPK];
-            const float inv = l > 0.f ? 1.0f / l : 0.f;
-            orow[(k / HPK) * D + dim0 + (k % HPK)] = acc_o[k] * inv;
-        }
+        store_direct(po.orow, acc_o, l_run);
     };
 
     // ---- the stream: the first NBUF tiles of the range go out together, then one tile per step
@@ -724,6 +741,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     load_q(cc);
     uint32_t issued = 1;
     issue_tile(ci, 0);
+#ifdef MLC_PROLOGUE_FULL
 #pragma unroll
     for (int i = 1; i < NBUF; ++i) {
         if (issued < n) {
@@ -733,9 +751,13 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
             ++issued;
         }
     }
+#endif
     uint32_t seg_first = g0;  // first tile consumed for the pair under cc
     bool drain = false;       // stores are in flight: they do not complete in order with loads
     uint32_t slot = 0;        // stage of tile k
+    bool kept = false;        // the range's first pair waits in registers for the end of the range
+    PairOut kept_po{};
+    float kept_o[OPL], kept_m[HPW], kept_l[HPW];
     for (uint32_t k = 0; k < n; ++k) {
         // this wave's loads of tile k have landed ...
         if (k < 6) MLC_PROBE(8 + 3 * k);
@@ -744,25 +766,94 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         sd_barrier();   // ... and everyone's; everyone has left tile k-1, whose stage is free
         if (k < 6) MLC_PROBE(9 + 3 * k);
         if (k == 0) MLC_PROBE(3);
+#ifndef MLC_PROLOGUE_FULL
+        // one tile went out up front; from the first step on the stream runs NBUF - 1 tiles ahead
+        // (all stages requested at once would make every workgroup wait for the whole burst)
+        while (issued < n && issued < k + (uint32_t)NBUF) {
+            advance(ci);
+            if (!pages_ready(ci)) fetch_pages(ci);
+            issue_tile(ci, issued % (uint32_t)NBUF);
+            ++issued;
+        }
+#else
         if (k >= 1 && issued < n) {
             advance(ci);
             if (!pages_ready(ci)) fetch_pages(ci);  // another request, or 64 tiles on
             issue_tile(ci, slot == 0 ? (uint32_t)(NBUF - 1) : slot - 1u);
             ++issued;
         }
+#endif
 #ifndef MLC_NO_COMPUTE
         consume_tile(slot, cc.t, cc.lim);
 #endif
         const bool pair_done = cc.t + 1u == cc.tiles;
+        const bool range_done = k + 1 == n;
         if (k < 6) MLC_PROBE(10 + 3 * k);
-        if (k + 1 == n) MLC_PROBE(4);
-        if (pair_done || k + 1 == n) {
-            finalize(cc, seg_first, g0 + k + 1u);
+        if (range_done) MLC_PROBE(4);
+        if (pair_done || range_done) {
+            float o_un[OPL], m_all[HPW], l_all[HPW];
+            reduce_rows(o_un, m_all, l_all);
+            const uint32_t ps = req_start(cc.r) * Hkv + cc.kvh * cc.tiles;  // pair's first tile
+            const uint32_t pe = ps + cc.tiles;
+            const bool whole = seg_first == ps && g0 + k + 1u == pe;
+            bool cur = false;  // this pair is a partial to publish now (only at the end of the range)
+            PairOut cur_po{};
+            if (whole) {
+                store_direct(out_row(cc), o_un, l_all);
+                drain = true;
+            } else if (!range_done) {
+                kept = true;
+                kept_po = pair_out(cc, ps, pe);
+#pragma unroll
+                for (int i = 0; i < OPL; ++i) kept_o[i] = o_un[i];
+#pragma unroll
+                for (int h = 0; h < HPW; ++h) {
+                    kept_m[h] = m_all[h];
+                    kept_l[h] = l_all[h];
+                }
+            } else {
+                cur = true;
+                cur_po = pair_out(cc, ps, pe);
+            }
+#ifdef MLC_NO_TAIL
+            if (false) {
+#else
+            if (range_done && (kept || cur)) {
+#endif
+                if (kept) store_partial(kept_po.my_slot, kept_o, kept_m, kept_l);
+                if (cur) store_partial(cur_po.my_slot, o_un, m_all, l_all);
+                // The partials must have reached memory before an arrival counter is bumped: the
+                // write-through stores are complete once this wave's memory counter is zero.
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                sd_wait_vmcnt<0>();
+                MLC_PROBE(26);
+                uint32_t t_kept = 0, t_cur = 0;
+                uint32_t* c_kept = &a.counters[(size_t)kept_po.w_lo * NW + hg];
+                uint32_t* c_cur = &a.counters[(size_t)cur_po.w_lo * NW + hg];
+                if (lane == 0) {  // both tickets travel together
+                    if (kept) t_kept = __hip_atomic_fetch_add(c_kept, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (cur) t_cur = __hip_atomic_fetch_add(c_cur, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                t_kept = __shfl(t_kept, 0);
+                t_cur = __shfl(t_cur, 0);
+                MLC_PROBE(27);
+                const bool last_kept = kept && t_kept == kept_po.n_splits - 1u;
+                const bool last_cur = cur && t_cur == cur_po.n_splits - 1u;
+                if (last_kept || last_cur) {
+                    MLC_PROBE(28);
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                    if (lane == 0) {  // ready for the next launch
+                        if (last_kept) __hip_atomic_store(c_kept, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if (last_cur) __hip_atomic_store(c_cur, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                    if (last_kept) merge(kept_po);
+                    if (last_cur) merge(cur_po);
+                }
+            }
             reset_state();
             seg_first = g0 + k + 1u;
-            drain = true;
         }
-        if (k + 1 < n) {
+        if (!range_done) {
             advance(cc);
             if (pair_done) load_q(cc);
         }
