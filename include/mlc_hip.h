@@ -271,6 +271,44 @@ int mlc_hip_paged_attn_decode_noalloc(const void* q, const void* k_pages, const 
                                       size_t head_dim, size_t page_size_tokens, int apply_causal,
                                       void* stream);
 
+/* ---- a whole pass replayed from a HIP graph (no reference counterpart; the closest thing in
+ * the reference is its single command buffer per forward pass, metal_runtime.mm:6000-6064).
+ * The launches of a decode step are the same from step to step: what changes is the content of
+ * the page tables, the per-request lengths and positions, the (page, slot) of the new K / V rows
+ * and the caller's own buffers.  A captured pass keeps the launches and reads all of that from
+ * device memory at fixed addresses, so that a step costs one graph launch instead of the encode
+ * calls:
+ *
+ *   mlc_hip_begin(); <encode the step once, uncaptured>; mlc_hip_flush();     // everything resident
+ *   mlc_hip_begin(); mlc_hip_capture_begin(); <the same encode calls>; h = mlc_hip_capture_end();
+ *   per step: upload the step's inputs into the same buffers (mlc_hip_upload);
+ *             mlc_hip_replay_update(h, <the step's tables>); mlc_hip_replay(h); mlc_hip_flush();
+ *
+ * While a pass is being captured the encode calls record their launches instead of running them;
+ * a call that would have to allocate, copy metadata or wait fails (and the capture with it): run
+ * the pass once uncaptured first, which puts weights, norm vectors and tables on the device.  The
+ * decode attention of a captured pass must be served by the tile-balanced kernel (head_dim 64 or
+ * 128, page size a multiple of its tile, 16-byte aligned buffers).  mlc_hip_capture_end returns a
+ * handle > 0, or 0 (then nothing was kept; encode the pass uncaptured).
+ *
+ * mlc_hip_replay_update copies the step's tables over the device copies the captured launches
+ * read (same addresses, ordered on the library's stream) and checks what the capture took for
+ * granted: the same batch size; tables that cover their seq_lens; if the attention launch of the
+ * captured pass does the step's KV write, that (page_ids, slots_in_page) are every request's newest
+ * position on pages no two requests share.  It returns 0 when the step cannot be replayed (encode
+ * it uncaptured; capture again if it said the copies had to move).  page_ids / slots_in_page may
+ * be NULL for a pass without KV write.  The replay reads whatever the tables' device copy holds
+ * when it runs: call mlc_hip_replay_update right before mlc_hip_replay. */
+int    mlc_hip_capture_begin(void);
+int    mlc_hip_capture_end(void);
+size_t mlc_hip_captured_launches(int handle);
+int    mlc_hip_replay_update(int handle, const uint32_t* page_tables_flat, size_t n_page_tables_flat,
+                             const uint32_t* page_table_offsets, const uint32_t* seq_lens,
+                             const uint32_t* q_positions, const uint32_t* page_ids,
+                             const uint32_t* slots_in_page, size_t batch);
+int    mlc_hip_replay(int handle);
+void   mlc_hip_capture_release(int handle);
+
 /* ---- measurement helpers (no reference counterpart) ------------------------
  * The library's stream as a hipStream_t, for callers that need to order their
  * own work or events with it. */

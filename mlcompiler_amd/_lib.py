@@ -47,6 +47,12 @@ SIGNATURES = {
     "mlc_hip_matmul_q6_k_batched": (C.c_int, [C.c_char_p, _vp, _sz, _vp, _sz, _sz, _sz, _sz, _vp, C.c_int]),
     "mlc_hip_paged_attn_prefill": (C.c_int, [_vp, _vp, _vp, _vp, _u32p, _sz, _u32p, _u32p, _u32p,
                                              _sz, _sz, _sz, _sz, _sz, _sz, C.c_int]),
+    "mlc_hip_capture_begin": (C.c_int, []),
+    "mlc_hip_capture_end": (C.c_int, []),
+    "mlc_hip_captured_launches": (_sz, [C.c_int]),
+    "mlc_hip_replay_update": (C.c_int, [C.c_int, _u32p, _sz, _u32p, _u32p, _u32p, _u32p, _u32p, _sz]),
+    "mlc_hip_replay": (C.c_int, [C.c_int]),
+    "mlc_hip_capture_release": (None, [C.c_int]),
     "mlc_hip_stream": (_vp, []),
     "mlc_hip_timer_start": (C.c_int, []),
     "mlc_hip_timer_stop": (C.c_float, []),

@@ -263,12 +263,11 @@ int mlc_bench_layer_loop(const MlcBenchLayer* L, void* const* k_pools, void* con
 }
 
 // The same loop with one pass over the n_layers layers (n_layers even, so that a pass ends in
-// the buffer the next one starts from) captured into a HIP graph and replayed `replays` times:
-// measures what replaying prebuilt launches saves over encoding them call by call.  The pass
-// is run once uncaptured first, so that every weight, norm vector, page table and scratch
-// buffer is already on the device and the captured pass holds kernel launches only.
-// event_ms receives the time of all replays.  Returns 1 on success, 0 on failure, and -1 when
-// the captured pass held something other than kernels (then nothing is replayed).
+// the buffer the next one starts from) captured into a HIP graph through the library's capture
+// calls and replayed `replays` times: measures what replaying prebuilt launches saves over
+// encoding them call by call.  The pass is run once uncaptured first, so that every weight, norm
+// vector, page table and scratch buffer is already on the device (a capture holds kernel launches
+// only).  event_ms receives the time of all replays.  Returns 1 on success, 0 on failure.
 int mlc_bench_layer_loop_graph(const MlcBenchLayer* L, void* const* k_pools, void* const* v_pools,
                                size_t n_layers, size_t replays, float* event_ms, size_t* n_nodes) {
     if (n_layers == 0 || n_layers % 2 != 0) return 0;
@@ -277,49 +276,20 @@ int mlc_bench_layer_loop_graph(const MlcBenchLayer* L, void* const* k_pools, voi
     for (size_t i = 0; i < n_layers; ++i)
         if (!encode_layer_step(L, names, k_pools, v_pools, n_layers, i)) return 0;
     if (!mlc_hip_flush() || !mlc_hip_begin()) return 0;
-    hipStream_t stream = static_cast<hipStream_t>(mlc_hip_stream());
-    hipGraph_t graph = nullptr;
-    hipGraphExec_t exec = nullptr;
-    if (hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal) != hipSuccess) return 0;
+    if (!mlc_hip_capture_begin()) return 0;
     int ok = 1;
     for (size_t i = 0; ok && i < n_layers; ++i) ok = encode_layer_step(L, names, k_pools, v_pools, n_layers, i);
-    (void)mlc_hip_stream();  // launches what the library still holds back
-    if (hipStreamEndCapture(stream, &graph) != hipSuccess || !ok || !graph) {
-        (void)hipGetLastError();
-        if (graph) (void)hipGraphDestroy(graph);
-        return 0;
-    }
-    size_t count = 0;
-    int rc = 1;
-    std::vector<hipGraphNode_t> nodes;
-    if (hipGraphGetNodes(graph, nullptr, &count) != hipSuccess) rc = 0;
-    if (rc) {
-        nodes.resize(count);
-        if (count && hipGraphGetNodes(graph, nodes.data(), &count) != hipSuccess) rc = 0;
-    }
-    for (size_t i = 0; rc == 1 && i < count; ++i) {
-        hipGraphNodeType type;
-        if (hipGraphNodeGetType(nodes[i], &type) != hipSuccess) rc = 0;
-        else if (type != hipGraphNodeTypeKernel) rc = -1;
-    }
-    if (n_nodes) *n_nodes = count;
-    hipEvent_t e0 = nullptr, e1 = nullptr;
-    if (rc == 1 && hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0) != hipSuccess) rc = 0;
-    if (rc == 1 && (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)) rc = 0;
-    if (rc == 1) {
-        rc = hipGraphLaunch(exec, stream) == hipSuccess && hipStreamSynchronize(stream) == hipSuccess;
-        rc = rc && hipEventRecord(e0, stream) == hipSuccess;
-        for (size_t i = 0; rc == 1 && i < replays; ++i) rc = hipGraphLaunch(exec, stream) == hipSuccess;
-        rc = rc && hipEventRecord(e1, stream) == hipSuccess && hipEventSynchronize(e1) == hipSuccess;
-        float ms = 0.f;
-        rc = rc && hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
-        if (event_ms) *event_ms = ms;
-    }
-    if (e0) (void)hipEventDestroy(e0);
-    if (e1) (void)hipEventDestroy(e1);
-    if (exec) (void)hipGraphExecDestroy(exec);
-    (void)hipGraphDestroy(graph);
-    if (!mlc_hip_flush()) return 0;
+    const int handle = mlc_hip_capture_end();
+    if (!ok || handle <= 0) return 0;
+    if (n_nodes) *n_nodes = mlc_hip_captured_launches(handle);
+    int rc = mlc_hip_replay(handle) && mlc_hip_flush() && mlc_hip_begin();   // one replay to warm up
+    rc = rc && mlc_hip_timer_start();
+    for (size_t i = 0; rc && i < replays; ++i) rc = mlc_hip_replay(handle);
+    const float ms = rc ? mlc_hip_timer_stop() : -1.f;
+    if (ms < 0.f) rc = 0;
+    if (event_ms) *event_ms = ms;
+    if (!mlc_hip_flush()) rc = 0;
+    mlc_hip_capture_release(handle);
     return rc;
 }
 

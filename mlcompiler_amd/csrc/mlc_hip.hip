@@ -45,11 +45,20 @@ namespace {
 using namespace mlc_hip;
 
 thread_local std::string g_err;
+bool g_capture_failed = false;   // a call failed while a pass was being captured
+bool g_capturing = false;        // between mlc_hip_capture_begin and mlc_hip_capture_end
 
 int fail(const std::string& msg) {
     g_err = msg;
+    if (g_capturing) g_capture_failed = true;
     return 0;
 }
+
+// For calls that allocate, copy or wait: none of that can be part of a captured pass.
+#define NOT_WHILE_CAPTURING(what)                                                                   \
+    do {                                                                                            \
+        if (g_capturing) return fail(what ": not possible while a pass is being captured");         \
+    } while (0)
 
 #define HIP_OK(expr)                                                                  \
     do {                                                                              \
@@ -81,30 +90,26 @@ constexpr size_t kScratchCounterBytes = (size_t)kStreamMaxWgs * 4 * sizeof(uint3
 constexpr size_t kScratchBytes = kScratchPartOBytes + kScratchPartMlBytes + kScratchCounterBytes;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
-// Device copy of the flat page table (and, for batches whose per-request arrays do not fit
-// the kernel arguments, of those arrays) as the tile-balanced decode kernel reads it; uploaded
-// only when the content changes.  A ring of four slots: slot i is rewritten only after the
-// upload into slot i + 1 has completed, which is later in the stream than every launch that
-// read slot i.
+// Device copy of the flat page table (and, where the per-request arrays do not travel inside the
+// kernel arguments, of those arrays) as the tile-balanced decode kernel reads it; uploaded only
+// when the content changes.  One grow-only device buffer: its address stays the same from call to
+// call (a captured pass keeps reading it), and a new content is copied over the old one in
+// stream order, behind every launch that read the old one, from a slot of the pinned ring.
 struct StreamTables {
-    struct Slot {
-        void* host = nullptr;
-        void* dev = nullptr;
-        size_t cap = 0;
-        hipEvent_t uploaded = nullptr;
-        bool has_event = false;
-    } slots[4];
-    int cur = -1;
+    void* dev = nullptr;
+    size_t cap = 0;
+    bool filled = false;          // dev holds `flat` (version `uploaded`) and `meta`
     std::vector<uint32_t> flat;   // the caller's flat table as last seen
     uint64_t version = 0;         // counts the changes of `flat`
-    uint64_t uploaded = ~0ull;    // version of `flat` that slots[cur] holds
+    uint64_t uploaded = ~0ull;    // version of `flat` that dev holds
     std::vector<uint32_t> meta;   // seq_lens | q_positions | offsets when they are uploaded too
-    size_t meta_off = 0;          // byte offset of the arrays in the slot
+    size_t meta_off = 0;          // byte offset of the arrays in dev
     uint32_t max_page = 0;        // largest page id in flat
     // does some page id occur in two requests' tables (then a row written for one request may be
     // read for another)?  -1: not computed for this content
     int shared_pages = -1;
     std::vector<uint32_t> off;    // page_table_offsets the shared_pages answer was computed for
+    std::vector<uint32_t> last_meta;  // seq_lens | q_positions | offsets of the last decode call (host copy)
 };
 
 struct DecodePlan {
@@ -231,6 +236,25 @@ struct Ctx {
     long opt_stream_stages = 0;     // tile-balanced kernel: LDS stages per workgroup (0 = automatic)
     long opt_grid_wgs = 0;          // tile-balanced kernel: exact grid size (0 = from workgroups per CU)
     long table_uploads = 0;         // page-table uploads of the tile-balanced path (for tests)
+    // A captured pass: the kernel launches of the encode calls between mlc_hip_capture_begin and
+    // mlc_hip_capture_end as an executable HIP graph, and what the launches read that changes from
+    // decode step to decode step (device copies at fixed addresses, refreshed in place).
+    struct Captured {
+        hipGraph_t graph = nullptr;
+        hipGraphExec_t exec = nullptr;
+        size_t n_nodes = 0;
+        bool used_tables = false;            // a decode launch reads the device page table and arrays
+        const void* tables_flat = nullptr;
+        const void* tables_meta = nullptr;
+        size_t B = 0, H = 0, Hkv = 0, D = 0, P = 0;
+        int causal = 0;
+        bool carried_kv = false;             // ... and does the step's KV write
+        const void* ids_dev = nullptr;       // device copy of the KV write's page ids and slots
+        size_t ids_batch = 0;
+    };
+    std::map<int, Captured> captures;
+    int next_capture = 1;
+    Captured cap;                            // the pass being captured
 };
 
 Ctx g;
@@ -265,6 +289,9 @@ bool init_once() {
 }
 
 int slot_reserve(MetaSlot& s, size_t bytes) {
+    // (every copy of metadata to the device comes through here)
+    NOT_WHILE_CAPTURING("copying metadata to the device (run the pass once uncaptured first; the planned and "
+                        "generic decode kernels, one-request scatter / gather and prefill copy on every call)");
     if (s.pending) {
         HIP_OK(hipEventSynchronize(s.done));
         s.pending = false;
@@ -302,7 +329,7 @@ size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 const void* resident_blob(int kind, const void* key, const void* blob, size_t bytes) {
     // A caller that never repeats itself: start over -- but only while no held-back operator
     // refers to one of the copies (their launches come later).
-    if (g.resident.size() > 1024 && !g.rows.active && !g.kv.active && !g.gemm.active) {
+    if (g.resident.size() > 1024 && !g.rows.active && !g.kv.active && !g.gemm.active && !g_capturing) {
         if (hipStreamSynchronize(g.stream) != hipSuccess) { fail("resident: synchronize failed"); return nullptr; }
         for (auto& kv : g.resident)
             if (kv.second.dev) (void)hipFree(kv.second.dev);
@@ -311,6 +338,7 @@ const void* resident_blob(int kind, const void* key, const void* blob, size_t by
     Ctx::Resident& r = g.resident[std::make_tuple(kind, key, bytes)];
     if (r.dev && r.content.size() == bytes && std::memcmp(r.content.data(), blob, bytes) == 0) return r.dev;
     if (bytes > r.cap) {
+        if (g_capturing) { fail("capture: a small host array is not on the device yet (run the pass once uncaptured first)"); return nullptr; }
         if (r.dev && hipFree(r.dev) != hipSuccess) { fail("resident: hipFree failed"); return nullptr; }
         r.dev = nullptr;
         r.cap = 0;
@@ -473,6 +501,7 @@ void rows_begin(const void* src, size_t batch, size_t len) {
 int finish(int sync) {
     HIP_OK(hipGetLastError());
     if (sync) {
+        NOT_WHILE_CAPTURING("a call with sync = 1");
         if (!settle()) return 0;
         HIP_OK(hipStreamSynchronize(g.stream));
     }
@@ -486,7 +515,12 @@ const void* resident_ids(const uint32_t* page_ids, const uint32_t* slots, size_t
     blob.assign(ids_bytes * 2, 0);
     std::memcpy(blob.data(), page_ids, batch * 4);
     std::memcpy(blob.data() + ids_bytes, slots, batch * 4);
-    return resident_blob(1, nullptr, blob.data(), blob.size());
+    const void* dev = resident_blob(1, nullptr, blob.data(), blob.size());
+    if (dev && g_capturing) {
+        g.cap.ids_dev = dev;
+        g.cap.ids_batch = batch;
+    }
+    return dev;
 }
 
 // ---------------------------------------------------------------- decode plan
@@ -665,6 +699,7 @@ int ensure_partials(size_t n_part, size_t G, size_t D, size_t nw) {
     const size_t need_ml = n_part * G * 2;
     const size_t need_c = n_part * nw;
     if (need_o > g.part_o_cap || need_ml > g.part_ml_cap || need_c > g.counters_cap) {
+        NOT_WHILE_CAPTURING("growing the split-K partial buffers");
         HIP_OK(hipStreamSynchronize(g.stream));
         if (g.part_o) HIP_OK(hipFree(g.part_o));
         if (g.part_ml) HIP_OK(hipFree(g.part_ml));
@@ -766,51 +801,53 @@ void tables_refresh(const uint32_t* flat, size_t n_flat, const uint32_t* off, si
 
 // Makes the device copy of the flat table (and of the per-request arrays when `meta3` is
 // given: seq_lens | q_positions | offsets, B each) current.  Returns the device pointer of the
-// table in *d_flat and of the arrays in *d_meta.
+// table in *d_flat and of the arrays in *d_meta.  The arrays sit behind room for twice the
+// table's entries (at least 16 Ki), so that a table that grows by a page now and then keeps both
+// addresses.
 int tables_upload(const uint32_t* meta3, size_t B, const uint32_t** d_flat, const uint32_t** d_meta) {
     StreamTables& t = g.tables;
     const size_t n_flat = t.flat.size();
-    const size_t flat_bytes = align_up(std::max<size_t>(n_flat, 1) * 4, 16);
     const size_t meta_bytes = meta3 ? 3 * B * 4 : 0;
-    // (the table may have changed any number of calls ago: calls that take another kernel
-    // refresh what is remembered but upload nothing)
-    bool upload = t.uploaded != t.version || t.cur < 0;
+    size_t flat_room = t.meta_off;
+    if (n_flat * 4 > flat_room) flat_room = align_up(std::max<size_t>(2 * n_flat, 16384) * 4, 256);
+    const size_t total = flat_room + std::max<size_t>(meta_bytes, 3 * 4096 * 4);
+    bool upload = t.uploaded != t.version || !t.filled || flat_room != t.meta_off;
     if (meta3) {
         if (t.meta.size() != 3 * B || std::memcmp(t.meta.data(), meta3, meta_bytes) != 0) upload = true;
     }
     if (upload) {
-        const int nxt = (t.cur + 1) % 4;
-        StreamTables::Slot& after = t.slots[(nxt + 1) % 4];
-        if (after.has_event) HIP_OK(hipEventSynchronize(after.uploaded));  // nobody reads slot nxt any more
-        StreamTables::Slot& s = t.slots[nxt];
-        const size_t total = flat_bytes + meta_bytes;
-        if (total > s.cap) {
-            const size_t cap = std::max<size_t>(16384, total * 2);
-            if (s.host) HIP_OK(hipHostFree(s.host));
-            if (s.dev) HIP_OK(hipFree(s.dev));
-            s.host = s.dev = nullptr;
-            s.cap = 0;
-            HIP_OK(hipHostMalloc(&s.host, cap, hipHostMallocDefault));
-            HIP_OK(hipMalloc(&s.dev, cap));
-            s.cap = cap;
+        if (total > t.cap) {
+            HIP_OK(hipStreamSynchronize(g.stream));
+            if (t.dev) HIP_OK(hipFree(t.dev));
+            t.dev = nullptr;
+            t.cap = 0;
+            HIP_OK(hipMalloc(&t.dev, total));
+            t.cap = total;
         }
-        if (!s.uploaded) HIP_OK(hipEventCreateWithFlags(&s.uploaded, hipEventDisableTiming));
-        if (n_flat) std::memcpy(s.host, t.flat.data(), n_flat * 4);
+        MetaSlot& s = g.ring[g.ring_next];
+        g.ring_next = (g.ring_next + 1) % 8;
+        const size_t bytes = flat_room + meta_bytes;
+        if (!slot_reserve(s, bytes)) return 0;
+        char* h = static_cast<char*>(s.host);
+        if (n_flat) std::memcpy(h, t.flat.data(), n_flat * 4);
         if (meta3) {
-            std::memcpy(static_cast<char*>(s.host) + flat_bytes, meta3, meta_bytes);
+            std::memcpy(h + flat_room, meta3, meta_bytes);
             t.meta.assign(meta3, meta3 + 3 * B);
+            // table and arrays in two copies: what lies between them is not sent
+            if (n_flat) HIP_OK(hipMemcpyAsync(t.dev, h, n_flat * 4, hipMemcpyHostToDevice, g.stream));
+            HIP_OK(hipMemcpyAsync(static_cast<char*>(t.dev) + flat_room, h + flat_room, meta_bytes,
+                                  hipMemcpyHostToDevice, g.stream));
         } else {
             t.meta.clear();
+            if (n_flat) HIP_OK(hipMemcpyAsync(t.dev, h, n_flat * 4, hipMemcpyHostToDevice, g.stream));
         }
-        HIP_OK(hipMemcpyAsync(s.dev, s.host, total, hipMemcpyHostToDevice, g.stream));
-        HIP_OK(hipEventRecord(s.uploaded, g.stream));
-        s.has_event = true;
-        t.cur = nxt;
+        if (!slot_mark(s)) return 0;
+        t.filled = true;
         t.uploaded = t.version;
-        t.meta_off = flat_bytes;
+        t.meta_off = flat_room;
         ++g.table_uploads;
     }
-    const char* dev = static_cast<const char*>(t.slots[t.cur].dev);
+    const char* dev = static_cast<const char*>(t.dev);
     *d_flat = reinterpret_cast<const uint32_t*>(dev);
     *d_meta = meta3 ? reinterpret_cast<const uint32_t*>(dev + t.meta_off) : nullptr;
     return 1;
@@ -906,6 +943,7 @@ const char* mlc_hip_last_error(void) { return g_err.c_str(); }
 
 void* mlc_hip_alloc(size_t bytes) {
     if (!init_once()) return nullptr;
+    if (g_capturing) { fail("alloc: not possible while a pass is being captured"); return nullptr; }
     void* p = nullptr;
     if (hipMalloc(&p, bytes ? bytes : 1) != hipSuccess) {
         g_err = "hipMalloc failed";
@@ -918,6 +956,7 @@ void* mlc_hip_alloc(size_t bytes) {
 
 void mlc_hip_free(void* buffer) {
     if (!buffer || !init_once()) return;
+    if (g_capturing) { fail("free: not possible while a pass is being captured"); return; }
     (void)settle();
     (void)hipStreamSynchronize(g.stream);
     g.allocs.erase(buffer);
@@ -930,6 +969,7 @@ void* cached_buffer(const char* name, size_t bytes) {
     if (!init_once() || !name) return nullptr;
     auto it = g.cached.find(name);
     if (it != g.cached.end() && it->second.second >= bytes) return it->second.first;
+    if (g_capturing) { fail("cached buffer: allocation is not possible while a pass is being captured"); return nullptr; }
     if (it != g.cached.end()) {  // grow-only reallocation, metal_runtime.mm:8222-8241
         (void)hipStreamSynchronize(g.stream);
         g.allocs.erase(it->second.first);
@@ -955,6 +995,7 @@ void* mlc_hip_cached(const char* name, size_t bytes) {
 
 int mlc_hip_upload(void* buffer, const void* src, size_t bytes, size_t dst_offset) {
     if (!init_once()) return fail("GPU unavailable");
+    NOT_WHILE_CAPTURING("upload");
     if (!settle()) return 0;
     if (!buffer || (!src && bytes)) return fail("upload: null pointer");
     if (!bytes) return 1;
@@ -968,6 +1009,7 @@ int mlc_hip_upload(void* buffer, const void* src, size_t bytes, size_t dst_offse
 
 int mlc_hip_download(const void* buffer, void* dst, size_t bytes, size_t src_offset) {
     if (!init_once()) return fail("GPU unavailable");
+    NOT_WHILE_CAPTURING("download");
     if (!settle()) return 0;
     if (!buffer || (!dst && bytes)) return fail("download: null pointer");
     if (!bytes) return 1;
@@ -981,6 +1023,7 @@ int mlc_hip_download(const void* buffer, void* dst, size_t bytes, size_t src_off
 
 int mlc_hip_zero(void* buffer, size_t bytes) {
     if (!init_once()) return fail("GPU unavailable");
+    NOT_WHILE_CAPTURING("zero fill (a memset node in a replayed graph is not reliable on this platform)");
     if (!settle()) return 0;
     if (!buffer) return fail("zero: null pointer");
     const size_t known = known_bytes(buffer);
@@ -997,6 +1040,7 @@ int mlc_hip_begin(void) {
 
 int mlc_hip_flush(void) {
     if (!init_once()) return fail("GPU unavailable");
+    NOT_WHILE_CAPTURING("flush");
     if (!settle()) return 0;
     if (!g.pass_open) return 1;
     g.pass_open = false;
@@ -1108,14 +1152,15 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
     g.last_launches = 0;
     if (use_stream) {
         // per-request arrays: inside the kernel arguments when they fit, else uploaded with the table
-        const bool embed = batch <= kStreamEmbBatch;
-        static thread_local std::vector<uint32_t> meta3;
-        if (!embed) {
-            meta3.resize(3 * batch);
-            std::memcpy(meta3.data(), seq_lens, batch * 4);
-            std::memcpy(meta3.data() + batch, q_positions, batch * 4);
-            std::memcpy(meta3.data() + 2 * batch, page_table_offsets, batch * 4);
-        }
+        // (a captured pass reads them from the device copy, which mlc_hip_replay_update refreshes)
+        const bool embed = batch <= kStreamEmbBatch && !g_capturing;
+        // (kept on the host in any case: mlc_hip_capture_begin sends them to the device, so that a
+        // pass captured right after this call finds them there)
+        std::vector<uint32_t>& meta3 = g.tables.last_meta;
+        meta3.resize(3 * batch);
+        std::memcpy(meta3.data(), seq_lens, batch * 4);
+        std::memcpy(meta3.data() + batch, q_positions, batch * 4);
+        std::memcpy(meta3.data() + 2 * batch, page_table_offsets, batch * 4);
         const uint32_t* d_flat = nullptr;
         const uint32_t* d_meta = nullptr;
         if (!tables_upload(embed ? nullptr : meta3.data(), batch, &d_flat, &d_meta)) return 0;
@@ -1151,6 +1196,17 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
         }
         if (!launch_stream_variant(head_dim, s_hpw, s_nw, nbuf, a, n_wg, dyn_lds, g.stream))
             return fail("decode: kernel variant not built");
+        if (g_capturing) {
+            Ctx::Captured& c = g.cap;
+            if (c.used_tables && (c.B != batch || c.tables_flat != d_flat || c.tables_meta != d_meta))
+                return fail("capture: every decode call of a captured pass must use the same tables");
+            c.used_tables = true;
+            c.tables_flat = d_flat;
+            c.tables_meta = d_meta;
+            c.B = batch; c.H = num_heads; c.Hkv = kv_heads; c.D = head_dim; c.P = page_size_tokens;
+            c.causal = apply_causal ? 1 : 0;
+            c.carried_kv = c.carried_kv || carries_kv;
+        }
         g.last_items = (int)std::min<uint64_t>(n_wg, total_tiles);
         std::snprintf(g.last_kernel, sizeof g.last_kernel, "stream<%zu,%d,%d,%s,%s,%d>", head_dim, s_hpw, s_nw,
                       g.opt_pv_fp16 ? "pv16" : "pv32", batch <= 64 ? "regs" : "lds", nbuf);
@@ -1774,6 +1830,7 @@ Ctx::Q4Weight* q4_weight(const char* name, const uint8_t* host, size_t bytes, si
                          size_t stride) {
     Ctx::Q4Weight& w = g.q4_weights[name];
     if (w.raw && w.bytes == bytes && w.rows == rows && w.cols == cols && w.stride == stride) return &w;
+    if (g_capturing) { fail("q4 matmul: the weights are not on the device yet (run the pass once uncaptured first)"); return nullptr; }
     (void)hipStreamSynchronize(g.stream);
     for (void** p : {&w.raw, &w.qs, &w.d})
         if (*p) { (void)hipFree(*p); *p = nullptr; }
@@ -1937,6 +1994,7 @@ Ctx::Q6KWeight* q6k_weight(const char* name, const uint8_t* host, size_t bytes, 
                            size_t stride) {
     Ctx::Q6KWeight& w = g.q6k_weights[name];
     if (w.raw && w.bytes == bytes && w.rows == rows && w.cols == cols && w.stride == stride) return &w;
+    if (g_capturing) { fail("q6_k matmul: the weights are not on the device yet (run the pass once uncaptured first)"); return nullptr; }
     (void)hipStreamSynchronize(g.stream);
     for (void** p : {&w.raw, &w.qa, &w.sc, &w.d})
         if (*p) { (void)hipFree(*p); *p = nullptr; }
@@ -2121,6 +2179,161 @@ int mlc_hip_paged_attn_prefill(const void* q_f16, const void* k_pages, const voi
     return finish(sync);
 }
 
+// ---------------------------------------------------------------- captured passes (HIP graph)
+
+int mlc_hip_capture_begin(void) {
+    if (!init_once()) return fail("GPU unavailable");
+    if (g_capturing) return fail("capture: a pass is already being captured");
+    if (!g.pass_open) return fail("capture: no open forward pass");
+    if (!settle()) return 0;  // what was encoded before belongs to the uncaptured part
+    // The per-request arrays of the last decode call travelled inside its kernel arguments; a
+    // captured launch reads them from the device copy, which is brought up to date now.
+    if (!g.tables.last_meta.empty() && g.tables.filled) {
+        const uint32_t* d_flat = nullptr;
+        const uint32_t* d_meta = nullptr;
+        if (!tables_upload(g.tables.last_meta.data(), g.tables.last_meta.size() / 3, &d_flat, &d_meta)) return 0;
+    }
+    g.cap = Ctx::Captured{};
+    g_capture_failed = false;
+    HIP_OK(hipStreamBeginCapture(g.stream, hipStreamCaptureModeThreadLocal));
+    g_capturing = true;
+    return 1;
+}
+
+int mlc_hip_capture_end(void) {
+    if (!g.inited || !g_capturing) return fail("capture: no pass is being captured");
+    const int settled = settle();  // the operators still held back are launches of the captured pass
+    g_capturing = false;
+    hipGraph_t graph = nullptr;
+    const hipError_t e = hipStreamEndCapture(g.stream, &graph);
+    if (e != hipSuccess || !graph) {
+        (void)hipGetLastError();
+        if (graph) (void)hipGraphDestroy(graph);
+        return fail(std::string("capture: hipStreamEndCapture: ") + hipGetErrorString(e));
+    }
+    if (!settled || g_capture_failed) {
+        (void)hipGraphDestroy(graph);
+        if (g_capture_failed) return 0;  // the failing call's message stands
+        return fail("capture: the held-back operators could not be launched");
+    }
+    // kernel launches only: anything else (a copy, a memset) means some call did more than encode
+    size_t count = 0;
+    std::vector<hipGraphNode_t> nodes;
+    bool ok = hipGraphGetNodes(graph, nullptr, &count) == hipSuccess;
+    if (ok && count) {
+        nodes.resize(count);
+        ok = hipGraphGetNodes(graph, nodes.data(), &count) == hipSuccess;
+    }
+    for (size_t i = 0; ok && i < count; ++i) {
+        hipGraphNodeType type;
+        ok = hipGraphNodeGetType(nodes[i], &type) == hipSuccess && type == hipGraphNodeTypeKernel;
+    }
+    if (!ok || count == 0) {
+        (void)hipGraphDestroy(graph);
+        return fail(count == 0 ? "capture: nothing was encoded" : "capture: the pass holds something other than kernel launches");
+    }
+    hipGraphExec_t exec = nullptr;
+    if (hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0) != hipSuccess || !exec) {
+        (void)hipGetLastError();
+        (void)hipGraphDestroy(graph);
+        return fail("capture: hipGraphInstantiate failed");
+    }
+    Ctx::Captured c = g.cap;
+    c.graph = graph;
+    c.exec = exec;
+    c.n_nodes = count;
+    const int handle = g.next_capture++;
+    g.captures[handle] = c;
+    return handle;
+}
+
+size_t mlc_hip_captured_launches(int handle) {
+    auto it = g.captures.find(handle);
+    return it == g.captures.end() ? 0 : it->second.n_nodes;
+}
+
+int mlc_hip_replay_update(int handle, const uint32_t* page_tables_flat, size_t n_flat,
+                          const uint32_t* page_table_offsets, const uint32_t* seq_lens,
+                          const uint32_t* q_positions, const uint32_t* page_ids, const uint32_t* slots_in_page,
+                          size_t batch) {
+    if (!init_once()) return fail("GPU unavailable");
+    NOT_WHILE_CAPTURING("replay update");
+    auto it = g.captures.find(handle);
+    if (it == g.captures.end()) return fail("replay: unknown handle");
+    const Ctx::Captured& c = it->second;
+    if (!settle()) return 0;
+    if (c.used_tables) {
+        if (!page_table_offsets || !seq_lens || !q_positions || (n_flat && !page_tables_flat))
+            return fail("replay: null metadata");
+        if (batch != c.B) return fail("replay: the batch size differs from the captured pass (capture again)");
+        if (n_flat < page_table_offsets[batch]) return fail("replay: page table shorter than offsets");
+        const size_t tile = c.D == 64 ? 64 : 32;
+        uint64_t total_tiles = 0;
+        for (size_t r = 0; r < batch; ++r) {
+            const size_t pages = ((size_t)seq_lens[r] + c.P - 1) / c.P;
+            if ((size_t)page_table_offsets[r] + pages > n_flat) return fail("replay: page table does not cover seq_len");
+            uint64_t lim = seq_lens[r];
+            if (c.causal && (uint64_t)q_positions[r] + 1 < lim) lim = (uint64_t)q_positions[r] + 1;
+            total_tiles += (lim + tile - 1) / tile;
+        }
+        if (total_tiles * c.Hkv >= 0x7FFFFFFFull) return fail("replay: too many KV tiles for the captured kernel");
+        tables_refresh(page_tables_flat, n_flat, page_table_offsets, batch);
+        static thread_local std::vector<uint32_t> meta3;
+        meta3.resize(3 * batch);
+        std::memcpy(meta3.data(), seq_lens, batch * 4);
+        std::memcpy(meta3.data() + batch, q_positions, batch * 4);
+        std::memcpy(meta3.data() + 2 * batch, page_table_offsets, batch * 4);
+        const uint32_t* d_flat = nullptr;
+        const uint32_t* d_meta = nullptr;
+        if (!tables_upload(meta3.data(), batch, &d_flat, &d_meta)) return 0;
+        if (d_flat != c.tables_flat || d_meta != c.tables_meta)
+            return fail("replay: the device copy of the tables had to move (capture again)");
+        if (c.carried_kv) {
+            // the captured attention launch writes the step's K / V rows itself: they must still be
+            // every request's newest visible position, on pages no two requests share
+            if (!page_ids || !slots_in_page) return fail("replay: the captured pass writes K / V rows, page ids needed");
+            bool ok = g.tables.shared_pages == 0;
+            for (size_t r = 0; ok && r < batch; ++r) {
+                const uint64_t S = seq_lens[r];
+                const bool visible = !c.causal || (uint64_t)q_positions[r] + 1 >= S;
+                ok = S > 0 && visible && slots_in_page[r] == (S - 1) % c.P &&
+                     page_ids[r] == page_tables_flat[page_table_offsets[r] + (S - 1) / c.P];
+            }
+            if (!ok) return fail("replay: the rows to write are not every request's newest position (run this step uncaptured)");
+        }
+    }
+    if (c.ids_dev) {
+        if (!page_ids || !slots_in_page) return fail("replay: the captured pass writes K / V rows, page ids needed");
+        if (batch != c.ids_batch) return fail("replay: the batch size differs from the captured pass (capture again)");
+        for (size_t r = 0; r < batch; ++r)
+            if (c.P && slots_in_page[r] >= c.P) return fail("replay: slot >= page size");
+        const void* dev = resident_ids(page_ids, slots_in_page, batch, align_up(batch * 4, 16));
+        if (!dev) return 0;
+        if (dev != c.ids_dev) return fail("replay: the device copy of the page ids had to move (capture again)");
+    }
+    return 1;
+}
+
+int mlc_hip_replay(int handle) {
+    if (!init_once()) return fail("GPU unavailable");
+    NOT_WHILE_CAPTURING("replay");
+    auto it = g.captures.find(handle);
+    if (it == g.captures.end()) return fail("replay: unknown handle");
+    if (!settle()) return 0;
+    HIP_OK(hipGraphLaunch(it->second.exec, g.stream));
+    return 1;
+}
+
+void mlc_hip_capture_release(int handle) {
+    auto it = g.captures.find(handle);
+    if (it == g.captures.end()) return;
+    (void)hipStreamSynchronize(g.stream);
+    if (it->second.exec) (void)hipGraphExecDestroy(it->second.exec);
+    if (it->second.graph) (void)hipGraphDestroy(it->second.graph);
+    g.captures.erase(it);
+}
+
+
 void* mlc_hip_stream(void) {
     if (!init_once() || !settle()) return nullptr;  // the caller may enqueue behind what has been encoded
     return static_cast<void*>(g.stream);
@@ -2128,6 +2341,7 @@ void* mlc_hip_stream(void) {
 
 int mlc_hip_timer_start(void) {
     if (!init_once()) return fail("GPU unavailable");
+    NOT_WHILE_CAPTURING("timer");
     if (!settle()) return 0;
     HIP_OK(hipEventRecord(g.ev0, g.stream));
     return 1;
@@ -2135,6 +2349,7 @@ int mlc_hip_timer_start(void) {
 
 float mlc_hip_timer_stop(void) {
     if (!init_once()) return -1.f;
+    if (g_capturing) { fail("timer: not possible while a pass is being captured"); return -1.f; }
     if (!settle()) return -1.f;
     if (hipEventRecord(g.ev1, g.stream) != hipSuccess) return -1.f;
     if (hipEventSynchronize(g.ev1) != hipSuccess) return -1.f;

@@ -238,6 +238,32 @@ class HipExecutor:
             _ptr(off), _ptr(sl), _ptr(qs), batch, chunk, num_heads, kv_heads, head_dim,
             page_size_tokens, int(bool(sync))))
 
+    # -- a pass replayed from a HIP graph
+    def captureBegin(self) -> bool:
+        return bool(self._lib.mlc_hip_capture_begin())
+
+    def captureEnd(self) -> int:
+        """Handle > 0 of the captured pass, or 0 (see lastError)."""
+        return int(self._lib.mlc_hip_capture_end())
+
+    def capturedLaunches(self, handle: int) -> int:
+        return int(self._lib.mlc_hip_captured_launches(handle))
+
+    def replayUpdate(self, handle, page_tables_flat, page_table_offsets, seq_lens, q_positions,
+                     page_ids=None, slots_in_page=None) -> bool:
+        flat, off, seq, pos = (_u32(x) for x in (page_tables_flat, page_table_offsets, seq_lens, q_positions))
+        ids = _u32(page_ids) if page_ids is not None else None
+        slots = _u32(slots_in_page) if slots_in_page is not None else None
+        return bool(self._lib.mlc_hip_replay_update(handle, _ptr(flat), flat.size, _ptr(off), _ptr(seq), _ptr(pos),
+                                                    _ptr(ids) if ids is not None else None,
+                                                    _ptr(slots) if slots is not None else None, seq.size))
+
+    def replay(self, handle: int) -> bool:
+        return bool(self._lib.mlc_hip_replay(handle))
+
+    def captureRelease(self, handle: int) -> None:
+        self._lib.mlc_hip_capture_release(handle)
+
     # -- measurement helpers
     def timerStart(self) -> bool:
         return bool(self._lib.mlc_hip_timer_start())
