@@ -65,6 +65,11 @@ constexpr int stream_static_lds_bytes(int NBUF) { return NBUF * 2 * 8192; }
 // dynamic LDS: tile prefix [B + 1], visible lengths [B], page-table offsets [B]
 inline size_t stream_dynamic_lds_bytes(size_t batch) { return (3 * batch + 1) * 4; }
 
+// Timing probes, compiled in only for experiments (results then are wrong or partly so):
+//   -DMLC_STREAM_PROBE  thread 0 of every workgroup writes the 100 MHz counter at fixed points
+//   -DMLC_NO_LOADS      the tile loads are not issued (what the arithmetic alone takes)
+//   -DMLC_NO_COMPUTE    the tiles are loaded but not consumed (what the loads alone take)
+//   -DMLC_NO_TAIL       partials are neither stored nor merged (what publication and merge take)
 #ifdef MLC_STREAM_PROBE
 #define MLC_PROBE(i)                                                                                   \
     do {                                                                                               \
@@ -425,26 +430,27 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         const uint32_t tile_start = t * TT;
         const uint4* kl = reinterpret_cast<const uint4*>(cur) + lane;
         const uint4* vl = kl + TILE_BYTES / 16;
+        // All sixteen LDS reads of the tile are requested before anything is computed, K first
+        // (64 registers): left to the compiler the reads sit next to their uses, two at a time,
+        // and every pair exposes the LDS latency to a wave that has one other wave to hide behind.
+        // The empty statements keep the reads from being moved back down.
+        uint4 kreg[8], vreg[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) kreg[j] = kl[j * 64];
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int j = 0; j < 8; ++j) vreg[j] = vl[j * 64];
+        asm volatile("" ::: "memory");
         float part[HPW][8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const uint4 kq = kl[j * 64];
+            const uint4 kq = kreg[j];
             const half8_t kh = __builtin_bit_cast(half8_t, kq);
 #pragma unroll
             for (int h = 0; h < HPW; ++h) {
-#ifdef MLC_QK_DOT2
-                const uint32_t* kw = reinterpret_cast<const uint32_t*>(&kq);
-                float s = 0.f;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const half2_t qq = {(_Float16)qv[h][2 * i], (_Float16)qv[h][2 * i + 1]};
-                    s = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, kw[i]), qq, s, false);
-                }
-#else
                 float s = 0.f;
 #pragma unroll
                 for (int i = 0; i < 8; ++i) s = fmaf(qv[h][i], (float)kh[i], s);  // v_fma_mix_f32 throughout
-#endif
                 part[h][j] = s;
             }
         }
@@ -510,8 +516,8 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
             }
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-                const uint4 va4 = vl[(2 * k) * 64];
-                const uint4 vb4 = vl[(2 * k + 1) * 64];
+                const uint4 va4 = vreg[2 * k];
+                const uint4 vb4 = vreg[2 * k + 1];
                 const uint32_t* va = reinterpret_cast<const uint32_t*>(&va4);
                 const uint32_t* vb = reinterpret_cast<const uint32_t*>(&vb4);
                 uint32_t vp[8];
@@ -555,7 +561,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
             }
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const uint4 vq = vl[j * 64];
+                const uint4 vq = vreg[j];
                 const half8_t vh = __builtin_bit_cast(half8_t, vq);
 #pragma unroll
                 for (int h = 0; h < HPW; ++h)
@@ -741,17 +747,6 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     load_q(cc);
     uint32_t issued = 1;
     issue_tile(ci, 0);
-#ifdef MLC_PROLOGUE_FULL
-#pragma unroll
-    for (int i = 1; i < NBUF; ++i) {
-        if (issued < n) {
-            advance(ci);
-            if (!pages_ready(ci)) fetch_pages(ci);
-            issue_tile(ci, (uint32_t)i);
-            ++issued;
-        }
-    }
-#endif
     uint32_t seg_first = g0;  // first tile consumed for the pair under cc
     bool drain = false;       // stores are in flight: they do not complete in order with loads
     uint32_t slot = 0;        // stage of tile k
@@ -766,7 +761,6 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         sd_barrier();   // ... and everyone's; everyone has left tile k-1, whose stage is free
         if (k < 6) MLC_PROBE(9 + 3 * k);
         if (k == 0) MLC_PROBE(3);
-#ifndef MLC_PROLOGUE_FULL
         // one tile went out up front; from the first step on the stream runs NBUF - 1 tiles ahead
         // (all stages requested at once would make every workgroup wait for the whole burst)
         while (issued < n && issued < k + (uint32_t)NBUF) {
@@ -775,14 +769,6 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
             issue_tile(ci, issued % (uint32_t)NBUF);
             ++issued;
         }
-#else
-        if (k >= 1 && issued < n) {
-            advance(ci);
-            if (!pages_ready(ci)) fetch_pages(ci);  // another request, or 64 tiles on
-            issue_tile(ci, slot == 0 ? (uint32_t)(NBUF - 1) : slot - 1u);
-            ++issued;
-        }
-#endif
 #ifndef MLC_NO_COMPUTE
         consume_tile(slot, cc.t, cc.lim);
 #endif
