@@ -826,16 +826,16 @@ int tables_upload(const uint32_t* meta3, size_t B, const uint32_t** d_flat, cons
         }
         MetaSlot& s = g.ring[g.ring_next];
         g.ring_next = (g.ring_next + 1) % 8;
-        const size_t bytes = flat_room + meta_bytes;
-        if (!slot_reserve(s, bytes)) return 0;
+        const size_t flat_stage = align_up(n_flat * 4, 16);   // the staging slot holds the two side by side
+        if (!slot_reserve(s, flat_stage + meta_bytes)) return 0;
         char* h = static_cast<char*>(s.host);
         if (n_flat) std::memcpy(h, t.flat.data(), n_flat * 4);
         if (meta3) {
-            std::memcpy(h + flat_room, meta3, meta_bytes);
+            std::memcpy(h + flat_stage, meta3, meta_bytes);
             t.meta.assign(meta3, meta3 + 3 * B);
-            // table and arrays in two copies: what lies between them is not sent
+            // table and arrays in two copies: what lies between them on the device is not sent
             if (n_flat) HIP_OK(hipMemcpyAsync(t.dev, h, n_flat * 4, hipMemcpyHostToDevice, g.stream));
-            HIP_OK(hipMemcpyAsync(static_cast<char*>(t.dev) + flat_room, h + flat_room, meta_bytes,
+            HIP_OK(hipMemcpyAsync(static_cast<char*>(t.dev) + flat_room, h + flat_stage, meta_bytes,
                                   hipMemcpyHostToDevice, g.stream));
         } else {
             t.meta.clear();
@@ -1161,9 +1161,12 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
         std::memcpy(meta3.data(), seq_lens, batch * 4);
         std::memcpy(meta3.data() + batch, q_positions, batch * 4);
         std::memcpy(meta3.data() + 2 * batch, page_table_offsets, batch * 4);
+        // ... and the flat table with them when it fits behind them: then nothing is copied to the
+        // device, however often the tables change
+        const bool embed_table = embed && 3 * batch + n_flat <= kStreamEmbWords;
         const uint32_t* d_flat = nullptr;
         const uint32_t* d_meta = nullptr;
-        if (!tables_upload(embed ? nullptr : meta3.data(), batch, &d_flat, &d_meta)) return 0;
+        if (!embed_table && !tables_upload(embed ? nullptr : meta3.data(), batch, &d_flat, &d_meta)) return 0;
         const size_t dyn_lds = batch <= 64 ? 0 : stream_dynamic_lds_bytes(batch);
         const int nbuf = stream_stages(batch);
         const unsigned n_wg = stream_grid(G, head_dim, nbuf, dyn_lds);
@@ -1180,13 +1183,12 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
             size_t pages = std::min(kk ? kk / page_bytes : SIZE_MAX, kv ? kv / page_bytes : SIZE_MAX);
             if (pages != SIZE_MAX) a.capacity_pages = (uint32_t)std::min<size_t>(pages, 0xFFFFFFFFu);
         }
+        a.meta_stride = (uint32_t)batch;
         if (embed) {
-            std::memcpy(a.emb, seq_lens, batch * 4);
-            std::memcpy(a.emb + kStreamEmbBatch, q_positions, batch * 4);
-            std::memcpy(a.emb + 2 * kStreamEmbBatch, page_table_offsets, batch * 4);
+            std::memcpy(a.emb, meta3.data(), 3 * batch * 4);
+            if (embed_table && n_flat) std::memcpy(a.emb + 3 * batch, page_tables_flat, n_flat * 4);
         } else {
             a.meta = d_meta;
-            a.meta_stride = (uint32_t)batch;
         }
         if (carries_kv) {
             a.new_k = static_cast<const uint4*>(g.kv.src[0]);
@@ -1341,9 +1343,10 @@ int mlc_hip_paged_attn_decode_noalloc(const void* q, const void* k_pages, const 
         const size_t pages = std::min(kk ? kk / page_bytes : SIZE_MAX, kv ? kv / page_bytes : SIZE_MAX);
         if (pages != SIZE_MAX) a.capacity_pages = (uint32_t)std::min<size_t>(pages, 0xFFFFFFFFu);
     }
+    a.meta_stride = (uint32_t)batch;
     std::memcpy(a.emb, seq_lens, batch * 4);
-    std::memcpy(a.emb + kStreamEmbBatch, q_positions, batch * 4);
-    std::memcpy(a.emb + 2 * kStreamEmbBatch, page_table_offsets, batch * 4);
+    std::memcpy(a.emb + batch, q_positions, batch * 4);
+    std::memcpy(a.emb + 2 * batch, page_table_offsets, batch * 4);
     hipStream_t st = stream ? static_cast<hipStream_t>(stream) : g.stream;
     if (!launch_stream_variant(head_dim, hpw, nw, nbuf, a, n_wg, dyn_lds, st))
         return fail("decode: kernel variant not built");

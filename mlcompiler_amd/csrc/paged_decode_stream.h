@@ -28,6 +28,7 @@
 namespace mlc_hip {
 
 static constexpr uint32_t kStreamEmbBatch = 256;    // requests whose arrays fit the kernel arguments
+static constexpr uint32_t kStreamEmbWords = 960;    // words of the kernel arguments that carry tables
 static constexpr uint32_t kStreamMaxBatch = 4096;   // 64-ary search over the tile prefix in two levels
 static constexpr uint32_t kStreamMaxWgs = 2048;     // workgroups per launch, at most
 
@@ -36,9 +37,9 @@ struct StreamArgs {
     const uint4* k_pages;       // fp16 pages, viewed as 16-byte chunks
     const uint4* v_pages;
     float* o;                   // [B][H][D]
-    const uint32_t* pt_flat;    // device copy of page_tables_flat
+    const uint32_t* pt_flat;    // device copy of page_tables_flat; null: the table is in emb, behind the arrays
     const uint32_t* meta;       // device [3][meta_stride]: seq_lens, q_positions, page_table_offsets;
-                                // null: the arrays are in emb (stride kStreamEmbBatch)
+                                // null: the arrays are in emb (same layout)
     float* part_o;              // [2 * n_wg][G][D] un-normalised partial outputs
     float* part_ml;             // [2 * n_wg][G][2] (m in log2 units, l)
     uint32_t* counters;         // [n_wg][NW] arrival counters, zero between launches
@@ -57,8 +58,11 @@ struct StreamArgs {
     const uint4* new_v;
     const uint32_t* new_ids;
     const uint32_t* new_slots;
-    uint32_t emb[3 * kStreamEmbBatch];
+    // seq_lens | q_positions | page_table_offsets (meta_stride words each) and, where it fits as
+    // well, the flat page table: a call whose tables travel here copies nothing to the device
+    uint32_t emb[kStreamEmbWords];
 };
+static_assert(sizeof(StreamArgs) <= 4096, "kernel arguments are limited to 4 KiB");
 
 // LDS of one workgroup: NBUF stages of one K tile and one V tile (8 KiB each)
 constexpr int stream_static_lds_bytes(int NBUF) { return NBUF * 2 * 8192; }
@@ -168,7 +172,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         // The arrays inside the kernel arguments are read before anything else is known (their
         // address is the argument segment's, no pointer has to be fetched first); lanes past
         // the batch read other arguments and are masked.
-        uint32_t seq = a.emb[lane], qp = a.emb[kStreamEmbBatch + lane], off = a.emb[2 * kStreamEmbBatch + lane];
+        uint32_t seq = a.emb[lane], qp = a.emb[a.meta_stride + lane], off = a.emb[2 * a.meta_stride + lane];
         if (a.meta != nullptr && (uint32_t)lane < B) {
             seq = a.meta[lane];
             qp = a.meta[a.meta_stride + lane];
@@ -185,7 +189,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     } else {
         if (wave == 0) {
             const uint32_t* meta = a.meta ? a.meta : a.emb;
-            const uint32_t stride = a.meta ? a.meta_stride : kStreamEmbBatch;
+            const uint32_t stride = a.meta_stride;
             uint32_t carry = 0;
             for (uint32_t b0 = 0; b0 < B; b0 += 64) {
                 const uint32_t i = b0 + lane;
@@ -299,6 +303,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     seek(cc, g0);
     ci = cc;
 
+    const uint32_t* pt_flat = a.pt_flat ? a.pt_flat : a.emb + 3u * a.meta_stride;
     // Page ids of the issue side's request, 64 tiles at a time: lane i holds the page of tile
     // pv_win + i.  Refetched when the issue side enters another request or another window.
     uint32_t pv = 0, pv_win = 0, pv_req = 0xFFFFFFFFu;
@@ -307,7 +312,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         pv_win = cu.t & ~63u;
         const uint32_t t = pv_win + (uint32_t)lane;
         pv = 0;
-        if (t < cu.tiles) pv = a.pt_flat[cu.off + t / tpp];
+        if (t < cu.tiles) pv = pt_flat[cu.off + t / tpp];
         // The ids are waited for here, inside whatever branch fetches them: left pending, the
         // compiler would wait at every later join of the control flow, and as it does not know
         // of the tile loads, that wait would be for all of them.

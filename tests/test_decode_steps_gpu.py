@@ -99,7 +99,52 @@ def test_130_consecutive_decode_steps(exe):
         for b in (k_buf, v_buf, q_buf, o_buf, nk_buf, nv_buf):
             exe.releaseScratchBuffer(b)
     assert exe.kvWritesInDecodeLaunches() - carried0 == STEPS       # the attention launch took every write
-    # the table went to the device only when its content changed: at the first step and at the
-    # steps where some request opened a page
-    assert exe.tableUploads() - uploads0 == grew_steps
-    assert grew_steps < STEPS // 4
+    # tables of this size travel inside the kernel arguments: nothing was copied to the device,
+    # although the table changed at every step where some request opened a page
+    assert exe.tableUploads() - uploads0 == 0
+    assert 0 < grew_steps < STEPS // 4
+
+
+def test_large_page_table_is_uploaded_only_when_it_changes(exe):
+    H, HKV, D, P = 32, 4, 64, 64
+    lens = [30000 - 2, 29000, 64 * 300 - 1]       # 1 240 pages: more than the kernel arguments hold
+    B = len(lens)
+    cap = sum((s + 8 + P - 1) // P for s in lens) + 2
+    rng = np.random.default_rng(31)
+    free = list(rng.permutation(cap).astype(np.uint32))
+    tables = [[free.pop() for _ in range((s + P - 1) // P)] for s in lens]
+    row = HKV * D
+    k_pool = rng.standard_normal(cap * P * row, dtype=np.float32).astype(np.float16).view(np.uint16)
+    v_pool = rng.standard_normal(cap * P * row, dtype=np.float32).astype(np.float16).view(np.uint16)
+    k_buf, v_buf = exe.allocateScratchBuffer(k_pool.nbytes), exe.allocateScratchBuffer(v_pool.nbytes)
+    q_buf, o_buf = exe.allocateScratchBuffer(B * H * D * 4), exe.allocateScratchBuffer(B * H * D * 4)
+    uploads = []
+    try:
+        assert exe.uploadToBuffer(k_buf, k_pool) and exe.uploadToBuffer(v_buf, v_pool)
+        for step in range(4):
+            grew = False
+            for r in range(B):
+                if lens[r] % P == 0:
+                    tables[r].append(free.pop())
+                    grew = True
+                lens[r] += 1
+            flat = np.array([p for t in tables for p in t], np.uint32)
+            off = np.zeros(B + 1, np.uint32)
+            off[1:] = np.cumsum([len(t) for t in tables])
+            seq = np.array(lens, np.uint32)
+            q = rng.standard_normal((B, H, D), dtype=np.float32)
+            assert exe.uploadToBuffer(q_buf, q)
+            before = exe.tableUploads()
+            for _layer in range(3):        # the layers of a step pass the same tables
+                assert exe.runPagedFlashAttention(q_buf, k_buf, v_buf, o_buf, flat, off, seq, seq - 1, B, H, HKV, D, P,
+                                                  True), exe.lastError()
+            uploads.append((grew or step == 0, exe.tableUploads() - before))
+            got = np.empty((B, H, D), np.float32)
+            assert exe.downloadFromBuffer(o_buf, got)
+            want = po.paged_attention_executor(q, k_pool, v_pool, flat, off, seq, seq - 1, B, H, HKV, D, P, True, 8)
+            assert_parity(got, want, D, f"long requests, step {step}")
+    finally:
+        for b in (k_buf, v_buf, q_buf, o_buf):
+            exe.releaseScratchBuffer(b)
+    assert [n for _, n in uploads] == [1 if changed else 0 for changed, _ in uploads], uploads
+    assert sum(changed for changed, _ in uploads) in (2, 3)     # the first step and where a request opened a page
