@@ -83,6 +83,12 @@ inline size_t stream_dynamic_lds_bytes(size_t batch) { return (3 * batch + 1) * 
 #else
 #define MLC_PROBE(i)
 #endif
+// (-DMLC_STREAM_PROBE_TILES adds three stamps per tile; each stamp costs about 0.2 us)
+#ifdef MLC_STREAM_PROBE_TILES
+#define MLC_PROBE_TILE(i) MLC_PROBE(i)
+#else
+#define MLC_PROBE_TILE(i)
+#endif
 
 // 16-byte global -> LDS load that bypasses the register file: lane i's 16 bytes land at LDS byte
 // address lds_base + 16*i (lds_base wave-uniform).  Issued as inline assembly on purpose: the
@@ -392,7 +398,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
             const int tensor = (NW == 1) ? p : (NW == 2 ? hg : hg / 2);
             const int j0 = (NW == 4) ? (hg % 2) * 4 : 0;
             const uint4* base = (tensor ? a.v_pages : a.k_pages) + row0;
-            const uint32_t dst = stages_lds + slot * STAGE_BYTES + tensor * TILE_BYTES;
+            const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)(stages_lds + slot * STAGE_BYTES + tensor * TILE_BYTES));
 #pragma unroll
             for (int jj = 0; jj < JN; ++jj) {
                 const int j = j0 + jj;
@@ -679,11 +685,45 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     };
     // Merge of a pair's partials by the wave that arrived last, in the order of their slots (so
     // the result does not depend on who arrived last).  64 partials at a time: lane s holds the
-    // (m, l) of partial s for every head; the partial outputs are loaded eight at a time, the
-    // first eight (nearly always: all) together with the (m, l) pairs, before anything is
-    // consumed: one memory round trip.
-    auto merge = [&](const PairOut& po) {
-        auto slot_of = [&](uint32_t i) { return i == 0 ? po.slot_first : 2u * (po.w_lo + i); };
+    // (m, l) of partial s for every head; the partial outputs are loaded eight at a time.  The
+    // loads of the first round -- the (m, l) pairs and the first eight outputs, nearly always all
+    // there is -- are a step of their own (merge_fetch), so that a wave that merges two pairs
+    // has both pairs' loads in flight together: one memory round trip in all.
+    constexpr int MUNR = 8;
+    struct MergeLoads {
+        float pvv[MUNR][OPL];
+        float ms[HPW], ls[HPW];
+    };
+    auto merge_slot = [&](const PairOut& po, uint32_t i) { return i == 0 ? po.slot_first : 2u * (po.w_lo + i); };
+    auto merge_fetch_outputs = [&](const PairOut& po, uint32_t first, uint32_t cnt, float (&pvv)[MUNR][OPL]) {
+#pragma unroll
+        for (int u = 0; u < MUNR; ++u) {
+            const float* src = a.part_o + ((size_t)merge_slot(po, first + u) * G + hg * HPW) * D;
+#pragma unroll
+            for (int k = 0; k < OPL; ++k) {
+                pvv[u][k] = 0.f;
+                if ((uint32_t)u < cnt) pvv[u][k] = ld_dev(src + k * 64 + lane);
+            }
+        }
+    };
+    auto merge_fetch_ml = [&](const PairOut& po, uint32_t s0, uint32_t cnt, float (&ms)[HPW], float (&ls)[HPW]) {
+        const float* ml = a.part_ml + ((size_t)merge_slot(po, s0 + (uint32_t)lane) * G + hg * HPW) * 2;
+#pragma unroll
+        for (int h = 0; h < HPW; ++h) {
+            ms[h] = kNegBig;
+            ls[h] = 0.f;
+            if ((uint32_t)lane < cnt) {
+                ms[h] = ld_dev(ml + h * 2);
+                ls[h] = ld_dev(ml + h * 2 + 1);
+            }
+        }
+    };
+    auto merge_fetch = [&](const PairOut& po, MergeLoads& ld) {
+        const uint32_t cnt = min(64u, po.n_splits);
+        merge_fetch_outputs(po, 0, cnt, ld.pvv);
+        merge_fetch_ml(po, 0, cnt, ld.ms, ld.ls);
+    };
+    auto merge = [&](const PairOut& po, MergeLoads& ld) {
         float acc_o[OPL], m_run[HPW], l_run[HPW];
 #pragma unroll
         for (int k = 0; k < OPL; ++k) acc_o[k] = 0.f;
@@ -692,54 +732,31 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
             m_run[h] = kNegBig;
             l_run[h] = 0.f;
         }
-        constexpr int UNR = 8;
         for (uint32_t s0 = 0; s0 < po.n_splits; s0 += 64) {
             const uint32_t cnt = min(64u, po.n_splits - s0);
-            float pvv[UNR][OPL];
-            auto load_outputs = [&](uint32_t u0) {
-#pragma unroll
-                for (int u = 0; u < UNR; ++u) {
-                    const float* src = a.part_o + ((size_t)slot_of(s0 + u0 + u) * G + hg * HPW) * D;
-#pragma unroll
-                    for (int k = 0; k < OPL; ++k) {
-                        pvv[u][k] = 0.f;
-                        if (u0 + u < cnt) pvv[u][k] = ld_dev(src + k * 64 + lane);
-                    }
-                }
-            };
-            load_outputs(0);
-            float ms[HPW], ls[HPW];
-            {
-                const float* ml = a.part_ml + ((size_t)slot_of(s0 + (uint32_t)lane) * G + hg * HPW) * 2;
-#pragma unroll
-                for (int h = 0; h < HPW; ++h) {
-                    ms[h] = kNegBig;
-                    ls[h] = 0.f;
-                    if ((uint32_t)lane < cnt) {
-                        ms[h] = ld_dev(ml + h * 2);
-                        ls[h] = ld_dev(ml + h * 2 + 1);
-                    }
-                }
+            if (s0) {
+                merge_fetch_outputs(po, s0, cnt, ld.pvv);
+                merge_fetch_ml(po, s0, cnt, ld.ms, ld.ls);
             }
             float wgt[HPW];
 #pragma unroll
             for (int h = 0; h < HPW; ++h) {
-                const float m_new = max_nn(m_run[h], wave_max(ms[h]));
+                const float m_new = max_nn(m_run[h], wave_max(ld.ms[h]));
                 const float keep = fast_exp2(m_run[h] - m_new);
-                wgt[h] = fast_exp2(ms[h] - m_new);  // lanes >= cnt: exp2(-1e30 - m) = 0
+                wgt[h] = fast_exp2(ld.ms[h] - m_new);  // lanes >= cnt: exp2(-1e30 - m) = 0
                 l_run[h] = l_run[h] * keep + __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(
-                                                 int, wave_sum(wgt[h] * ls[h]))));
+                                                 int, wave_sum(wgt[h] * ld.ls[h]))));
                 m_run[h] = m_new;
 #pragma unroll
                 for (int kk = 0; kk < HPK; ++kk) acc_o[h * HPK + kk] *= keep;
             }
-            for (uint32_t u0 = 0; u0 < cnt; u0 += UNR) {
-                if (u0) load_outputs(u0);
+            for (uint32_t u0 = 0; u0 < cnt; u0 += MUNR) {
+                if (u0) merge_fetch_outputs(po, s0 + u0, cnt - u0, ld.pvv);
 #pragma unroll
-                for (int u = 0; u < UNR; ++u) {
+                for (int u = 0; u < MUNR; ++u) {
                     if (u0 + u < cnt) {
 #pragma unroll
-                        for (int k = 0; k < OPL; ++k) acc_o[k] += __shfl(wgt[k / HPK], (int)(u0 + u)) * pvv[u][k];
+                        for (int k = 0; k < OPL; ++k) acc_o[k] += __shfl(wgt[k / HPK], (int)(u0 + u)) * ld.pvv[u][k];
                     }
                 }
             }
@@ -760,11 +777,11 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     float kept_o[OPL], kept_m[HPW], kept_l[HPW];
     for (uint32_t k = 0; k < n; ++k) {
         // this wave's loads of tile k have landed ...
-        if (k < 6) MLC_PROBE(8 + 3 * k);
+        if (k < 6) MLC_PROBE_TILE(8 + 3 * k);
         if (drain) sd_wait_vmcnt<0>(); else wait_tile(issued - k - 1u);
         drain = false;
         sd_barrier();   // ... and everyone's; everyone has left tile k-1, whose stage is free
-        if (k < 6) MLC_PROBE(9 + 3 * k);
+        if (k < 6) MLC_PROBE_TILE(9 + 3 * k);
         if (k == 0) MLC_PROBE(3);
         // one tile went out up front; from the first step on the stream runs NBUF - 1 tiles ahead
         // (all stages requested at once would make every workgroup wait for the whole burst)
@@ -779,7 +796,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
 #endif
         const bool pair_done = cc.t + 1u == cc.tiles;
         const bool range_done = k + 1 == n;
-        if (k < 6) MLC_PROBE(10 + 3 * k);
+        if (k < 6) MLC_PROBE_TILE(10 + 3 * k);
         if (range_done) MLC_PROBE(4);
         if (pair_done || range_done) {
             float o_un[OPL], m_all[HPW], l_all[HPW];
@@ -837,8 +854,11 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
                         if (last_kept) __hip_atomic_store(c_kept, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                         if (last_cur) __hip_atomic_store(c_cur, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     }
-                    if (last_kept) merge(kept_po);
-                    if (last_cur) merge(cur_po);
+                    MergeLoads ld_kept, ld_cur;
+                    if (last_kept) merge_fetch(kept_po, ld_kept);
+                    if (last_cur) merge_fetch(cur_po, ld_cur);
+                    if (last_kept) merge(kept_po, ld_kept);
+                    if (last_cur) merge(cur_po, ld_cur);
                 }
             }
             reset_state();
