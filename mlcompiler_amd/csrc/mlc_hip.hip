@@ -816,6 +816,7 @@ int tables_upload(const uint32_t* meta3, size_t B, const uint32_t** d_flat, cons
         if (t.meta.size() != 3 * B || std::memcmp(t.meta.data(), meta3, meta_bytes) != 0) upload = true;
     }
     if (upload) {
+        NOT_WHILE_CAPTURING("copying the decode tables to the device (run the pass once uncaptured first)");
         if (total > t.cap) {
             HIP_OK(hipStreamSynchronize(g.stream));
             if (t.dev) HIP_OK(hipFree(t.dev));
@@ -2191,7 +2192,7 @@ int mlc_hip_capture_begin(void) {
     if (!settle()) return 0;  // what was encoded before belongs to the uncaptured part
     // The per-request arrays of the last decode call travelled inside its kernel arguments; a
     // captured launch reads them from the device copy, which is brought up to date now.
-    if (!g.tables.last_meta.empty() && g.tables.filled) {
+    if (!g.tables.last_meta.empty()) {
         const uint32_t* d_flat = nullptr;
         const uint32_t* d_meta = nullptr;
         if (!tables_upload(g.tables.last_meta.data(), g.tables.last_meta.size() / 3, &d_flat, &d_meta)) return 0;

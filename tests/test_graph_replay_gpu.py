@@ -193,3 +193,39 @@ def test_what_a_capture_and_a_replay_refuse(exe):
         if handle:
             exe.captureRelease(handle)
         bufs.free()
+
+
+def test_capture_in_a_process_that_only_saw_small_tables():
+    """Small tables travel inside the kernel arguments and are never copied to the device by an
+    ordinary call; a capture must still find them there (capture_begin sends them).  Run in a
+    process of its own, so that no earlier test has put tables on the device."""
+    import os
+    import subprocess
+    import sys
+    code = r"""
+import sys, numpy as np
+sys.path.insert(0, %r); sys.path.insert(0, %r)
+import test_graph_replay_gpu as t
+from mlcompiler_amd import HipExecutor
+exe = HipExecutor.Instance(); exe.requireAvailable()
+rng = np.random.default_rng(3)
+reqs = t._Requests([5, 70], 8, rng)
+pool = rng.standard_normal(8 * t.P * t.ROW, dtype=np.float32).astype(np.float16).view(np.uint16)
+bufs = t._Buffers(exe, pool, pool, 2)
+tab = reqs.step()
+bufs.inputs(rng.standard_normal((2, t.H, t.D), dtype=np.float32), pool[:2 * t.ROW], pool[:2 * t.ROW])
+assert exe.beginForwardPassCB(); bufs.encode(tab, 2); assert exe.flushForwardPassCB()
+assert exe.tableUploads() == 0
+assert exe.beginForwardPassCB() and exe.captureBegin(), exe.lastError()
+bufs.encode(tab, 2)
+h = exe.captureEnd()
+assert h > 0, exe.lastError()
+assert exe.flushForwardPassCB()
+a = bufs.outputs(2)[0]
+assert exe.replayUpdate(h, tab["flat"], tab["off"], tab["seq"], tab["qpos"], tab["ids"], tab["slots"]), exe.lastError()
+assert exe.beginForwardPassCB() and exe.replay(h) and exe.flushForwardPassCB()
+assert np.array_equal(a, bufs.outputs(2)[0])
+print("ok")
+""" % (os.path.dirname(os.path.dirname(os.path.abspath(__file__))), os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=240)
+    assert proc.returncode == 0 and "ok" in proc.stdout, proc.stdout + proc.stderr
