@@ -779,6 +779,12 @@ def main() -> int:
               "use --gpus 1", file=sys.stderr)
         return 2
 
+    if args.opt:
+        from mlcompiler_amd import HipExecutor
+        for kv in args.opt:
+            name, value = kv.split("=")
+            assert HipExecutor.Instance().setOption(name, int(value)), f"unknown option {kv}"
+
     if args.workload == "cfg5":
         print(json.dumps(bench_prefill(args)))
         return 0
@@ -800,10 +806,6 @@ def main() -> int:
         assert exe.setOption("decode_wgs_per_cu", args.wgs_per_cu)
     if args.stages:
         assert exe.setOption("decode_stages", args.stages)
-    for kv in args.opt:
-        name, value = kv.split("=")
-        assert exe.setOption(name, int(value)), f"unknown option {kv}"
-
     per_config = args.per_config == 1 or (args.per_config < 0 and args.workload == "cfg2" and not args.no_cpu)
     r = run_decode(args, args.workload, args.steps, args.warmup, args.cpu_budget, full=True)
     c = r["case"]

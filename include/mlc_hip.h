@@ -235,6 +235,8 @@ int mlc_hip_matmul_q6_k_batched(const char* weight_name, const void* weights, si
  *   q  fp16 [batch][chunk][num_heads][head_dim]; row i of request r sits at
  *      absolute position q_start[r] + i and attends kv positions <= that and
  *      < seq_lens[r].   o  fp32, same shape as q.
+ * page_table_offsets has batch entries; request r's table holds at least
+ * ceil(seq_lens[r] / page_size_tokens) page ids from there on.
  * sync as above (0 needs an open pass). */
 int mlc_hip_paged_attn_prefill(const void* q_f16, const void* k_pages, const void* v_pages,
                                void* o,
@@ -370,6 +372,9 @@ long mlc_hip_decode_table_uploads(void);
  *                           the same page ids) become one launch.
  *                           0 = each operator is launched when it is encoded
  *   "prefill_stages"        2, 4, 6 or 8 K/V tiles staged in LDS by the prefill kernel (0 = automatic)
+ *   "prefill_rows64"        1 (default) = heads/kv_heads up to 4 run the prefill kernel with 64
+ *                           chunk rows per wave; 0 = the kernel with 32 rows per wave for every
+ *                           ratio (ratio 8 always runs it)
  * Returns 0 for an unknown name or value. */
 int mlc_hip_set_option(const char* name, long value);
 

@@ -224,6 +224,7 @@ struct Ctx {
     long opt_buffers = 0;                                      // LDS staging buffers per workgroup (1, 2; 0 = automatic)
     long opt_tile_rows = 1;                                    // wave rows that share an item's tiles
     long opt_prefill_stages = 0;                               // LDS pipeline depth of the prefill kernel (0 = automatic)
+    long opt_prefill_rows64 = 1;                               // prefill: 64 chunk rows per wave where the GQA ratio allows it
     long opt_pv_fp16 = 1;                                      // softmax weights rounded to fp16 for P.V
     int last_launches = 0;
     int last_items = 0;
@@ -2178,7 +2179,7 @@ int mlc_hip_paged_attn_prefill(const void* q_f16, const void* k_pages, const voi
     a.page_size = (uint32_t)page_size_tokens;
     a.scale_log2e = (1.0f / std::sqrt(static_cast<float>(head_dim))) * 1.44269504088896340736f;
     a.row_blocks = 0;  // set by the launcher
-    launch_prefill(a, head_dim, (int)g.opt_prefill_stages, g.stream);
+    launch_prefill(a, head_dim, (int)g.opt_prefill_stages, g.opt_prefill_rows64 != 0, g.stream);
     if (!slot_mark(s)) return 0;
     return finish(sync);
 }
@@ -2417,6 +2418,11 @@ int mlc_hip_set_option(const char* name, long value) {
     if (!std::strcmp(name, "prefill_stages")) {
         if (value != 0 && value != 2 && value != 4 && value != 6 && value != 8) return 0;
         g.opt_prefill_stages = value;
+        return 1;
+    }
+    if (!std::strcmp(name, "prefill_rows64")) {
+        if (value != 0 && value != 1) return 0;
+        g.opt_prefill_rows64 = value;
         return 1;
     }
     if (!std::strcmp(name, "decode_buffers")) {

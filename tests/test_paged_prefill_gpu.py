@@ -172,3 +172,24 @@ def test_prefill_baseline_config5_every_row_of_one_request(exe):
     rep = po.per_head_report(got[r], want[0], 128)
     print("[prefill] config 5, request 3, 256 rows:", rep, flush=True)
     assert rep["min_cosine"] >= MIN_COSINE and rep["max_abs"] <= MAX_ABS, rep
+
+
+def test_prefill_32_rows_per_wave_kernel_for_small_gqa_ratios(exe):
+    """GQA ratios up to 4 run the 64-rows-per-wave kernel by default; the 32-row kernel (the only
+    one for ratio 8) must stay right for them too."""
+    assert exe.setOption("prefill_rows64", 0)
+    try:
+        for H, Hkv, D in ((8, 2, 128), (8, 8, 64)):
+            w = make_prefill(2, 40, H, Hkv, D, 64, [100, 0], seed=H + D + 1)
+            check(exe, w, f"rows32 H{H} Hkv{Hkv} D{D}")
+    finally:
+        assert exe.setOption("prefill_rows64", 1)
+
+
+def test_prefill_more_than_64_pages_and_one_tile_per_page(exe):
+    """32-token pages (one K/V tile per page) and a sequence of more than 64 pages: the page ids
+    are held 64 at a time; also a sequence shorter than the tiles kept in flight."""
+    w = make_prefill(2, 64, 8, 2, 64, 32, [2500, 3], seed=21)
+    check(exe, w, "80 pages of 32 tokens")
+    w = make_prefill(1, 48, 4, 1, 128, 32, [2100], seed=22)
+    check(exe, w, "68 pages, head_dim 128, one KV head")
