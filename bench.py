@@ -829,8 +829,9 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32 accumulate and output (fp16 K/V storage, fp32 q; softmax weights rounded to fp16 for P.V, "
-                 "option decode_pv_fp16: us_per_layer_pv_fp32 is the time with fp32 weights)",
+        "dtype": "f32 accumulate and output (fp16 K/V storage; products on f16 MFMA: fp32 q enters as the sum of "
+                 "two fp16 numbers, softmax weights are rounded to fp16 for P.V; option decode_pv_fp16 = 0: fp32 "
+                 "weights on the vector pipe, us_per_layer_pv_fp32 is its time)",
         "data": "synthetic",
         "config": {
             "workload": workload_text(c, r["n_layers"]),

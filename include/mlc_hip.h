@@ -358,7 +358,7 @@ long mlc_hip_decode_table_uploads(void);
  *   "decode_tile_rows"      1 or 2: wave rows of a workgroup that share an item's tiles
  *   "decode_buffers"        1 or 2 LDS staging buffers per workgroup (0 = automatic)
  *   "decode_pv_fp16"        1 = softmax weights rounded to fp16 for the P.V product
- *                           (v_dot2_f32_f16, fp32 accumulate), 0 = fp32 weights
+ *                           (fp32 accumulate), 0 = fp32 weights (vector pipe only)
  *   "decode_force_generic"  1 = always use the shape-agnostic kernel
  *   "q4_force_generic"      1 = Q4_0 matmul always on the scalar kernel
  *   "q4_ksplit"             K slices of the Q4_0 MFMA matmul (0 = automatic)
@@ -371,6 +371,9 @@ long mlc_hip_decode_table_uploads(void);
  *                           batched scatters of its fp16 rows (or two batched scatters with
  *                           the same page ids) become one launch.
  *                           0 = each operator is launched when it is encoded
+ *   "decode_mfma"           1 (default) = the tile-balanced decode kernel does a tile's arithmetic
+ *                           on the matrix pipe where the shape allows it (4 to 16 query heads per
+ *                           KV head in 4 waves, fp16 softmax weights); 0 = on the vector pipe
  *   "prefill_stages"        2, 4, 6 or 8 K/V tiles staged in LDS by the prefill kernel (0 = automatic)
  *   "prefill_rows64"        1 (default) = heads/kv_heads up to 4 run the prefill kernel with 64
  *                           chunk rows per wave; 0 = the kernel with 32 rows per wave for every

@@ -34,7 +34,7 @@ namespace mlc_hip {
 MLC_DECL(64, 1) MLC_DECL(64, 2) MLC_DECL(64, 4) MLC_DECL(64, 8)
 MLC_DECL(128, 1) MLC_DECL(128, 2) MLC_DECL(128, 4) MLC_DECL(128, 8)
 #undef MLC_DECL
-#define MLC_DECL(d, h) bool launch_decode_stream_##d##_##h(int, int, bool, const StreamArgs&, unsigned, size_t, hipStream_t);
+#define MLC_DECL(d, h) bool launch_decode_stream_##d##_##h(int, int, int, const StreamArgs&, unsigned, size_t, hipStream_t);
 MLC_DECL(64, 1) MLC_DECL(64, 2) MLC_DECL(64, 4) MLC_DECL(64, 8)
 MLC_DECL(128, 1) MLC_DECL(128, 2) MLC_DECL(128, 4) MLC_DECL(128, 8)
 #undef MLC_DECL
@@ -224,6 +224,7 @@ struct Ctx {
     long opt_buffers = 0;                                      // LDS staging buffers per workgroup (1, 2; 0 = automatic)
     long opt_tile_rows = 1;                                    // wave rows that share an item's tiles
     long opt_prefill_stages = 0;                               // LDS pipeline depth of the prefill kernel (0 = automatic)
+    long opt_decode_mfma = 1;                                  // tile-balanced decode kernel: tile arithmetic on the matrix pipe
     long opt_prefill_rows64 = 1;                               // prefill: 64 chunk rows per wave where the GQA ratio allows it
     long opt_pv_fp16 = 1;                                      // softmax weights rounded to fp16 for P.V
     int last_launches = 0;
@@ -900,11 +901,22 @@ unsigned stream_grid(size_t G, size_t D, int nbuf, size_t dyn_lds) {
     return (unsigned)std::max<size_t>(W, 1);
 }
 
+// Arithmetic mode of the tile-balanced kernel: 0 fp32 softmax weights, 1 fp16 weights on the vector
+// pipe, 2 matrix pipe (4 waves per workgroup, at most 16 heads per KV head).
+int stream_pv_mode(int hpw, int nw) {
+    if (!g.opt_pv_fp16) return 0;
+    return (g.opt_decode_mfma && nw == 4 && hpw * nw <= 16) ? 2 : 1;
+}
+const char* stream_pv_name(int hpw, int nw) {
+    const int m = stream_pv_mode(hpw, nw);
+    return m == 2 ? "mfma" : m == 1 ? "pv16" : "pv32";
+}
+
 bool launch_stream_variant(size_t D, int hpw, int nw, int nbuf, const StreamArgs& a, unsigned n_wg, size_t dyn_lds,
                            hipStream_t stream) {
-    const bool pv16 = g.opt_pv_fp16 != 0;
+    const int pvm = stream_pv_mode(hpw, nw);
 #define MLC_CASE(d, h) \
-    if (D == d && hpw == h) return launch_decode_stream_##d##_##h(nw, nbuf, pv16, a, n_wg, dyn_lds, stream);
+    if (D == d && hpw == h) return launch_decode_stream_##d##_##h(nw, nbuf, pvm, a, n_wg, dyn_lds, stream);
     MLC_CASE(64, 1) MLC_CASE(64, 2) MLC_CASE(64, 4) MLC_CASE(64, 8)
     MLC_CASE(128, 1) MLC_CASE(128, 2) MLC_CASE(128, 4) MLC_CASE(128, 8)
 #undef MLC_CASE
@@ -1213,7 +1225,7 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
         }
         g.last_items = (int)std::min<uint64_t>(n_wg, total_tiles);
         std::snprintf(g.last_kernel, sizeof g.last_kernel, "stream<%zu,%d,%d,%s,%s,%d>", head_dim, s_hpw, s_nw,
-                      g.opt_pv_fp16 ? "pv16" : "pv32", batch <= 64 ? "regs" : "lds", nbuf);
+                      stream_pv_name(s_hpw, s_nw), batch <= 64 ? "regs" : "lds", nbuf);
         if (carries_kv) {
             g.kv.active = false;
             ++g.kv_fused;
@@ -1355,7 +1367,7 @@ int mlc_hip_paged_attn_decode_noalloc(const void* q, const void* k_pages, const 
     HIP_OK(hipGetLastError());
     g.last_items = (int)std::min<uint64_t>(n_wg, total_tiles);
     std::snprintf(g.last_kernel, sizeof g.last_kernel, "stream<%zu,%d,%d,%s,%s,%d>", head_dim, hpw, nw,
-                  g.opt_pv_fp16 ? "pv16" : "pv32", batch <= 64 ? "regs" : "lds", nbuf);
+                  stream_pv_name(hpw, nw), batch <= 64 ? "regs" : "lds", nbuf);
     g.last_launches = 1;
     return 1;
 }
@@ -2418,6 +2430,11 @@ int mlc_hip_set_option(const char* name, long value) {
     if (!std::strcmp(name, "prefill_stages")) {
         if (value != 0 && value != 2 && value != 4 && value != 6 && value != 8) return 0;
         g.opt_prefill_stages = value;
+        return 1;
+    }
+    if (!std::strcmp(name, "decode_mfma")) {
+        if (value != 0 && value != 1) return 0;
+        g.opt_decode_mfma = value;
         return 1;
     }
     if (!std::strcmp(name, "prefill_rows64")) {

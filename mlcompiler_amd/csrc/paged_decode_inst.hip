@@ -51,36 +51,44 @@ bool MLC_CAT(MLC_D, MLC_HPW)(int nw, int ns, int nbuf, bool pv16, const DecodeAr
 
 namespace {
 template <int NW, bool SMALL, int NBUF>
-void launch_stream_pv(bool pv16, const StreamArgs& a, unsigned n_wg, size_t dyn_lds, hipStream_t stream) {
+void launch_stream_pv(int pvm, const StreamArgs& a, unsigned n_wg, size_t dyn_lds, hipStream_t stream) {
     const dim3 grid(n_wg), block(64 * NW);
-    if (pv16)
-        hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, true, SMALL, NBUF>), grid, block, dyn_lds, stream, a);
+    if constexpr (NW == 4 && MLC_HPW * NW <= 16) {
+        if (pvm == 2) {
+            hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, 2, SMALL, NBUF>), grid, block, dyn_lds, stream, a);
+            return;
+        }
+    }
+    if (pvm)
+        hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, 1, SMALL, NBUF>), grid, block, dyn_lds, stream, a);
     else
-        hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, false, SMALL, NBUF>), grid, block, dyn_lds, stream, a);
+        hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, 0, SMALL, NBUF>), grid, block, dyn_lds, stream, a);
 }
 template <int NW>
-bool launch_stream(int nbuf, bool pv16, const StreamArgs& a, unsigned n_wg, size_t dyn_lds, hipStream_t stream) {
+bool launch_stream(int nbuf, int pvm, const StreamArgs& a, unsigned n_wg, size_t dyn_lds, hipStream_t stream) {
     // at most 64 requests: the variant that keeps the per-request figures in registers; larger
     // batches keep them in dynamic LDS, next to two or three stages
     if (a.batch <= 64) {
-        if (nbuf == 2) launch_stream_pv<NW, true, 2>(pv16, a, n_wg, 0, stream);
-        else if (nbuf == 3) launch_stream_pv<NW, true, 3>(pv16, a, n_wg, 0, stream);
-        else launch_stream_pv<NW, true, 4>(pv16, a, n_wg, 0, stream);
+        if (nbuf == 2) launch_stream_pv<NW, true, 2>(pvm, a, n_wg, 0, stream);
+        else if (nbuf == 3) launch_stream_pv<NW, true, 3>(pvm, a, n_wg, 0, stream);
+        else launch_stream_pv<NW, true, 4>(pvm, a, n_wg, 0, stream);
     } else {
-        if (nbuf == 2) launch_stream_pv<NW, false, 2>(pv16, a, n_wg, dyn_lds, stream);
-        else launch_stream_pv<NW, false, 3>(pv16, a, n_wg, dyn_lds, stream);
+        if (nbuf == 2) launch_stream_pv<NW, false, 2>(pvm, a, n_wg, dyn_lds, stream);
+        else launch_stream_pv<NW, false, 3>(pvm, a, n_wg, dyn_lds, stream);
     }
     return true;
 }
 }  // namespace
 
 // Tile-balanced kernel: nw = waves over the GQA group, nbuf = LDS stages (large batches: at most 3),
-// n_wg = grid size; false for an unbuilt combination.
-bool MLC_SCAT(MLC_D, MLC_HPW)(int nw, int nbuf, bool pv16, const StreamArgs& a, unsigned n_wg, size_t dyn_lds, hipStream_t stream) {
+// pvm = arithmetic mode (0 fp32 weights, 1 fp16 weights on the vector pipe, 2 matrix pipe where
+// built: 4 waves and at most 16 heads per KV head, else mode 1), n_wg = grid size; false for an
+// unbuilt combination.
+bool MLC_SCAT(MLC_D, MLC_HPW)(int nw, int nbuf, int pvm, const StreamArgs& a, unsigned n_wg, size_t dyn_lds, hipStream_t stream) {
     switch (nw) {
-        case 1: return launch_stream<1>(nbuf, pv16, a, n_wg, dyn_lds, stream);
-        case 2: return launch_stream<2>(nbuf, pv16, a, n_wg, dyn_lds, stream);
-        case 4: return launch_stream<4>(nbuf, pv16, a, n_wg, dyn_lds, stream);
+        case 1: return launch_stream<1>(nbuf, pvm, a, n_wg, dyn_lds, stream);
+        case 2: return launch_stream<2>(nbuf, pvm, a, n_wg, dyn_lds, stream);
+        case 4: return launch_stream<4>(nbuf, pvm, a, n_wg, dyn_lds, stream);
         default: return false;
     }
 }

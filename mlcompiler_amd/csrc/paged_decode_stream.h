@@ -129,8 +129,18 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t x) {
 // SMALL: at most 64 requests; lane r of every wave holds request r's figures in registers and
 // nothing goes through LDS.  Otherwise they are kept in (dynamic) LDS.
 // NBUF: tiles staged in LDS per workgroup; tile k + NBUF - 1 is requested while tile k is consumed.
-template <int D, int HPW, int NW, bool PV16, bool SMALL, int NBUF>
+// PVM: how a tile's arithmetic is done.  0: on the vector pipe with fp32 softmax weights; 1: on the
+// vector pipe, weights rounded to fp16 for P.V (v_dot2); 2: on the matrix pipe (4 waves, at most
+// 16 query heads per KV head): every wave takes a quarter of the tile's tokens for all heads of
+// the group, S^T = K.q^T with v_mfma_f32_16x16x32_f16 (q as the sum of two fp16 numbers, so that
+// the products are as exact as with fp32 q), O^T += V^T.P^T with v_mfma_f32_16x16x16_f16 (fp16
+// weights as in mode 1), V^T through the transposing LDS read; the waves' results are combined
+// through LDS where a pair of (request, KV head) ends.
+template <int D, int HPW, int NW, int PVM, bool SMALL, int NBUF>
 __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const StreamArgs a) {
+    constexpr bool PV16 = PVM == 1;
+    constexpr bool MF = PVM == 2;
+    static_assert(!MF || (NW == 4 && HPW * NW <= 16), "matrix-pipe mode: 4 waves, at most 16 heads per KV head");
     static_assert(NBUF >= 2 && NBUF <= 4, "2 to 4 stages");
     static_assert(D == 64 || D == 128, "head_dim 64 and 128");
     static_assert(NW == 1 || NW == 2 || NW == 4, "waves per GQA group");
@@ -143,7 +153,13 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     constexpr int TILE_BYTES = TT * D * 2;  // one tensor, one KV head: 8 KiB
     constexpr int LPW = 16 / NW;            // tile-load instructions per wave and tile (8 K + 8 V in all)
     constexpr int STAGE_BYTES = 2 * TILE_BYTES;
+    constexpr int TW = TT / NW;             // matrix-pipe mode: tokens of a tile per wave (16 or 8)
+    constexpr int KST = D / 32;             // ... MFMA steps over head_dim for S^T
+    constexpr int DB = D / 16;              // ... 16-row blocks of O^T
     __shared__ __attribute__((aligned(16))) unsigned char stages[NBUF * STAGE_BYTES];
+    // matrix-pipe mode: the waves' (o, m, l) of a pair, combined where the pair ends
+    __shared__ __attribute__((aligned(16))) float comb_o[MF ? NW * G * D : 4];
+    __shared__ float comb_ml[MF ? 2 * NW * G : 2];
     extern __shared__ uint32_t s_meta[];
     const uint32_t B = a.batch;
     uint32_t* s_start = s_meta;            // [B + 1] tiles of the requests before r (one KV head)
@@ -365,9 +381,51 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         sd_barrier();
     }
 
+    // matrix-pipe mode: lane coordinates of the 16x16 MFMA layouts, the q operand (B of S^T =
+    // K.q^T: column n16 = head of the group, dims 8*g4 .. +7 of every 32-dim step) as the sum of
+    // two fp16 numbers, and the LDS offsets of this lane's K and V^T operand reads inside a tile.
+    // K rows are stored with their 16-byte chunks permuted by chunk ^ ((row / (128 / D)) % CPR), V
+    // rows by chunk ^ 2*((row % 4) / (128 / D)) (see issue_tile): the 16 lanes that the hardware
+    // serves together then hit 16 different bank groups.
+    const int n16 = lane % 16, g4 = lane / 16;
+    typedef _Float16 sd_half4 __attribute__((ext_vector_type(4)));
+    typedef float sd_f4 __attribute__((ext_vector_type(4)));
+    half8_t qh[MF ? KST : 1], ql[MF ? KST : 1];
+    uint32_t mf_k_off[MF ? KST : 1], mf_v_off[MF ? DB : 1];
+    if constexpr (MF) {
+        constexpr int RPB = 128 / D;   // rows per 256 bytes
+        const uint32_t krow = (uint32_t)(wave * TW + n16 % TW);
+#pragma unroll
+        for (int ks = 0; ks < KST; ++ks)
+            mf_k_off[ks] = krow * (D * 2) + ((((uint32_t)(ks * 4 + g4)) ^ ((krow / RPB) % CPR)) * 16);
+        const uint32_t e4 = (uint32_t)n16 / 4, q4 = (uint32_t)n16 % 4;
+        const uint32_t vrow = (uint32_t)(wave * TW + (4 * g4 + (int)e4) % TW);
+        const uint32_t fv = 2u * ((vrow % 4u) / RPB);
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+            mf_v_off[b] = TILE_BYTES + vrow * (D * 2) + (((uint32_t)(2 * b) + q4 / 2) ^ fv) * 16 + (q4 % 2) * 8;
+    }
     // q of this wave's heads, dims c*8 .. c*8+7, scaled
     float qv[HPW][8];
     auto load_q = [&](const Cursor& cu) {
+        if constexpr (MF) {
+            const int hcol = n16 < G ? n16 : G - 1;
+            const float* qb = a.q + ((size_t)cu.r * a.num_heads + cu.kvh * G + hcol) * D + 8 * g4;
+#pragma unroll
+            for (int ks = 0; ks < KST; ++ks) {
+                const float4 x0 = *reinterpret_cast<const float4*>(qb + 32 * ks);
+                const float4 x1 = *reinterpret_cast<const float4*>(qb + 32 * ks + 4);
+                const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float v = n16 < G ? x[i] * a.scale_log2e : 0.f;
+                    const _Float16 hi = (_Float16)v;
+                    qh[ks][i] = hi;
+                    ql[ks][i] = (_Float16)(v - (float)hi);
+                }
+            }
+            return;
+        }
         const float* qbase = a.q + ((size_t)cu.r * a.num_heads + cu.kvh * G + hg * HPW) * D + c * 8;
 #pragma unroll
         for (int h = 0; h < HPW; ++h) {
@@ -391,23 +449,34 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         const uint32_t slot0 = tile_start % a.page_size;
         const uint32_t last = cu.lim - 1u - tile_start;
         const size_t row0 = ((size_t)page_id * a.page_size + slot0) * row_u4 + cu.kvh * CPR + c;
-        constexpr int PARTS = (NW == 1) ? 2 : 1;
-        constexpr int JN = (NW == 4) ? 4 : 8;
+        // (matrix-pipe mode: every wave loads exactly the rows it consumes, two loads of K and two
+        // of V, so that no wave ever waits for another one's loads)
+        constexpr int PARTS = (NW == 1 || MF) ? 2 : 1;
+        constexpr int JN = MF ? 2 : (NW == 4) ? 4 : 8;
 #pragma unroll
         for (int p = 0; p < PARTS; ++p) {
-            const int tensor = (NW == 1) ? p : (NW == 2 ? hg : hg / 2);
-            const int j0 = (NW == 4) ? (hg % 2) * 4 : 0;
+            const int tensor = (NW == 1 || MF) ? p : (NW == 2 ? hg : hg / 2);
+            const int j0 = MF ? 2 * hg : (NW == 4) ? (hg % 2) * 4 : 0;
             const uint4* base = (tensor ? a.v_pages : a.k_pages) + row0;
             const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)(stages_lds + slot * STAGE_BYTES + tensor * TILE_BYTES));
 #pragma unroll
             for (int jj = 0; jj < JN; ++jj) {
                 const int j = j0 + jj;
                 uint32_t tr = (uint32_t)((j ^ gsw) * RPI + r_l);
+                const uint4* src = base;
+                if constexpr (MF) {
+                    // rows in order, chunks permuted (see above): LDS chunk c of row tr holds the
+                    // row's chunk c ^ f(tr)
+                    constexpr int RPB = 128 / D;
+                    tr = (uint32_t)(j * RPI + r_l);
+                    const uint32_t f = tensor ? 2u * ((tr % 4u) / RPB) : (tr / RPB) % CPR;
+                    src = base - c + ((uint32_t)c ^ f);
+                }
                 tr = tr < last ? tr : last;
 #ifndef MLC_NO_LOADS
-                sd_g2lds16(base + (size_t)tr * row_u4, dst + j * 1024);
+                sd_g2lds16(src + (size_t)tr * row_u4, dst + j * 1024);
 #else
-                asm volatile("" ::"v"(base + (size_t)tr * row_u4), "s"(dst + j * 1024));
+                asm volatile("" ::"v"(src + (size_t)tr * row_u4), "s"(dst + j * 1024));
 #endif
             }
         }
@@ -424,7 +493,18 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
 
     float acc[HPW][8];
     float m_ref[HPW], l_sum[HPW];
+    // matrix-pipe mode: O^T of this wave's tokens (lane: head n16, dims 16*b + 4*g4 .. +3), the
+    // reference of column n16 (the same in its four lanes) and this lane's part of the row sum
+    sd_f4 mf_o[MF ? DB : 1];
+    float mf_m = kNegBig, mf_l = 0.f;
     auto reset_state = [&]() {
+        if constexpr (MF) {
+            mf_m = kNegBig;
+            mf_l = 0.f;
+#pragma unroll
+            for (int b = 0; b < DB; ++b) mf_o[b] = sd_f4{0.f, 0.f, 0.f, 0.f};
+            return;
+        }
 #pragma unroll
         for (int h = 0; h < HPW; ++h) {
             m_ref[h] = kNegBig;
@@ -439,6 +519,51 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     auto consume_tile = [&](uint32_t slot, uint32_t t, uint32_t lim) {
         const unsigned char* cur = stages + (size_t)slot * STAGE_BYTES;
         const uint32_t tile_start = t * TT;
+        if constexpr (MF) {
+            typedef __fp16 sd_fp16x4 __attribute__((vector_size(8)));
+            half8_t ka[KST];
+#pragma unroll
+            for (int ks = 0; ks < KST; ++ks) ka[ks] = *reinterpret_cast<const half8_t*>(cur + mf_k_off[ks]);
+            sd_half4 va[DB];
+#pragma unroll
+            for (int b = 0; b < DB; ++b)
+                va[b] = __builtin_bit_cast(sd_half4, __builtin_amdgcn_ds_read_tr16_b64_v4f16(
+                    (sd_fp16x4 __attribute__((address_space(3)))*)(cur + mf_v_off[b])));
+            sd_f4 s4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KST; ++ks) {
+                s4 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[ks], qh[ks], s4, 0, 0, 0);
+                s4 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[ks], ql[ks], s4, 0, 0, 0);
+            }
+            // lane (n16, g4) holds the scores of head n16 for the wave's keys 4*g4 .. 4*g4+3
+            const uint32_t key0 = tile_start + (uint32_t)(wave * TW + 4 * g4);
+            float mloc = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const bool visible = (4 * g4 + i < TW) && key0 + (uint32_t)i < lim;
+                s4[i] = visible ? s4[i] : -INFINITY;
+                mloc = max_nn(mloc, s4[i]);
+            }
+            if (__any(mloc > mf_m + kLazyTau)) {
+                float mcol = max_nn(mloc, __shfl_xor(mloc, 16));
+                mcol = max_nn(mcol, __shfl_xor(mcol, 32));
+                const float m_new = max_nn(mf_m, mcol);
+                const float alpha = fast_exp2(mf_m - m_new);
+                mf_m = m_new;
+                mf_l *= alpha;
+#pragma unroll
+                for (int b = 0; b < DB; ++b) mf_o[b] *= alpha;
+            }
+            sd_half4 pb;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                pb[i] = (_Float16)fast_exp2(s4[i] - mf_m);
+                mf_l += (float)pb[i];
+            }
+#pragma unroll
+            for (int b = 0; b < DB; ++b) mf_o[b] = __builtin_amdgcn_mfma_f32_16x16x16f16(va[b], pb, mf_o[b], 0, 0, 0);
+            return;
+        }
         const uint4* kl = reinterpret_cast<const uint4*>(cur) + lane;
         const uint4* vl = kl + TILE_BYTES / 16;
         // All sixteen LDS reads of the tile are requested before anything is computed, K first
@@ -600,6 +725,52 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     // partner, the last step of head_dim 64 goes over lane ^ 8).  Lane (r, c) ends up with
     // dims c*8 + r*HPK + kk (kk < HPK) of every head, summed over all tokens of the wave.
     auto reduce_rows = [&](float (&o_un)[OPL], float (&m_all)[HPW], float (&l_all)[HPW]) {
+        if constexpr (MF) {
+            // every wave leaves its (o, m, l) of all heads of the group in LDS; wave hg then
+            // combines the four for its own heads, in the lane layout the code below expects
+            // (lane (r, c): dims c*8 + r*HPK + kk).  The sums run over the waves in a fixed
+            // order in every lane, so l does not depend on the lane it is read from.
+            float lt = mf_l + __shfl_xor(mf_l, 16);
+            lt += __shfl_xor(lt, 32);
+            if (n16 < G) {
+#pragma unroll
+                for (int b = 0; b < DB; ++b)
+                    *reinterpret_cast<sd_f4*>(&comb_o[((size_t)wave * G + n16) * D + b * 16 + 4 * g4]) = mf_o[b];
+                if (g4 == 0) {
+                    comb_ml[wave * G + n16] = mf_m;
+                    comb_ml[NW * G + wave * G + n16] = lt;
+                }
+            }
+            sd_barrier();
+#pragma unroll
+            for (int h = 0; h < HPW; ++h) {
+                const int hh = hg * HPW + h;
+                float mw[NW], m = kNegBig;
+#pragma unroll
+                for (int w2 = 0; w2 < NW; ++w2) {
+                    mw[w2] = comb_ml[w2 * G + hh];
+                    m = max_nn(m, mw[w2]);
+                }
+                m_all[h] = m;
+                float l = 0.f, o[HPK];
+#pragma unroll
+                for (int kk = 0; kk < HPK; ++kk) o[kk] = 0.f;
+#pragma unroll
+                for (int w2 = 0; w2 < NW; ++w2) {
+                    const float wgt = fast_exp2(mw[w2] - m);
+                    l += comb_ml[NW * G + w2 * G + hh] * wgt;
+#pragma unroll
+                    for (int kk = 0; kk < HPK; ++kk)
+                        o[kk] += comb_o[((size_t)w2 * G + hh) * D + c * 8 + r_l * HPK + kk] * wgt;
+                }
+                l_all[h] = l;
+#pragma unroll
+                for (int kk = 0; kk < HPK; ++kk) o_un[h * HPK + kk] = o[kk];
+            }
+            sd_barrier();   // the waves run on their own between pairs: nobody writes the next pair's
+                            // figures before everybody has read these
+            return;
+        }
 #pragma unroll
         for (int h = 0; h < HPW; ++h) {
             float m = m_ref[h];
@@ -780,7 +951,9 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         if (k < 6) MLC_PROBE_TILE(8 + 3 * k);
         if (drain) sd_wait_vmcnt<0>(); else wait_tile(issued - k - 1u);
         drain = false;
-        sd_barrier();   // ... and everyone's; everyone has left tile k-1, whose stage is free
+        // ... and everyone's; everyone has left tile k-1, whose stage is free (matrix-pipe mode: a
+        // wave loads, reads and overwrites only its own rows of a stage, no barrier)
+        if constexpr (!MF) sd_barrier();
         if (k < 6) MLC_PROBE_TILE(9 + 3 * k);
         if (k == 0) MLC_PROBE(3);
         // one tile went out up front; from the first step on the stream runs NBUF - 1 tiles ahead

@@ -10,13 +10,17 @@ from paged_cases import (DeviceCase, assert_parity, baseline_config, make_case, 
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(params=["balanced", "planned"], autouse=True)
+@pytest.fixture(params=["balanced", "balanced-vector", "planned"], autouse=True)
 def decode_kernel(exe, request):
     """Every test runs on both tiled decode kernels: the tile-balanced one (fixed grid, work
-    derived from the tables in the kernel; the default) and the planned one (host-built items)."""
+    derived from the tables in the kernel; the default), with the tile arithmetic on the matrix
+    pipe where the shape allows it (the default) and on the vector pipe, and the planned one
+    (host-built items)."""
     assert exe.setOption("decode_kernel", 1 if request.param == "planned" else 0)
-    yield request.param
+    assert exe.setOption("decode_mfma", 0 if request.param == "balanced-vector" else 1)
+    yield "balanced" if request.param == "balanced-vector" else request.param
     exe.setOption("decode_kernel", 0)
+    exe.setOption("decode_mfma", 1)
 
 
 # how each kernel's split of the work is varied: items aimed for / exact grid size
