@@ -608,6 +608,16 @@ def run_decode(args, name: str, steps: int, warmup: int, cpu_budget: float, full
         assert exe.setOption("decode_pv_fp16", 1)
         r["pv_fp32_us"] = ev32 / steps * 1e3
 
+        # ---- products on the vector pipe (decode_mfma = 0), fp16 softmax weights as in the default
+        if any(kv.startswith("decode_mfma=") for kv in args.opt):
+            r["vector_pipe_us"] = float("nan")  # the caller chose the mode: nothing to compare
+        else:
+            assert exe.setOption("decode_mfma", 0)
+            native_loop(n_layers)
+            evv, _ = native_loop(steps)
+            assert exe.setOption("decode_mfma", 1)
+            r["vector_pipe_us"] = evv / steps * 1e3
+
         # ---- a plain streaming read of the same number of bytes from the same pools
         each = min(c.kv_bytes // 2 // 16 * 16, pool_bytes)
         ms_r = C.c_float()
@@ -831,7 +841,8 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": "f32 accumulate and output (fp16 K/V storage; products on f16 MFMA: fp32 q enters as the sum of "
                  "two fp16 numbers, softmax weights are rounded to fp16 for P.V; option decode_pv_fp16 = 0: fp32 "
-                 "weights on the vector pipe, us_per_layer_pv_fp32 is its time)",
+                 "weights on the vector pipe, us_per_layer_pv_fp32 is its time; option decode_mfma = 0: every product on the "
+                 "vector pipe with fp32 q, us_per_layer_vector_pipe is its time)",
         "data": "synthetic",
         "config": {
             "workload": workload_text(c, r["n_layers"]),
@@ -844,6 +855,7 @@ def main() -> int:
             "kernel": r["kernel"],
             "work_items": r["items"],
             "us_per_layer_pv_fp32": round(r["pv_fp32_us"], 3),
+            "us_per_layer_vector_pipe": None if r["vector_pipe_us"] != r["vector_pipe_us"] else round(r["vector_pipe_us"], 3),
             "us_per_layer_tables_change": r["tables_change_us"],
             "us_per_layer_page_table_changes": r["page_table_changes_us"],
             "single_launch_us": r["single_us"],

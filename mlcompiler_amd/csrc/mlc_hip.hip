@@ -875,11 +875,11 @@ bool stream_variant(size_t G, size_t D, int* hpw_out, int* nw_out) {
     return true;
 }
 
-// LDS stages of the tile-balanced kernel.  Two by default: swept over 2..4 stages and 2..5
-// workgroups per CU on MI355X, two stages and two workgroups per CU were fastest at 38 MB and at
-// 1.2 GB of KV per launch (deeper stages only delay the first tile of every workgroup: the
-// kernel's steady state is bound by VALU issue, not by loads in flight).  Batches above 64
-// requests keep their per-request figures in LDS as well and take three stages at most.
+// LDS stages of the tile-balanced kernel.  Two by default: swept over 2..4 stages and 1..5
+// workgroups per CU on MI355X, in both arithmetic modes, two stages and two workgroups per CU
+// were fastest at 38 MB and at 1.2 GB of KV per launch (deeper stages only delay the first tile
+// of every workgroup).  Batches above 64 requests keep their per-request figures in LDS as well
+// and take three stages at most.
 int stream_stages(size_t batch) {
     const int most = batch <= 64 ? 4 : 3;
     int nbuf = 2;
@@ -890,7 +890,8 @@ int stream_stages(size_t batch) {
 // Grid of the tile-balanced kernel: as many workgroups as stay resident (LDS decides), within
 // what the scratch array holds.
 unsigned stream_grid(size_t G, size_t D, int nbuf, size_t dyn_lds) {
-    const size_t lds = (size_t)stream_static_lds_bytes(nbuf) + dyn_lds;
+    const bool matrix_pipe = g.opt_pv_fp16 && g.opt_decode_mfma && G >= 4 && G <= 16;
+    const size_t lds = stream_static_lds_bytes(nbuf, G, D, matrix_pipe) + dyn_lds;
     size_t per_cu = std::max<size_t>(1, std::min<size_t>(160 * 1024 / lds, 2));
     if (g.opt_wgs_per_cu > 0) per_cu = (size_t)g.opt_wgs_per_cu;
     size_t W = (size_t)g.n_cu * per_cu;

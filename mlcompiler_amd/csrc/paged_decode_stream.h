@@ -64,8 +64,11 @@ struct StreamArgs {
 };
 static_assert(sizeof(StreamArgs) <= 4096, "kernel arguments are limited to 4 KiB");
 
-// LDS of one workgroup: NBUF stages of one K tile and one V tile (8 KiB each)
-constexpr int stream_static_lds_bytes(int NBUF) { return NBUF * 2 * 8192; }
+// LDS of one workgroup: NBUF stages of one K tile and one V tile (8 KiB each), and in matrix-pipe
+// mode (four waves, G query heads per KV head) the waves' results of a pair
+constexpr size_t stream_static_lds_bytes(int NBUF, size_t G, size_t D, bool matrix_pipe) {
+    return (size_t)NBUF * 2 * 8192 + (matrix_pipe ? (4 * G * D + 2 * 4 * G) * 4 : 24);
+}
 // dynamic LDS: tile prefix [B + 1], visible lengths [B], page-table offsets [B]
 inline size_t stream_dynamic_lds_bytes(size_t batch) { return (3 * batch + 1) * 4; }
 
