@@ -362,6 +362,9 @@ long mlc_hip_decode_table_uploads(void);
  *   "decode_force_generic"  1 = always use the shape-agnostic kernel
  *   "q4_force_generic"      1 = Q4_0 matmul always on the scalar kernel
  *   "q4_ksplit"             K slices of the Q4_0 MFMA matmul (0 = automatic)
+ *   "q4_int_operand"        1 (default) = the Q4_0 MFMA matmul multiplies the integers q - 8 and
+ *                           applies the block scale to each block's sum in fp32; 0 = it
+ *                           multiplies d * (q - 8) as an exact pair of fp16 numbers
  *   "fuse_row_ops"          1 (default) = row-local operators encoded back to back in a pass
  *                           (sum of matmul K slices, add, RMSNorm, gate/up SiLU, the fp16 split
  *                           of the next matmul's input) are collected and launched as one

@@ -154,6 +154,7 @@ struct Ctx {
     };
     std::unordered_map<std::string, Q6KWeight> q6k_weights;
     long opt_q4_force_generic = 0;
+    long opt_q4_int_operand = 1;  // Q4_0 matrix-core kernel: integer weights as operand, d applied per block
     long opt_q4_ksplit = 0;  // 0 = automatic
     MetaSlot ring[8];
     int ring_next = 0;
@@ -373,6 +374,22 @@ constexpr size_t kRowMaxLen = 16384;  // row_program_kernel: 8 groups of 8 eleme
 
 bool row_len_ok(size_t len) { return len > 0 && len % 8 == 0 && len <= kRowMaxLen; }
 
+// The matrix-core Q4_0 kernel for nbt batch tiles of 32 and rt row tiles per workgroup; option
+// q4_int_operand picks the arithmetic (see q4_matmul_kernels.h).
+void launch_q4_mfma(int nbt, int rt, dim3 grid, const Q4Args& a) {
+#define MLC_Q4(NBT, RT, WAVES)                                                                              \
+    if (g.opt_q4_int_operand)                                                                               \
+        hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<NBT, RT, WAVES, true>), grid, dim3(WAVES * 64), 0, g.stream, a); \
+    else                                                                                                    \
+        hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<NBT, RT, WAVES, false>), grid, dim3(WAVES * 64), 0, g.stream, a)
+    if (nbt == 1) {
+        if (rt == 1) { MLC_Q4(1, 1, 16); } else { MLC_Q4(1, 2, 16); }
+    } else {
+        if (rt == 1) { MLC_Q4(2, 1, 8); } else { MLC_Q4(2, 2, 8); }
+    }
+#undef MLC_Q4
+}
+
 // Launches the held-back matmul, with the split + RoPE + cast of its output as epilogue when
 // `rope` is given.
 int settle_gemm(const RopeArgs* rope = nullptr) {
@@ -386,13 +403,7 @@ int settle_gemm(const RopeArgs* rope = nullptr) {
         ++g.gemm_rope_fused;
     }
     const dim3 grid(m.grid_x, 1);
-    if (m.nbt == 1) {
-        if (m.rt == 1) hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<1, 1, 16>), grid, dim3(1024), 0, g.stream, a);
-        else hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<1, 2, 16>), grid, dim3(1024), 0, g.stream, a);
-    } else {
-        if (m.rt == 1) hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<2, 1, 8>), grid, dim3(512), 0, g.stream, a);
-        else hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<2, 2, 8>), grid, dim3(512), 0, g.stream, a);
-    }
+    launch_q4_mfma(m.nbt, m.rt, grid, a);
     HIP_OK(hipGetLastError());
     return 1;
 }
@@ -1972,13 +1983,7 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
             return finish(sync);
         }
         const dim3 grid((unsigned)wgs, (unsigned)ksplit);
-        if (bpad == 32) {
-            if (row_tiles == 1) hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<1, 1, 16>), grid, dim3(1024), 0, g.stream, a);
-            else hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<1, 2, 16>), grid, dim3(1024), 0, g.stream, a);
-        } else {
-            if (row_tiles == 1) hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<2, 1, 8>), grid, dim3(512), 0, g.stream, a);
-            else hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<2, 2, 8>), grid, dim3(512), 0, g.stream, a);
-        }
+        launch_q4_mfma(bpad == 32 ? 1 : 2, row_tiles, grid, a);
         if (ksplit > 1) {
             const uint32_t n = (uint32_t)(bn * rows);
             if (g.opt_fuse_rows && batch <= 64 && rows <= 2 * kRowMaxLen) {
@@ -2423,6 +2428,7 @@ int mlc_hip_set_option(const char* name, long value) {
     }
     if (!std::strcmp(name, "decode_pv_fp16")) { g.opt_pv_fp16 = value ? 1 : 0; return 1; }
     if (!std::strcmp(name, "q4_force_generic")) { g.opt_q4_force_generic = value ? 1 : 0; return 1; }
+    if (!std::strcmp(name, "q4_int_operand")) { g.opt_q4_int_operand = value ? 1 : 0; return 1; }
     if (!std::strcmp(name, "q4_ksplit")) {
         if (value < 0 || value > 64) return 0;
         g.opt_q4_ksplit = value;

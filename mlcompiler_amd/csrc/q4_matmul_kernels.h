@@ -216,7 +216,15 @@ __device__ __forceinline__ q4_half2 q4_pair(uint32_t bytes, uint32_t sel) {
 // waves' sums meet in LDS at the end.  With the whole K range in one workgroup (ksplit = 1) the
 // result goes straight to the output; K slices are only worth it when there are too few row
 // tiles to fill the chip and K is long.
-template <int NBT, int RT, int WAVES>
+//
+// IOP (integer operand): the matrix product runs over the exact integers q - 8 and the block
+// scale d is applied to each block's sum in fp32, acc += d * ((q-8).x_hi + (q-8).x_lo): four
+// MFMAs and 16 multiply-adds per (block, tile) instead of six MFMAs and the exact hi + lo split
+// of d * (q - 8).  The weights are then the B operand (a lane holds weight row lane % 32, so d
+// is one number per lane) and the activations the A operand; both fragment layouts serve either
+// role unchanged.  No product is rounded and no term is dropped: what remains is the fp32
+// rounding of the additions and of one multiply per block.
+template <int NBT, int RT, int WAVES, bool IOP>
 __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Args a) {
     constexpr int PF = WAVES >= 16 ? 2 : 4;  // blocks in flight per wave
     constexpr int PITCH = 65;                // floats per accumulator register in LDS (bank spread)
@@ -279,6 +287,35 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
                         a.xfrag + ((((size_t)t * ksteps + blk * 2 + ks) * 2 + p) * 64 + lane) * 8);
     };
     auto multiply = [&](const Block& k) __attribute__((always_inline)) {
+        if constexpr (IOP) {
+#pragma unroll
+            for (int r = 0; r < RT; ++r) {
+                const float d = k.real ? (float)k.d[r] : 0.0f;
+                q4_half8 w[2];
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks) {
+                    const uint32_t w0 = (ks ? (k.q[r].x >> 4) : k.q[r].x) & 0x0F0F0F0Fu;
+                    const uint32_t w1 = (ks ? (k.q[r].y >> 4) : k.q[r].y) & 0x0F0F0F0Fu;
+                    const q4_half2 n0 = q4_pair(w0, 0x04010400u), n1 = q4_pair(w0, 0x04030402u);
+                    const q4_half2 n2 = q4_pair(w1, 0x04010400u), n3 = q4_pair(w1, 0x04030402u);
+                    w[ks] = q4_half8{n0[0], n0[1], n1[0], n1[1], n2[0], n2[1], n3[0], n3[1]};
+                }
+#pragma unroll
+                for (int t = 0; t < NBT; ++t) {
+                    q4_float16 sblk;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) sblk[i] = 0.f;
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks) {
+                        sblk = __builtin_amdgcn_mfma_f32_32x32x16_f16(k.x[t][ks][0], w[ks], sblk, 0, 0, 0);
+                        sblk = __builtin_amdgcn_mfma_f32_32x32x16_f16(k.x[t][ks][1], w[ks], sblk, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) acc[r][t][i] = fmaf(d, sblk[i], acc[r][t][i]);
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int r = 0; r < RT; ++r) {
             const _Float16 d = k.real ? k.d[r] : (_Float16)0.0f;
@@ -327,7 +364,8 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
     }
 
     // ---- the waves' sums meet in LDS.  Accumulator layout: lane holds batch column l32 of the
-    // tile and, in register i, weight row (i/4)*8 + (lane/32)*4 + i%4 of the 32-row tile.
+    // tile and, in register i, weight row (i/4)*8 + (lane/32)*4 + i%4 of the 32-row tile (IOP:
+    // the other way round, lane holds the weight row and the register the batch column).
 #pragma unroll
     for (int r = 0; r < RT; ++r)
 #pragma unroll
@@ -337,13 +375,14 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
                 red[(((wave * RT + r) * NBT + t) * 16 + i) * PITCH + lane] = acc[r][t][i];
     __syncthreads();
     const uint32_t r = row / 32, rr = row % 32;
-    const uint32_t i = (rr / 8) * 4 + rr % 4, hf = (rr % 8) / 4;
     float* out = a.out + (size_t)slice * a.batch * a.rows;
 #pragma unroll
     for (uint32_t pass = 0; pass < PASSES; ++pass) {
         const uint32_t b = pass * COLS_PER_PASS + bsub;
         if (b >= a.batch) continue;
-        const uint32_t t = b / 32, ln = hf * 32 + b % 32;
+        const uint32_t t = b / 32;
+        const uint32_t in_reg = IOP ? b % 32 : rr, in_lane = IOP ? rr : b % 32;
+        const uint32_t i = (in_reg / 8) * 4 + in_reg % 4, ln = ((in_reg % 8) / 4) * 32 + in_lane;
         float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) sum += red[(((w * RT + r) * NBT + t) * 16 + i) * PITCH + ln];

@@ -4,9 +4,9 @@ the dequantised weights, through the C ABI.
 
 Tolerances, per output element, relative to A = sum_c |w_c * x_c| (the scale of the rounding
 errors of any summation): the fp32 sequential oracle itself is within about cols * 2^-24 * A of the
-exact value; the MFMA path splits operands into fp16 pairs with relative error 2^-22 per
-product and accumulates in fp32, so it must be within 4e-6 * A of the exact value and within
-2e-5 * A of the oracle.  The scalar fallback kernel is held to the same bounds."""
+exact value; the MFMA path multiplies the exact integers q - 8 with activations split into fp16
+pairs (relative error 2^-22 per product), accumulates in fp32 and applies the block scale in
+fp32, so it must be within 4e-6 * A of the exact value and within 2e-5 * A of the oracle.  The scalar fallback kernel is held to the same bounds."""
 import numpy as np
 import pytest
 
@@ -81,6 +81,19 @@ def test_q4_matmul_mfma_path(exe, rows, cols, batch):
     print(f"[q4 mfma] rows={rows} cols={cols} batch={batch}", flush=True)
     q, x, stride = make(rows, cols, batch, rows + cols + batch)
     got = run(exe, f"w_{rows}_{cols}", q, x, batch, rows, cols, stride)
+    check(got, q, x, batch, rows, cols, stride)
+
+
+@pytest.mark.parametrize("rows,cols,batch", [(2560, 2048, 32), (11264, 2048, 64), (128, 96, 33), (4096, 14336, 3)])
+def test_q4_matmul_weights_as_fp16_pairs(exe, rows, cols, batch):
+    # q4_int_operand = 0: the earlier arithmetic (d * (q - 8) as an exact fp16 pair, three MFMAs per
+    # k step) stays selectable and is held to the same bounds
+    q, x, stride = make(rows, cols, batch, rows + cols + batch + 1)
+    assert exe.setOption("q4_int_operand", 0)
+    try:
+        got = run(exe, f"p_{rows}_{cols}", q, x, batch, rows, cols, stride)
+    finally:
+        assert exe.setOption("q4_int_operand", 1)
     check(got, q, x, batch, rows, cols, stride)
 
 
