@@ -464,8 +464,13 @@ __global__ __launch_bounds__(256) void paged_prefill_mfma64_kernel(const Prefill
     constexpr int CHUNKS = kPfKeys * CPR;            // 16-byte chunks per tile and tensor
     constexpr int LPT = CHUNKS / NT;                 // chunks of each tensor per thread and tile
     static_assert(CHUNKS % NT == 0 && LPT >= 1, "whole chunks per thread");
-    constexpr int AHEAD = NST - 1;                   // tiles issued ahead of the one in work
-    constexpr int KEEP = (AHEAD - 3) * 2 * LPT;      // own loads that may stay in flight
+    // Eight stages: the waves meet only after every second step.  A step reads V(tile) and
+    // K(tile + 2), so what the two steps behind a barrier read (up to tile + 4 of the barrier's
+    // step) must have landed there, and what they load (tiles + 6, + 7) replaces the tiles of
+    // the two steps before the barrier.
+    constexpr bool B2 = NST == 8;
+    constexpr int AHEAD = B2 ? NST - 2 : NST - 1;    // tiles issued ahead of the one in work
+    constexpr int KEEP = (AHEAD - (B2 ? 4 : 3)) * 2 * LPT;  // own loads that may stay in flight
     constexpr int SLOTS_S = 2 * KSTEPS;              // MFMAs of S per step
     constexpr int SLOTS_PV = 2 * MB;                 // MFMAs of P.V per step and half
     static_assert(SLOTS_PV == KSTEPS, "one K operand read per slot of the first P.V half");
@@ -821,8 +826,10 @@ __global__ __launch_bounds__(256) void paged_prefill_mfma64_kernel(const Prefill
             for (int t = 0; t < 2; ++t) pw_cur[hb][t] = pw_next[hb][t];
         }
         tile_advance();
-        pf_wait_vmcnt<KEEP>();
-        pf_barrier();
+        if constexpr (!B2 || S % 2 == 1) {
+            pf_wait_vmcnt<KEEP>();
+            pf_barrier();
+        }
     };
 
     if (n_tiles > 0) {

@@ -193,3 +193,17 @@ def test_prefill_more_than_64_pages_and_one_tile_per_page(exe):
     check(exe, w, "80 pages of 32 tokens")
     w = make_prefill(1, 48, 4, 1, 128, 32, [2100], seed=22)
     check(exe, w, "68 pages, head_dim 128, one KV head")
+
+
+@pytest.mark.parametrize("stages", [4, 8])
+def test_prefill_other_stage_counts(exe, stages):
+    """Six K/V tiles staged in LDS is the default; four and eight are selectable, and with eight
+    the 64-rows-per-wave kernel lets its waves meet only after every second tile."""
+    assert exe.setOption("prefill_stages", stages)
+    try:
+        for H, Hkv, D in ((8, 2, 128), (8, 8, 64), (8, 1, 128)):
+            check(exe, make_prefill(2, 40, H, Hkv, D, 64, [100, 0], seed=H + D + stages), f"stages{stages} H{H}/{Hkv} D{D}")
+        check(exe, make_prefill(2, 256, 8, 2, 128, 64, [1000, 517], seed=9 + stages), f"stages{stages} chunk 256")
+        check(exe, make_prefill(2, 64, 8, 2, 64, 32, [2500, 3], seed=21 + stages), f"stages{stages} 80 pages of 32 tokens")
+    finally:
+        assert exe.setOption("prefill_stages", 0)
