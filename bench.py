@@ -494,6 +494,57 @@ def load_traffic(workload: str, kernel: str, work_items: int):
     return e.get("hbm_bytes_per_launch")
 
 
+def probe_timeline(n_wg: int) -> dict:
+    """Per-workgroup time stamps of the last tile-balanced decode launch, from a library built with
+    -DMLC_STREAM_PROBE (MLC_HIPCC_EXTRA; add -DMLC_STREAM_PROBE_TILES for three stamps per tile).
+    Thread 0 of every workgroup writes the 100 MHz counter at fixed points; the figures are us
+    after the first workgroup's entry, min / median / p90 / max over the workgroups."""
+    import ctypes as C
+
+    from mlcompiler_amd._lib import load
+    lib = load()
+    if not hasattr(lib, "mlc_hip_debug_probe"):
+        raise SystemExit("--probe needs a library built with MLC_HIPCC_EXTRA=-DMLC_STREAM_PROBE")
+    buf = np.zeros((n_wg, 32), np.uint64)
+    lib.mlc_hip_debug_probe.argtypes = [C.c_void_p, C.c_size_t]
+    if not lib.mlc_hip_debug_probe(buf.ctypes.data, n_wg):
+        raise RuntimeError("mlc_hip_debug_probe failed")
+    t = buf.astype(np.int64)
+    us = lambda x: (x - t[:, 0].min()) / 100.0
+
+    def st(x):
+        x = np.sort(np.asarray(x, np.float64))
+        if x.size == 0:
+            return None
+        return {"min": round(float(x[0]), 2), "median": round(float(x[x.size // 2]), 2),
+                "p90": round(float(x[x.size * 9 // 10]), 2), "max": round(float(x[-1]), 2)}
+    names = ["entry", "per_request_figures_known", "page_ids_fetched", "first_tile_landed", "last_tile_consumed", "exit"]
+    out = {"workgroups": n_wg, "tiles_per_workgroup": sorted(set(int(v) for v in t[:, 6]))}
+    for i, nm in enumerate(names):
+        out[nm] = st(us(t[:, i]))
+    lastc, ex = us(t[:, 4]), us(t[:, 5])
+    pub = (t[:, 26] >= t[:, 0]) & (t[:, 26] <= t[:, 5])
+    mer = (t[:, 28] >= t[:, 0]) & (t[:, 28] <= t[:, 5])
+    out["published"] = int(pub.sum())
+    out["partials_acknowledged_after_last_tile"] = st((us(t[:, 26]) - lastc)[pub])
+    out["ticket_after_acknowledgement"] = st((us(t[:, 27]) - us(t[:, 26]))[pub])
+    out["merged_by_wave_0"] = int(mer.sum())
+    out["exit_after_ticket_mergers"] = st((ex - us(t[:, 28]))[mer])
+    out["exit_after_last_tile_mergers"] = st((ex - lastc)[mer])
+    out["exit_after_last_tile_others"] = st((ex - lastc)[~mer])
+    if t[:, 8].max() > 0:  # stamps per tile: wait and work on each of the first six tiles
+        n = t[:, 6]
+        per_tile = []
+        for k in range(6):
+            m = n > k
+            if not m.any():
+                break
+            wb, ab, ac = us(t[m, 8 + 3 * k]), us(t[m, 9 + 3 * k]), us(t[m, 10 + 3 * k])
+            per_tile.append({"tile": k, "workgroups": int(m.sum()), "wait": st(ab - wb), "work": st(ac - ab), "done": st(ac)})
+        out["per_tile"] = per_tile
+    return out
+
+
 def run_decode(args, name: str, steps: int, warmup: int, cpu_budget: float, full: bool) -> dict:
     """Times one decode configuration through the C ABI and frees its buffers again.
     full: also the one-launch-at-a-time distribution, the changing-tables loop, the fp32-weight
@@ -560,6 +611,8 @@ def run_decode(args, name: str, steps: int, warmup: int, cpu_budget: float, full
     ev_ms, wall = native_loop(steps)
     r = {"case": c, "n_layers": n_layers, "steps": steps, "ev_us": ev_ms / steps * 1e3, "wall_us": wall / steps * 1e6,
          "launches": exe.lastDecodeLaunches(), "items": exe.lastDecodeWorkItems(), "kernel": exe.lastDecodeKernel()}
+    if args.probe:
+        r["probe_timeline"] = probe_timeline(r["items"])
 
     if full:
         # ---- one launch at a time, HIP events around each (the reference's harness reports its
@@ -776,6 +829,9 @@ def main() -> int:
                     help="0 = automatic (tile-balanced kernel), 1 = planned split-K items")
     ap.add_argument("--wgs-per-cu", type=int, default=0, help="tile-balanced kernel: workgroups per CU (0 = automatic)")
     ap.add_argument("--stages", type=int, default=0, help="tile-balanced kernel: LDS stages (0 = automatic)")
+    ap.add_argument("--probe", action="store_true",
+                    help="decode: print the per-workgroup timeline of the last launch as config.probe_timeline "
+                         "(needs a library built with MLC_HIPCC_EXTRA=-DMLC_STREAM_PROBE; its times mean nothing)")
     ap.add_argument("--opt", action="append", default=[], metavar="NAME=VALUE",
                     help="library tunable (mlc_hip_set_option), may be repeated")
     ap.add_argument("--prefill-stages", type=int, default=0, help="cfg5: LDS pipeline depth (0 = automatic)")
@@ -861,6 +917,7 @@ def main() -> int:
             "single_launch_us": r["single_us"],
             "us_per_layer_with_kv_write": round(r["kv_write_us"], 3),
             "host_cores": os.cpu_count(),
+            **({"probe_timeline": r["probe_timeline"]} if "probe_timeline" in r else {}),
         },
         "roofline": {
             "bound": "hbm",
