@@ -347,43 +347,6 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     fetch_pages(ci);
     MLC_PROBE(2);
 
-    // ---- the step's KV write: this workgroup owns the last tile of every pair that ends in
-    // its range, so it writes those pairs' slices of the new rows, waits for the stores, and
-    // only then loads anything.  2 * CPR lanes move one pair's K and V slice.
-    if (a.new_k != nullptr) {
-        constexpr int LPP = 2 * CPR;           // lanes per pair
-        constexpr int PPW = 64 / LPP;          // pairs per wave and round
-        // pairs that end in [g0, g1): the one under the cursor, then every following one that
-        // ends before g1.  Pair index p counts pairs with tiles only, from the cursor's.
-        const uint32_t first_end = g0 + (cc.tiles - cc.t);  // one past the last tile of the first pair
-        if (first_end <= g1) {
-            // walk the pairs with a cursor of their own; each wave takes PPW pairs per round
-            Cursor cw = cc;
-            uint32_t end = first_end, idx = 0;
-            for (;;) {
-                const uint32_t slot = idx % (uint32_t)(PPW * NW);
-                if (slot / PPW == (uint32_t)wave && (uint32_t)lane / LPP == slot % PPW) {
-                    const uint32_t l2 = (uint32_t)lane % LPP;
-                    const bool is_v = l2 >= (uint32_t)CPR;
-                    const uint32_t cch = l2 % CPR;
-                    const size_t row = (size_t)a.new_ids[cw.r] * a.page_size + a.new_slots[cw.r];
-                    const uint4 val = (is_v ? a.new_v : a.new_k)[((size_t)cw.r * Hkv + cw.kvh) * CPR + cch];
-                    uint4* dst = const_cast<uint4*>(is_v ? a.v_pages : a.k_pages);
-                    dst[(row * Hkv + cw.kvh) * CPR + cch] = val;
-                }
-                ++idx;
-                if (end >= g1) break;  // no tile of the range is left behind this pair
-                cw.t = cw.tiles - 1;
-                advance(cw);           // first tile of the next pair
-                if (end + cw.tiles > g1) break;  // the next pair ends in a later range
-                end += cw.tiles;
-            }
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        sd_wait_vmcnt<0>();  // the rows have left this wave before any wave of the workgroup loads them
-        sd_barrier();
-    }
-
     // matrix-pipe mode: lane coordinates of the 16x16 MFMA layouts, the q operand (B of S^T =
     // K.q^T: column n16 = head of the group, dims 8*g4 .. +7 of every 32-dim step) as the sum of
     // two fp16 numbers, and the LDS offsets of this lane's K and V^T operand reads inside a tile.
@@ -940,9 +903,61 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
 
     // ---- the stream: the first NBUF tiles of the range go out together, then one tile per step
     // into the stage the step before has left
+    // ---- the step's KV write: this workgroup owns the last tile of every pair that ends in
+    // its range, so it writes those pairs' slices of the new rows before it loads the tiles
+    // that hold them.  A new row is its request's newest position, so it lies in the pair's
+    // last tile: where the range starts with another tile, that tile is requested first, the
+    // rows are written behind it (their page ids and slots are a memory round trip of their
+    // own), and the workgroup makes sure of the stores (every wave's memory counter at zero,
+    // then a barrier) before the second tile goes out; where the range starts with a pair's
+    // last tile, it writes and makes sure before it loads anything.  2 * CPR lanes move one
+    // pair's K and V slice.
+    bool kv_unsettled = false;
+    auto write_new_rows = [&]() {
+        constexpr int LPP = 2 * CPR;           // lanes per pair
+        constexpr int PPW = 64 / LPP;          // pairs per wave and round
+        // pairs that end in [g0, g1): the one under the cursor, then every following one that
+        // ends before g1.  Pair index p counts pairs with tiles only, from the cursor's.
+        const uint32_t first_end = g0 + (cc.tiles - cc.t);  // one past the last tile of the first pair
+        if (first_end <= g1) {
+            // walk the pairs with a cursor of their own; each wave takes PPW pairs per round
+            Cursor cw = cc;
+            uint32_t end = first_end, idx = 0;
+            for (;;) {
+                const uint32_t slot = idx % (uint32_t)(PPW * NW);
+                if (slot / PPW == (uint32_t)wave && (uint32_t)lane / LPP == slot % PPW) {
+                    const uint32_t l2 = (uint32_t)lane % LPP;
+                    const bool is_v = l2 >= (uint32_t)CPR;
+                    const uint32_t cch = l2 % CPR;
+                    const size_t row = (size_t)a.new_ids[cw.r] * a.page_size + a.new_slots[cw.r];
+                    const uint4 val = (is_v ? a.new_v : a.new_k)[((size_t)cw.r * Hkv + cw.kvh) * CPR + cch];
+                    uint4* dst = const_cast<uint4*>(is_v ? a.v_pages : a.k_pages);
+                    dst[(row * Hkv + cw.kvh) * CPR + cch] = val;
+                }
+                ++idx;
+                if (end >= g1) break;  // no tile of the range is left behind this pair
+                cw.t = cw.tiles - 1;
+                advance(cw);           // first tile of the next pair
+                if (end + cw.tiles > g1) break;  // the next pair ends in a later range
+                end += cw.tiles;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    };
+
+    const bool kv_first = a.new_k != nullptr && cc.t + 1u == cc.tiles;
+    if (kv_first) {
+        write_new_rows();
+        sd_wait_vmcnt<0>();  // the rows have left this wave before any wave of the workgroup loads them
+        sd_barrier();
+    }
     load_q(cc);
     uint32_t issued = 1;
     issue_tile(ci, 0);
+    if (a.new_k != nullptr && !kv_first) {
+        write_new_rows();
+        kv_unsettled = true;
+    }
     uint32_t seg_first = g0;  // first tile consumed for the pair under cc
     bool drain = false;       // stores are in flight: they do not complete in order with loads
     uint32_t slot = 0;        // stage of tile k
@@ -954,6 +969,11 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         if (k < 6) MLC_PROBE_TILE(8 + 3 * k);
         if (drain) sd_wait_vmcnt<0>(); else wait_tile(issued - k - 1u);
         drain = false;
+        if (kv_unsettled) {  // first step only: nothing but the first tile was behind the stores, the
+                             // counter has just been at zero in every wave that comes here
+            kv_unsettled = false;
+            sd_barrier();
+        }
         // ... and everyone's; everyone has left tile k-1, whose stage is free (matrix-pipe mode: a
         // wave loads, reads and overwrites only its own rows of a stage, no barrier)
         if constexpr (!MF) sd_barrier();
