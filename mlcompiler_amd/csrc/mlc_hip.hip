@@ -238,6 +238,9 @@ struct Ctx {
     long opt_wgs_per_cu = 0;        // tile-balanced kernel: workgroups per CU (0 = automatic)
     long opt_stream_stages = 0;     // tile-balanced kernel: LDS stages per workgroup (0 = automatic)
     long opt_grid_wgs = 0;          // tile-balanced kernel: exact grid size (0 = from workgroups per CU)
+    // tile-balanced kernel: units the end of a (request, KV head) pair counts for when the ranges are
+    // cut (a tile is one unit).  Swept 0..6 on MI355X at configurations 2, 3 and 4: 3 was fastest.
+    long opt_pair_cost = 3;
     long table_uploads = 0;         // page-table uploads of the tile-balanced path (for tests)
     // A captured pass: the kernel launches of the encode calls between mlc_hip_capture_begin and
     // mlc_hip_capture_end as an executable HIP graph, and what the launches read that changes from
@@ -953,6 +956,7 @@ void stream_fill_common(StreamArgs& a, const void* q, const void* k_pages, const
     a.meta = nullptr;
     a.meta_stride = 0;
     a.scale_log2e = (1.0f / std::sqrt(static_cast<float>(D))) * 1.44269504088896340736f;
+    a.pair_cost = (uint32_t)g.opt_pair_cost;
     a.new_k = a.new_v = nullptr;
     a.new_ids = a.new_slots = nullptr;
 }
@@ -1149,7 +1153,8 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
             total_tiles += (lim + tile - 1) / tile;
         }
         total_tiles *= kv_heads;
-        if (total_tiles >= 0x7FFFFFFFull) use_stream = false;
+        // (the kernel counts in units: tiles plus at most 64 per (request, KV head) pair)
+        if (total_tiles + 64ull * batch * kv_heads >= 0x7FFFFFFFull) use_stream = false;
     }
     const DecodePlan* plan = nullptr;
     if (!use_stream) {
@@ -1348,7 +1353,7 @@ int mlc_hip_paged_attn_decode_noalloc(const void* q, const void* k_pages, const 
         total_tiles += (lim + tile - 1) / tile;
     }
     total_tiles *= kv_heads;
-    if (total_tiles >= 0x7FFFFFFFull) return fail("decode (no allocation): too many KV tiles");
+    if (total_tiles + 64ull * batch * kv_heads >= 0x7FFFFFFFull) return fail("decode (no allocation): too many KV tiles");
     {
         const size_t qo_bytes = batch * num_heads * head_dim * 4;
         const size_t kq = known_bytes(q), ko = known_bytes(o), kt = known_bytes(page_tables_flat_device);
@@ -2437,6 +2442,11 @@ int mlc_hip_set_option(const char* name, long value) {
     if (!std::strcmp(name, "prefill_stages")) {
         if (value != 0 && value != 2 && value != 4 && value != 6 && value != 8) return 0;
         g.opt_prefill_stages = value;
+        return 1;
+    }
+    if (!std::strcmp(name, "decode_pair_cost")) {
+        if (value < 0 || value > 64) return 0;
+        g.opt_pair_cost = value;
         return 1;
     }
     if (!std::strcmp(name, "decode_mfma")) {

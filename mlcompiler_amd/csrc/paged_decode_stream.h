@@ -51,6 +51,7 @@ struct StreamArgs {
     uint32_t capacity_pages;    // page ids are clamped below this (0: not clamped)
     uint32_t meta_stride;
     float scale_log2e;          // log2(e) / sqrt(D)
+    uint32_t pair_cost;         // units a pair's end counts for when the ranges are cut (0: tiles only)
     // The step's KV write done by this launch (null: none), as in DecodeArgs: the workgroup
     // that owns a pair's last tile writes that pair's slice of the new rows before it loads
     // anything.
@@ -70,7 +71,7 @@ constexpr size_t stream_static_lds_bytes(int NBUF, size_t G, size_t D, bool matr
     return (size_t)NBUF * 2 * 8192 + (matrix_pipe ? (4 * G * D + 2 * 4 * G) * 4 : 24);
 }
 // dynamic LDS: tile prefix [B + 1], visible lengths [B], page-table offsets [B]
-inline size_t stream_dynamic_lds_bytes(size_t batch) { return (3 * batch + 1) * 4; }
+inline size_t stream_dynamic_lds_bytes(size_t batch) { return (4 * batch + 2) * 4; }
 
 // Timing probes, compiled in only for experiments (results then are wrong or partly so):
 //   -DMLC_STREAM_PROBE  thread 0 of every workgroup writes the 100 MHz counter at fixed points
@@ -168,6 +169,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     uint32_t* s_start = s_meta;            // [B + 1] tiles of the requests before r (one KV head)
     uint32_t* s_lim = s_meta + B + 1;      // [B] visible tokens
     uint32_t* s_off = s_lim + B;           // [B] offset of the request's page ids
+    uint32_t* s_nzb = s_off + B;           // [B + 1] requests with tiles before r
 
     MLC_PROBE(0);
     // Everything the prologue needs from the kernel arguments is requested now, in one go: left
@@ -192,7 +194,9 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
 
     // ---- the per-request arrays: visible length, page-table offset, tile prefix
     uint32_t v_start = 0, v_tiles = 0, v_lim = 0, v_off = 0;  // SMALL: request `lane`
+    uint32_t v_nzb = 0;                                        // SMALL: requests with tiles before `lane`
     uint32_t tiles_head;                                       // tiles of all requests (one KV head)
+    uint32_t nz_head;                                          // requests with tiles
     if constexpr (SMALL) {
         // The arrays inside the kernel arguments are read before anything else is known (their
         // address is the argument segment's, no pointer has to be fetched first); lanes past
@@ -211,11 +215,14 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         const uint32_t incl = wave_inclusive_scan(v_tiles);
         v_start = incl - v_tiles;
         tiles_head = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+        const uint64_t nz = __ballot(v_tiles != 0);
+        v_nzb = (uint32_t)__builtin_popcountll(nz & ((1ull << lane) - 1ull));
+        nz_head = (uint32_t)__builtin_popcountll(nz);
     } else {
         if (wave == 0) {
             const uint32_t* meta = a.meta ? a.meta : a.emb;
             const uint32_t stride = a.meta_stride;
-            uint32_t carry = 0;
+            uint32_t carry = 0, carry_nz = 0;
             for (uint32_t b0 = 0; b0 < B; b0 += 64) {
                 const uint32_t i = b0 + lane;
                 uint32_t seq = 0, qp = 0, off = 0;
@@ -227,17 +234,24 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
                 const uint32_t lim = (a.causal && qp < seq) ? qp + 1u : seq;  // metal_runtime.mm:2286
                 const uint32_t tiles = (lim + TT - 1) / TT;
                 const uint32_t x = wave_inclusive_scan(tiles);
+                const uint64_t nz = __ballot(tiles != 0);
                 if (i < B) {
                     s_start[i] = carry + x - tiles;
                     s_lim[i] = lim;
                     s_off[i] = off;
+                    s_nzb[i] = carry_nz + (uint32_t)__builtin_popcountll(nz & ((1ull << lane) - 1ull));
                 }
                 carry += (uint32_t)__builtin_amdgcn_readlane((int)x, 63);
+                carry_nz += (uint32_t)__builtin_popcountll(nz);
             }
-            if (lane == 0) s_start[B] = carry;
+            if (lane == 0) {
+                s_start[B] = carry;
+                s_nzb[B] = carry_nz;
+            }
         }
         __syncthreads();
         tiles_head = s_start[B];
+        nz_head = s_nzb[B];
     }
     MLC_PROBE(1);
     auto req_start = [&](uint32_t r) {
@@ -247,6 +261,10 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     auto req_tiles = [&](uint32_t r) {
         if constexpr (SMALL) return (uint32_t)__builtin_amdgcn_readlane((int)v_tiles, (int)r);
         else return (uint32_t)__builtin_amdgcn_readfirstlane(s_start[r + 1] - s_start[r]);
+    };
+    auto req_nzb = [&](uint32_t r) {
+        if constexpr (SMALL) return (uint32_t)__builtin_amdgcn_readlane((int)v_nzb, (int)r);
+        else return (uint32_t)__builtin_amdgcn_readfirstlane(s_nzb[r]);
     };
     auto req_lim = [&](uint32_t r) {
         if constexpr (SMALL) return (uint32_t)__builtin_amdgcn_readlane((int)v_lim, (int)r);
@@ -266,16 +284,20 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         }
     }
 
+    // The ranges are cut in units: a tile is one unit, and the end of a pair (the waves meet, the
+    // pair's figures are put aside or published, q is fetched again) counts for PC more, so that a
+    // workgroup whose range crosses from one pair into the next gets fewer tiles.  Unit numbering:
+    // [request][kv head][the pair's tiles, then PC units that stand for its end].
     const uint32_t T = tiles_head * Hkv;                       // the host keeps this below 2^31
-    const uint32_t W = gridDim.x < T ? gridDim.x : T;          // every workgroup below W has work
+    // (nothing to balance where every tile gets a workgroup of its own)
+    const uint32_t PC = T > gridDim.x ? a.pair_cost : 0u;
+    const uint32_t UT = T + PC * nz_head * Hkv;                // ... and this
+    const uint32_t W = gridDim.x < UT ? gridDim.x : UT;
     const uint32_t w = blockIdx.x;
     if (w >= W) return;
-    // T = W * tq + trem: the first trem workgroups take tq + 1 tiles, the others tq
-    const uint32_t tq = __builtin_amdgcn_readfirstlane(T / W), trem = T - tq * W;
-    auto range_start = [&](uint32_t wg) { return wg * tq + (wg < trem ? wg : trem); };
-    const uint32_t g0 = range_start(w);
-    const uint32_t n = tq + (w < trem ? 1u : 0u);  // >= 1
-    const uint32_t g1 = g0 + n;
+    // UT = W * tq + trem: the first trem workgroups take tq + 1 units, the others tq
+    const uint32_t tq = __builtin_amdgcn_readfirstlane(UT / W), trem = UT - tq * W;
+    auto unit_start = [&](uint32_t wg) { return wg * tq + (wg < trem ? wg : trem); };
 
     // Position in the tile stream: request, KV head, tile of the request, and the request's
     // figures.  All wave-uniform (kept in scalar registers).
@@ -287,23 +309,38 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         cu.lim = req_lim(cu.r);
         cu.off = req_off(cu.r);
     };
-    // largest r with start[r] <= key (key < tiles_head)
-    auto find_request = [&](uint32_t key) {
+    // largest r with start[r] <= key (key below the total), starts counted in tiles (pc = 0) or
+    // in units (pc = PC)
+    auto find_request = [&](uint32_t key, uint32_t pc = 0) {
         if constexpr (SMALL) {
             // lanes past the batch hold the total, which is above any key
-            return (uint32_t)__builtin_popcountll(__ballot(v_start <= key)) - 1u;
+            return (uint32_t)__builtin_popcountll(__ballot(v_start + pc * v_nzb <= key)) - 1u;
         } else {
             uint32_t base = 0;
             if (B > 64) {  // 64-ary search, two levels
                 const uint32_t idx = (uint32_t)lane * 64u;
-                const uint32_t v = idx < B ? s_start[idx] : 0xFFFFFFFFu;
+                const uint32_t v = idx < B ? s_start[idx] + pc * s_nzb[idx] : 0xFFFFFFFFu;
                 base = (uint32_t)(__builtin_popcountll(__ballot(v <= key)) - 1) * 64u;
             }
             const uint32_t idx = base + (uint32_t)lane;
-            const uint32_t v = idx < B ? s_start[idx] : 0xFFFFFFFFu;
+            const uint32_t v = idx < B ? s_start[idx] + pc * s_nzb[idx] : 0xFFFFFFFFu;
             return (uint32_t)__builtin_amdgcn_readfirstlane(base + (uint32_t)__builtin_popcountll(__ballot(v <= key)) - 1u);
         }
     };
+    // tiles in front of unit u
+    auto tiles_before = [&](uint32_t u) {
+        if (PC == 0) return u;
+        if (u >= UT) return T;
+        const uint32_t r = find_request(u / Hkv, PC);
+        const uint32_t tiles = req_tiles(r), per = tiles + PC;
+        const uint32_t rem = u - (req_start(r) + PC * req_nzb(r)) * Hkv;
+        const uint32_t kvh = __builtin_amdgcn_readfirstlane(rem / per), x = rem - kvh * per;
+        return req_start(r) * Hkv + kvh * tiles + (x < tiles ? x : tiles);
+    };
+    const uint32_t g0 = tiles_before(unit_start(w));
+    const uint32_t g1 = tiles_before(unit_start(w + 1u));
+    const uint32_t n = g1 - g0;
+    if (n == 0) return;  // only the units of a pair's end
     auto seek = [&](Cursor& cu, uint32_t g) {
         cu.r = find_request(g / Hkv);
         load_request(cu);
@@ -776,10 +813,10 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     };
     // element (head k / HPK, dim) of output register k of this lane
     const int dim0 = c * 8 + r_l * HPK;
-    // workgroup that holds tile g
+    // workgroup that holds unit u
     const uint32_t thr = trem * (tq + 1u);
-    auto wg_of = [&](uint32_t g) {
-        return (uint32_t)__builtin_amdgcn_readfirstlane(g < thr ? g / (tq + 1u) : trem + (g - thr) / tq);
+    auto wg_of_unit = [&](uint32_t u) {
+        return (uint32_t)__builtin_amdgcn_readfirstlane(u < thr ? u / (tq + 1u) : trem + (u - thr) / tq);
     };
     auto out_row = [&](const Cursor& cu) {
         return a.o + ((size_t)cu.r * a.num_heads + cu.kvh * G + hg * HPW) * D;
@@ -788,9 +825,13 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     // slot 2w, a later (so: its last) pair slot 2w + 1.
     auto pair_out = [&](const Cursor& cu, uint32_t ps, uint32_t pe) {
         PairOut po;
-        po.w_lo = wg_of(ps);
-        po.n_splits = wg_of(pe - 1u) - po.w_lo + 1u;
-        po.slot_first = 2u * po.w_lo + (range_start(po.w_lo) == ps ? 0u : 1u);
+        // the pair's tiles are consecutive units; the PC units in front of them stand for the
+        // end of the pair before, so the first sharer has no tile of that pair (the pair is its
+        // first) exactly when its range starts inside them or at the pair's first tile
+        const uint32_t ups = ps + PC * (Hkv * req_nzb(cu.r) + cu.kvh);
+        po.w_lo = wg_of_unit(ups);
+        po.n_splits = wg_of_unit(ups + (pe - ps) - 1u) - po.w_lo + 1u;
+        po.slot_first = 2u * po.w_lo + (unit_start(po.w_lo) + PC >= ups ? 0u : 1u);
         po.my_slot = (ps <= g0) ? 2u * w : 2u * w + 1u;
         po.orow = out_row(cu);
         return po;

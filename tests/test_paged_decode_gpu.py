@@ -15,12 +15,16 @@ def decode_kernel(exe, request):
     """Every test runs on both tiled decode kernels: the tile-balanced one (fixed grid, work
     derived from the tables in the kernel; the default), with the tile arithmetic on the matrix
     pipe where the shape allows it (the default) and on the vector pipe, and the planned one
-    (host-built items)."""
+    (host-built items).  The default run cuts the workgroups' ranges with the end of a pair
+    counting three units, the vector-pipe run by tiles alone."""
     assert exe.setOption("decode_kernel", 1 if request.param == "planned" else 0)
     assert exe.setOption("decode_mfma", 0 if request.param == "balanced-vector" else 1)
+    # (the vector-pipe runs also cut the ranges by tiles alone; the default counts a pair's end)
+    assert exe.setOption("decode_pair_cost", 0 if request.param == "balanced-vector" else 3)
     yield "balanced" if request.param == "balanced-vector" else request.param
     exe.setOption("decode_kernel", 0)
     exe.setOption("decode_mfma", 1)
+    exe.setOption("decode_pair_cost", 3)
 
 
 # how each kernel's split of the work is varied: items aimed for / exact grid size
