@@ -20,11 +20,11 @@ def decode_kernel(exe, request):
     assert exe.setOption("decode_kernel", 1 if request.param == "planned" else 0)
     assert exe.setOption("decode_mfma", 0 if request.param == "balanced-vector" else 1)
     # (the vector-pipe runs also cut the ranges by tiles alone; the default counts a pair's end)
-    assert exe.setOption("decode_pair_cost", 0 if request.param == "balanced-vector" else 3)
+    assert exe.setOption("decode_pair_cost", 0 if request.param == "balanced-vector" else 3)  # (3: also for one and two waves)
     yield "balanced" if request.param == "balanced-vector" else request.param
     exe.setOption("decode_kernel", 0)
     exe.setOption("decode_mfma", 1)
-    exe.setOption("decode_pair_cost", 3)
+    exe.setOption("decode_pair_cost", -1)
 
 
 # how each kernel's split of the work is varied: items aimed for / exact grid size
