@@ -239,10 +239,10 @@ struct Ctx {
     long opt_stream_stages = 0;     // tile-balanced kernel: LDS stages per workgroup (0 = automatic)
     long opt_grid_wgs = 0;          // tile-balanced kernel: exact grid size (0 = from workgroups per CU)
     // tile-balanced kernel: units the end of a (request, KV head) pair counts for when the ranges are
-    // cut (a tile is one unit).  -1 = automatic: 3 for workgroups of four waves (swept 0..6 on
-    // MI355X at GQA ratios 4, 8 and 16, head_dim 64 and 128: 3 or 4 was fastest, up to a quarter
-    // faster than 0), 0 for the one- and two-wave workgroups of GQA ratios 1 and 2, whose pair ends
-    // are cheap (there 3 was 1 to 5 % slower than 0).
+    // cut (a tile is one unit).  -1 = automatic: 3 for workgroups of four waves, 4 where those hold
+    // 16 heads of 128 (swept 0..6 on MI355X at GQA ratios 4, 8 and 16, head_dim 64 and 128: 3 or 4
+    // was fastest, up to a quarter faster than 0), 0 for the one- and two-wave workgroups of GQA
+    // ratios 1 and 2, whose pair ends are cheap (there 3 was 1 to 5 % slower than 0).
     long opt_pair_cost = -1;
     long table_uploads = 0;         // page-table uploads of the tile-balanced path (for tests)
     // A captured pass: the kernel launches of the encode calls between mlc_hip_capture_begin and
@@ -919,9 +919,10 @@ unsigned stream_grid(size_t G, size_t D, int nbuf, size_t dyn_lds) {
     return (unsigned)std::max<size_t>(W, 1);
 }
 
-uint32_t stream_pair_cost(int nw) {
+uint32_t stream_pair_cost(int nw, size_t G, size_t D) {
     if (g.opt_pair_cost >= 0) return (uint32_t)g.opt_pair_cost;
-    return nw == 4 ? 3u : 0u;
+    if (nw != 4) return 0u;
+    return G * D >= 2048 ? 4u : 3u;  // (16 heads of 128: 30.9 us with 4 against 33.9 us with 3)
 }
 
 // Arithmetic mode of the tile-balanced kernel: 0 fp32 softmax weights, 1 fp16 weights on the vector
@@ -1212,7 +1213,7 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
         StreamArgs a;
         stream_fill_common(a, q, k_pages, v_pages, o, batch, num_heads, kv_heads, head_dim, page_size_tokens,
                            apply_causal);
-        a.pair_cost = stream_pair_cost(s_nw);
+        a.pair_cost = stream_pair_cost(s_nw, G, head_dim);
         a.pt_flat = d_flat;
         {
             // pools this library allocated: the kernel clamps page ids below their size (the host
@@ -1374,7 +1375,7 @@ int mlc_hip_paged_attn_decode_noalloc(const void* q, const void* k_pages, const 
     const unsigned n_wg = stream_grid(G, head_dim, nbuf, dyn_lds);
     StreamArgs a;
     stream_fill_common(a, q, k_pages, v_pages, o, batch, num_heads, kv_heads, head_dim, page_size_tokens, apply_causal);
-    a.pair_cost = stream_pair_cost(nw);
+    a.pair_cost = stream_pair_cost(nw, G, head_dim);
     a.pt_flat = page_tables_flat_device;
     {
         // the page ids are on the device and cannot be checked here: pools this library allocated
