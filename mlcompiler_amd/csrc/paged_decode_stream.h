@@ -337,10 +337,11 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         const uint32_t kvh = __builtin_amdgcn_readfirstlane(rem / per), x = rem - kvh * per;
         return req_start(r) * Hkv + kvh * tiles + (x < tiles ? x : tiles);
     };
-    const uint32_t g0 = tiles_before(unit_start(w));
-    const uint32_t g1 = tiles_before(unit_start(w + 1u));
-    const uint32_t n = g1 - g0;
-    if (n == 0) return;  // only the units of a pair's end
+    // This range in tiles: [g0, g1), n of them.  g0 comes with the cursor's start below; g1 and n
+    // are worked out behind the first tile's request, off the way to it (before it only where the
+    // launch carries the KV write, which needs them).
+    const uint32_t u0 = unit_start(w), u1 = unit_start(w + 1u);
+    uint32_t g0 = u0, g1 = 0, n = 0;
     auto seek = [&](Cursor& cu, uint32_t g) {
         cu.r = find_request(g / Hkv);
         load_request(cu);
@@ -362,7 +363,28 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     const uint32_t tpp = a.page_size / TT;  // tiles per page (page size is a multiple of the tile)
 
     Cursor ci, cc;  // issue side (one tile ahead) and consume side
-    seek(cc, g0);
+    if (PC == 0) {
+        seek(cc, g0);
+    } else {
+        // the cursor at unit u0, or, where that is one of the units of a pair's end, at the first
+        // tile behind it
+        cc.r = find_request(u0 / Hkv, PC);
+        load_request(cc);
+        const uint32_t per = cc.tiles + PC;
+        const uint32_t rem = u0 - (req_start(cc.r) + PC * req_nzb(cc.r)) * Hkv;
+        cc.kvh = __builtin_amdgcn_readfirstlane(rem / per);
+        const uint32_t x = rem - cc.kvh * per;
+        const uint32_t pair0 = req_start(cc.r) * Hkv + cc.kvh * cc.tiles;
+        if (x < cc.tiles) {
+            cc.t = x;
+            g0 = pair0 + x;
+        } else {
+            if (u0 + (per - x) >= u1) return;  // nothing but units of a pair's end
+            g0 = pair0 + cc.tiles;
+            cc.t = cc.tiles - 1u;
+            advance(cc);
+        }
+    }
     ci = cc;
 
     const uint32_t* pt_flat = a.pt_flat ? a.pt_flat : a.emb + 3u * a.meta_stride;
@@ -986,6 +1008,10 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     };
 
+    if (a.new_k != nullptr) {
+        g1 = tiles_before(u1);
+        n = g1 - g0;
+    }
     const bool kv_first = a.new_k != nullptr && cc.t + 1u == cc.tiles;
     if (kv_first) {
         write_new_rows();
@@ -995,6 +1021,10 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     load_q(cc);
     uint32_t issued = 1;
     issue_tile(ci, 0);
+    if (a.new_k == nullptr) {
+        g1 = tiles_before(u1);
+        n = g1 - g0;
+    }
     if (a.new_k != nullptr && !kv_first) {
         write_new_rows();
         kv_unsettled = true;
