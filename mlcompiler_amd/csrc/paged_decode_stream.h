@@ -339,7 +339,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     };
     // This range in tiles: [g0, g1), n of them.  g0 comes with the cursor's start below; g1 and n
     // are worked out behind the first tile's request, off the way to it (before it only where the
-    // launch carries the KV write, which needs them).
+    // range starts with a tile that holds a new row of the KV write, which needs them).
     const uint32_t u0 = unit_start(w), u1 = unit_start(w + 1u);
     uint32_t g0 = u0, g1 = 0, n = 0;
     auto seek = [&](Cursor& cu, uint32_t g) {
@@ -1008,12 +1008,10 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     };
 
-    if (a.new_k != nullptr) {
-        g1 = tiles_before(u1);
-        n = g1 - g0;
-    }
     const bool kv_first = a.new_k != nullptr && cc.t + 1u == cc.tiles;
     if (kv_first) {
+        g1 = tiles_before(u1);
+        n = g1 - g0;
         write_new_rows();
         sd_wait_vmcnt<0>();  // the rows have left this wave before any wave of the workgroup loads them
         sd_barrier();
@@ -1021,7 +1019,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     load_q(cc);
     uint32_t issued = 1;
     issue_tile(ci, 0);
-    if (a.new_k == nullptr) {
+    if (!kv_first) {
         g1 = tiles_before(u1);
         n = g1 - g0;
     }
