@@ -377,8 +377,7 @@ long mlc_hip_decode_table_uploads(void);
  *   "decode_pair_cost"      0..64: the tile-balanced decode kernel gives every workgroup the same
  *                           number of units, a KV tile counting one and the end of a (request,
  *                           KV head) pair this many; 0 = the same number of tiles; -1 (default) =
- *                           3 for GQA ratios of 4 and more (workgroups of four waves; 4 for 16
- *                           heads of 128), 0 below
+ *                           4 for GQA ratios of 4 and more (workgroups of four waves), 0 below
  *   "decode_mfma"           1 (default) = the tile-balanced decode kernel does a tile's arithmetic
  *                           on the matrix pipe where the shape allows it (4 to 16 query heads per
  *                           KV head in 4 waves, fp16 softmax weights); 0 = on the vector pipe

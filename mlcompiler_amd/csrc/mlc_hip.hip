@@ -239,10 +239,12 @@ struct Ctx {
     long opt_stream_stages = 0;     // tile-balanced kernel: LDS stages per workgroup (0 = automatic)
     long opt_grid_wgs = 0;          // tile-balanced kernel: exact grid size (0 = from workgroups per CU)
     // tile-balanced kernel: units the end of a (request, KV head) pair counts for when the ranges are
-    // cut (a tile is one unit).  -1 = automatic: 3 for workgroups of four waves, 4 where those hold
-    // 16 heads of 128 (swept 0..6 on MI355X at GQA ratios 4, 8 and 16, head_dim 64 and 128: 3 or 4
-    // was fastest, up to a quarter faster than 0), 0 for the one- and two-wave workgroups of GQA
-    // ratios 1 and 2, whose pair ends are cheap (there 3 was 1 to 5 % slower than 0).
+    // cut (a tile is one unit).  -1 = automatic: 4 for workgroups of four waves (swept 0..6 on
+    // MI355X at GQA ratios 4, 8 and 16, head_dim 64 and 128: 3 or 4 was fastest, up to a quarter
+    // faster than 0; 4 is as fast as 3 for the attention alone at the TinyLlama shape and 0.8 us
+    // faster where the launch also carries the step's KV write, and 3 us faster for 16 heads of
+    // 128), 0 for the one- and two-wave workgroups of GQA ratios 1 and 2, whose pair ends are cheap
+    // (there 3 was 1 to 5 % slower than 0).
     long opt_pair_cost = -1;
     long table_uploads = 0;         // page-table uploads of the tile-balanced path (for tests)
     // A captured pass: the kernel launches of the encode calls between mlc_hip_capture_begin and
@@ -921,8 +923,9 @@ unsigned stream_grid(size_t G, size_t D, int nbuf, size_t dyn_lds) {
 
 uint32_t stream_pair_cost(int nw, size_t G, size_t D) {
     if (g.opt_pair_cost >= 0) return (uint32_t)g.opt_pair_cost;
-    if (nw != 4) return 0u;
-    return G * D >= 2048 ? 4u : 3u;  // (16 heads of 128: 30.9 us with 4 against 33.9 us with 3)
+    (void)G;
+    (void)D;
+    return nw == 4 ? 4u : 0u;
 }
 
 // Arithmetic mode of the tile-balanced kernel: 0 fp32 softmax weights, 1 fp16 weights on the vector

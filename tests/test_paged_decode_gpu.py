@@ -15,8 +15,9 @@ def decode_kernel(exe, request):
     """Every test runs on both tiled decode kernels: the tile-balanced one (fixed grid, work
     derived from the tables in the kernel; the default), with the tile arithmetic on the matrix
     pipe where the shape allows it (the default) and on the vector pipe, and the planned one
-    (host-built items).  The default run cuts the workgroups' ranges with the end of a pair
-    counting three units, the vector-pipe run by tiles alone."""
+    (host-built items).  The first run cuts the workgroups' ranges with the end of a pair
+    counting three units, the vector-pipe run by tiles alone (the library's default, four units
+    for workgroups of four waves, is what the other test files run)."""
     assert exe.setOption("decode_kernel", 1 if request.param == "planned" else 0)
     assert exe.setOption("decode_mfma", 0 if request.param == "balanced-vector" else 1)
     # (the vector-pipe runs also cut the ranges by tiles alone; the default counts a pair's end)
