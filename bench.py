@@ -35,6 +35,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
+N_CU = 256  # MI355X compute units (8 XCDs of 32)
 
 
 def bench_copy(args) -> int:
@@ -526,10 +527,10 @@ def probe_timeline(n_wg: int) -> dict:
     pub = (t[:, 26] >= t[:, 0]) & (t[:, 26] <= t[:, 5])
     mer = (t[:, 28] >= t[:, 0]) & (t[:, 28] <= t[:, 5])
     out["published"] = int(pub.sum())
-    out["partials_acknowledged_after_last_tile"] = st((us(t[:, 26]) - lastc)[pub])
-    out["ticket_after_acknowledgement"] = st((us(t[:, 27]) - us(t[:, 26]))[pub])
+    out["partial_stores_issued_after_last_tile"] = st((us(t[:, 26]) - lastc)[pub])
     out["merged_by_wave_0"] = int(mer.sum())
-    out["exit_after_ticket_mergers"] = st((ex - us(t[:, 28]))[mer])
+    out["merge_begins_after_last_tile"] = st((us(t[:, 28]) - lastc)[mer])
+    out["exit_after_merge_begins"] = st((ex - us(t[:, 28]))[mer])
     out["exit_after_last_tile_mergers"] = st((ex - lastc)[mer])
     out["exit_after_last_tile_others"] = st((ex - lastc)[~mer])
     if t[:, 8].max() > 0:  # stamps per tile: wait and work on each of the first six tiles
@@ -635,7 +636,9 @@ def run_decode(args, name: str, steps: int, warmup: int, cpu_budget: float, full
         # (a) the per-request arrays change (one query position alternates); (b) the page table's
         # content changes too (two page ids of one request trade places: same bytes read), so
         # the device copy of the table is refreshed by every call.
-        n_b = min(steps, 200)
+        # (their own step count and a warm-up pass each: at the driver's --steps 20 a one-off upload or
+        # the first launches of a mode would dominate the figure)
+        n_b = 500
         for key, swap_pages in (("tables_change_us", False), ("page_table_changes_us", True)):
             pos = c.q_positions.copy()
             flat2 = c.page_tables_flat.copy()
@@ -643,40 +646,47 @@ def run_decode(args, name: str, steps: int, warmup: int, cpu_budget: float, full
             o0 = int(c.page_table_offsets[big])
             if int(c.page_table_offsets[big + 1]) - o0 >= 2:
                 flat2[o0], flat2[o0 + 1] = flat2[o0 + 1], flat2[o0]
+            pos_alt = [pos.copy(), pos.copy()]
+            pos_alt[1][0] = pos[0] - 1
+
+            def changing(i):
+                step(i % n_layers, flat=(flat2 if (swap_pages and i % 2) else None), pos=pos_alt[i % 2], causal=False)
+
+            exe.beginForwardPassCB()
+            for i in range(2 * n_layers):
+                changing(i)
+            assert exe.flushForwardPassCB()
             exe.beginForwardPassCB()
             exe.timerStart()
             tb = time.perf_counter()
             for i in range(n_b):
-                pos2 = pos.copy()
-                pos2[0] = pos[0] - (i % 2)
-                step(i % n_layers, flat=(flat2 if (swap_pages and i % 2) else None), pos=pos2, causal=False)
+                changing(i)
             ev = exe.timerStopMs()
             assert exe.flushForwardPassCB()
-            r[key] = {"wall": round((time.perf_counter() - tb) / n_b * 1e6, 3), "events": round(ev / n_b * 1e3, 3)}
+            r[key] = {"wall": round((time.perf_counter() - tb) / n_b * 1e6, 3), "events": round(ev / n_b * 1e3, 3),
+                      "steps": n_b}
 
         # ---- fp32 softmax weights for P.V (decode_pv_fp16 = 0: meets the reference's 1e-5 gate)
+        n_x = max(steps, 500)
         assert exe.setOption("decode_pv_fp16", 0)
-        native_loop(n_layers)
-        ev32, _ = native_loop(steps)
+        native_loop(2 * n_layers)
+        ev32, _ = native_loop(n_x)
         assert exe.setOption("decode_pv_fp16", 1)
-        r["pv_fp32_us"] = ev32 / steps * 1e3
+        r["pv_fp32_us"] = ev32 / n_x * 1e3
 
         # ---- products on the vector pipe (decode_mfma = 0), fp16 softmax weights as in the default
         if any(kv.startswith("decode_mfma=") for kv in args.opt):
             r["vector_pipe_us"] = float("nan")  # the caller chose the mode: nothing to compare
         else:
             assert exe.setOption("decode_mfma", 0)
-            native_loop(n_layers)
-            evv, _ = native_loop(steps)
+            native_loop(2 * n_layers)
+            evv, _ = native_loop(n_x)
             assert exe.setOption("decode_mfma", 1)
-            r["vector_pipe_us"] = evv / steps * 1e3
+            r["vector_pipe_us"] = evv / n_x * 1e3
 
         # ---- a plain streaming read of the same number of bytes from the same pools
         each = min(c.kv_bytes // 2 // 16 * 16, pool_bytes)
-        ms_r = C.c_float()
-        bl.mlc_bench_read_loop(kp, vp, C.c_size_t(n_layers), C.c_size_t(each), C.c_size_t(n_layers), C.byref(ms_r))
-        assert bl.mlc_bench_read_loop(kp, vp, C.c_size_t(n_layers), C.c_size_t(each), C.c_size_t(steps), C.byref(ms_r))
-        r["stream_read"] = {"bytes": 2 * each, "us_per_launch": ms_r.value / steps * 1e3}
+        r["stream_read"] = stream_read_sweep(bl, kp, vp, n_layers, each, N_CU)
 
     # ---- the layer as the batched step runs it (batched_walker.cpp:304-331): write the step's
     # new K row and V row (they land on the newest position: the bytes read stay the same), then
@@ -691,15 +701,19 @@ def run_decode(args, name: str, steps: int, warmup: int, cpu_budget: float, full
     ids = np.array([c.page_tables_flat[c.page_table_offsets[i] + last[i] // c.page_size] if c.seq_lens[i] else 0
                     for i in range(c.batch)], np.uint32)
     slots = (last % c.page_size).astype(np.uint32)
-    n_w = max(1, min(steps, 500))
+    n_w = 500
     ms_w, wall_w = C.c_float(), C.c_double()
-    ok = bl.mlc_bench_decode_step_loop(
-        C.c_void_p(q_buf), kp, vp, C.c_size_t(n_layers), C.c_void_p(o_buf), C.c_void_p(nk_buf), C.c_void_p(nv_buf),
-        ids.ctypes.data_as(u32p), slots.ctypes.data_as(u32p),
-        meta[0].ctypes.data_as(u32p), C.c_size_t(meta[0].size), meta[1].ctypes.data_as(u32p),
-        meta[2].ctypes.data_as(u32p), meta[3].ctypes.data_as(u32p), C.c_size_t(c.batch),
-        C.c_size_t(c.num_heads), C.c_size_t(c.kv_heads), C.c_size_t(c.head_dim), C.c_size_t(c.page_size),
-        C.c_size_t(n_w), C.byref(ms_w), C.byref(wall_w))
+
+    def step_loop(n: int):
+        return bl.mlc_bench_decode_step_loop(
+            C.c_void_p(q_buf), kp, vp, C.c_size_t(n_layers), C.c_void_p(o_buf), C.c_void_p(nk_buf), C.c_void_p(nv_buf),
+            ids.ctypes.data_as(u32p), slots.ctypes.data_as(u32p),
+            meta[0].ctypes.data_as(u32p), C.c_size_t(meta[0].size), meta[1].ctypes.data_as(u32p),
+            meta[2].ctypes.data_as(u32p), meta[3].ctypes.data_as(u32p), C.c_size_t(c.batch),
+            C.c_size_t(c.num_heads), C.c_size_t(c.kv_heads), C.c_size_t(c.head_dim), C.c_size_t(c.page_size),
+            C.c_size_t(n), C.byref(ms_w), C.byref(wall_w))
+
+    ok = step_loop(2 * n_layers) and step_loop(n_w)
     if not ok:
         raise RuntimeError("decode step loop failed: " + exe.lastError())
     r["kv_write_us"] = ms_w.value / n_w * 1e3
@@ -732,6 +746,46 @@ def run_decode(args, name: str, steps: int, warmup: int, cpu_budget: float, full
         r["parity"] = {"min_cosine": round(worst_cos, 7), "max_abs": float(f"{worst_abs:.3e}"),
                        "requests_checked": len(outs)}
     return r
+
+
+def stream_read_sweep(bl, kp, vp, n_layers: int, each: int, n_cu: int, launches: int = 300) -> dict:
+    """The practical ceiling of the memory system for a launch that reads `each` bytes of a K pool and
+    of a V pool and does nothing else: the streaming-read kernels of csrc/bench_loop.cpp (loads into
+    registers with 1..8 independent 16-byte loads per tensor in flight per lane, and global -> LDS
+    loads shaped like the decode kernel's tile loads) swept over 1, 2, 4 and 8 workgroups per CU,
+    each timed like the decode loop (same pools, rotated, HIP events around `launches` launches).
+    Reports the best average, the best block of a repeat run of that combination, and the untuned
+    grid-stride kernel."""
+    import ctypes as C
+    ms = C.c_float()
+
+    def tuned(kind, unroll, grid, n):
+        ok = bl.mlc_bench_read_tuned_loop(kp, vp, C.c_size_t(n_layers), C.c_size_t(each), C.c_size_t(n),
+                                          C.c_int(kind), C.c_int(unroll), C.c_uint(grid), C.byref(ms))
+        return ms.value / n * 1e3 if ok else None
+
+    bl.mlc_bench_read_loop(kp, vp, C.c_size_t(n_layers), C.c_size_t(each), C.c_size_t(n_layers), C.byref(ms))
+    assert bl.mlc_bench_read_loop(kp, vp, C.c_size_t(n_layers), C.c_size_t(each), C.c_size_t(launches), C.byref(ms))
+    plain_us = ms.value / launches * 1e3
+    rows = []
+    for kind, unrolls in ((0, (1, 2, 4, 8)), (1, (1, 2, 4))):
+        for u in unrolls:
+            for per_cu in (1, 2, 4, 8):
+                if kind == 1 and per_cu * 2 * 2 * u * 4096 > 160 * 1024:
+                    continue   # the LDS stages of that many workgroups do not fit a CU
+                grid = n_cu * per_cu
+                if tuned(kind, u, grid, n_layers) is None:
+                    continue
+                rows.append({"kind": "registers" if kind == 0 else "global->LDS", "loads_in_flight_per_lane": 2 * u * (1 if kind == 0 else 2),
+                             "wgs_per_cu": per_cu, "us": round(tuned(kind, u, grid, launches), 3),
+                             "_k": kind, "_u": u, "_g": grid})
+    best = min(rows, key=lambda x: x["us"])
+    blocks = [tuned(best["_k"], best["_u"], best["_g"], 100) for _ in range(10)]
+    for x in rows:
+        for k in ("_k", "_u", "_g"):
+            x.pop(k, None)
+    return {"bytes": 2 * each, "us_per_launch": best["us"], "best": best, "best_block_of_100_us": round(min(blocks), 3),
+            "untuned_grid_stride_us": round(plain_us, 3), "sweep": rows}
 
 
 def workload_text(c, n_layers) -> str:
@@ -829,6 +883,8 @@ def main() -> int:
                     help="0 = automatic (tile-balanced kernel), 1 = planned split-K items")
     ap.add_argument("--wgs-per-cu", type=int, default=0, help="tile-balanced kernel: workgroups per CU (0 = automatic)")
     ap.add_argument("--stages", type=int, default=0, help="tile-balanced kernel: LDS stages (0 = automatic)")
+    ap.add_argument("--read-sweep", action="store_true",
+                    help="decode: print every row of the streaming-read sweep, not only the best")
     ap.add_argument("--probe", action="store_true",
                     help="decode: print the per-workgroup timeline of the last launch as config.probe_timeline "
                          "(needs a library built with MLC_HIPCC_EXTRA=-DMLC_STREAM_PROBE; its times mean nothing)")
@@ -932,8 +988,12 @@ def main() -> int:
             "stream_read_ceiling": {"bytes": sr["bytes"], "us_per_launch": round(sr["us_per_launch"], 3),
                                     "GBs": round(sr["bytes"] / sr["us_per_launch"] / 1e3, 1),
                                     "frac": round(sr["bytes"] / sr["us_per_launch"] / 1e3 / HBM_PEAK_GBS, 4),
-                                    "note": "a kernel that only reads the same number of bytes contiguously from "
-                                            "the same pools, same run, same timing"},
+                                    "best": sr["best"], "best_block_of_100_us": sr["best_block_of_100_us"],
+                                    "untuned_grid_stride_us": sr["untuned_grid_stride_us"],
+                                    **({"sweep": sr["sweep"]} if args.read_sweep else {}),
+                                    "note": "kernels that only read the same number of bytes contiguously from the "
+                                            "same pools, same run, same timing: best of a sweep over loads in "
+                                            "flight per lane (registers or global->LDS) and workgroups per CU"},
             "note": "HIP events around the timed region on the library stream / steps: one step = one "
                     "decode kernel (split requests are merged inside it by the last workgroup to arrive)",
         },

@@ -291,7 +291,10 @@ int mlc_hip_paged_attn_decode_noalloc(const void* q, const void* k_pages, const 
  * the pass once uncaptured first, which puts weights, norm vectors and tables on the device.  The
  * decode attention of a captured pass must be served by the tile-balanced kernel (head_dim 64 or
  * 128, page size a multiple of its tile, 16-byte aligned buffers).  mlc_hip_capture_end returns a
- * handle > 0, or 0 (then nothing was kept; encode the pass uncaptured).
+ * handle > 0, or 0 (then nothing was kept; encode the pass uncaptured).  mlc_hip_captured_launches
+ * counts the launches of the encode calls; the pass holds one more, the library's own first launch,
+ * which moves a device word on by which the decode launches of one replay tell their split-K
+ * partials from those of the replay before.
  *
  * mlc_hip_replay_update copies the step's tables over the device copies the captured launches
  * read (same addresses, ordered on the library's stream) and checks what the capture took for

@@ -22,8 +22,7 @@ __global__ __launch_bounds__(256) void mlc_bench_copy_kernel(const uint4* __rest
 
 // Plain streaming read: every thread loads 16-byte units with a grid stride and folds them into
 // one word that is stored only if it has a value it never has.  The same number of bytes as a
-// decode launch, read contiguously with nothing else to do: the practical ceiling of the memory
-// system for a launch of that size, quoted beside the decode kernel.
+// decode launch, read contiguously with nothing else to do.
 __global__ __launch_bounds__(256) void mlc_bench_read_kernel(const uint4* __restrict__ a, const uint4* __restrict__ b,
                                                              size_t n_each, uint32_t* sink) {
     uint32_t acc = 0;
@@ -33,6 +32,80 @@ __global__ __launch_bounds__(256) void mlc_bench_read_kernel(const uint4* __rest
         acc ^= x.x ^ x.y ^ x.z ^ x.w ^ y.x ^ y.y ^ y.z ^ y.w;
     }
     if (acc == 0x9E3779B9u && sink) sink[0] = acc;
+}
+
+// Tuned streaming read, into registers: a workgroup takes 256 * U consecutive 16-byte units of each
+// tensor per trip, so every lane has 2 * U independent 16-byte loads in flight before it folds
+// any of them (the plain kernel above has two).  The grid is persistent (a few workgroups per CU)
+// and swept by the caller.  This is the yardstick for what the memory system delivers to a launch
+// of a given size with nothing else to do.
+template <int U>
+__global__ __launch_bounds__(256) void mlc_bench_read_unrolled_kernel(const uint4* __restrict__ a,
+                                                                      const uint4* __restrict__ b, size_t n_each,
+                                                                      uint32_t* sink) {
+    uint32_t acc = 0;
+    const size_t stride = (size_t)gridDim.x * 256 * U;
+    size_t i = (size_t)blockIdx.x * 256 * U + threadIdx.x;
+    for (; i + (size_t)(U - 1) * 256 < n_each; i += stride) {
+        uint4 x[U], y[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) x[u] = a[i + (size_t)u * 256];
+#pragma unroll
+        for (int u = 0; u < U; ++u) y[u] = b[i + (size_t)u * 256];
+#pragma unroll
+        for (int u = 0; u < U; ++u) acc ^= x[u].x ^ x[u].y ^ x[u].z ^ x[u].w ^ y[u].x ^ y[u].y ^ y[u].z ^ y[u].w;
+    }
+    for (int u = 0; u < U; ++u) {   // the ragged end of the last trip
+        const size_t j = i + (size_t)u * 256;
+        if (j < n_each) {
+            const uint4 x = a[j], y = b[j];
+            acc ^= x.x ^ x.y ^ x.z ^ x.w ^ y.x ^ y.y ^ y.z ^ y.w;
+        }
+    }
+    if (acc == 0x9E3779B9u && sink) sink[0] = acc;
+}
+
+// Tuned streaming read, global -> LDS, shaped like the decode kernel's tile loads: every wave
+// moves 1 KiB per instruction straight into LDS (no registers), U instructions per tensor and
+// trip, two trips in flight (the next trip is requested before the current one is waited for).
+// Units past the end are clamped onto the last one (in bounds, read twice).
+template <int U>
+__global__ __launch_bounds__(256) void mlc_bench_read_lds_kernel(const uint4* __restrict__ a, const uint4* __restrict__ b,
+                                                                 size_t n_each, uint32_t* sink) {
+    __shared__ __attribute__((aligned(16))) unsigned char stage[2][2 * U * 4096];
+    const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const uint32_t base = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)&stage[0][0];
+    const size_t stride = (size_t)gridDim.x * 256 * U;
+    const size_t first = (size_t)blockIdx.x * 256 * U + threadIdx.x;
+    auto issue = [&](size_t i, uint32_t buf) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const uint4* src = t ? b : a;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                size_t j = i + (size_t)u * 256;
+                j = j < n_each ? j : n_each - 1;
+                const uint32_t dst = __builtin_amdgcn_readfirstlane(base + buf * (2 * U * 4096) + (t * U + u) * 4096 + wave * 1024);
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(dst), "v"(src + j) : "memory", "m0");
+            }
+        }
+    };
+    if (first >= n_each) return;
+    uint32_t buf = 0;
+    issue(first, 0);
+    for (size_t i = first; i < n_each; i += stride) {
+        const bool more = i + stride < n_each;
+        if (more) {
+            issue(i + stride, buf ^ 1u);
+            asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * U) : "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        buf ^= 1u;
+    }
+    // one word of what landed, so that the loads have a consumer
+    const uint32_t w = reinterpret_cast<const uint32_t*>(&stage[0][0])[lane];
+    if (w == 0x9E3779B9u && sink) sink[0] = w;
 }
 
 extern "C" {
@@ -51,6 +124,34 @@ int mlc_bench_read_loop(void* const* k_pools, void* const* v_pools, size_t n_lay
     for (size_t i = 0; i < steps; ++i)
         hipLaunchKernelGGL(mlc_bench_read_kernel, dim3(grid), dim3(256), 0, stream,
                            static_cast<const uint4*>(k_pools[i % n_layers]),
+                           static_cast<const uint4*>(v_pools[i % n_layers]), n, static_cast<uint32_t*>(nullptr));
+    const float ms = mlc_hip_timer_stop();
+    if (ms < 0.f) return 0;
+    if (event_ms) *event_ms = ms;
+    return 1;
+}
+
+// The tuned reads: kind 0 = into registers, 1 = global -> LDS; unroll = 16-byte loads per tensor
+// and trip (1, 2, 4 or 8); grid = workgroups of 256 threads.  Same rotation over the pools and the
+// same timing as mlc_bench_read_loop.  Returns 0 for a combination that is not built.
+int mlc_bench_read_tuned_loop(void* const* k_pools, void* const* v_pools, size_t n_layers, size_t bytes_each,
+                              size_t steps, int kind, int unroll, unsigned grid, float* event_ms) {
+    hipStream_t stream = static_cast<hipStream_t>(mlc_hip_stream());
+    if (!stream || !k_pools || !v_pools || !n_layers || !grid) return 0;
+    const size_t n = bytes_each / 16;
+    if (!n) return 0;
+    void (*kern)(const uint4*, const uint4*, size_t, uint32_t*) = nullptr;
+    if (kind == 0) {
+        kern = unroll == 1 ? mlc_bench_read_unrolled_kernel<1> : unroll == 2 ? mlc_bench_read_unrolled_kernel<2>
+             : unroll == 4 ? mlc_bench_read_unrolled_kernel<4> : unroll == 8 ? mlc_bench_read_unrolled_kernel<8> : nullptr;
+    } else if (kind == 1) {
+        kern = unroll == 1 ? mlc_bench_read_lds_kernel<1> : unroll == 2 ? mlc_bench_read_lds_kernel<2>
+             : unroll == 4 ? mlc_bench_read_lds_kernel<4> : nullptr;
+    }
+    if (!kern) return 0;
+    if (!mlc_hip_timer_start()) return 0;
+    for (size_t i = 0; i < steps; ++i)
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), 0, stream, static_cast<const uint4*>(k_pools[i % n_layers]),
                            static_cast<const uint4*>(v_pools[i % n_layers]), n, static_cast<uint32_t*>(nullptr));
     const float ms = mlc_hip_timer_stop();
     if (ms < 0.f) return 0;

@@ -78,17 +78,23 @@ struct MetaSlot {
     bool pending = false;
 };
 
-// Scratch memory of the tile-balanced decode kernel: split-K partials (two slots per workgroup)
-// and arrival counters.  A file-scope device array, so that no entry point that uses it has to
-// allocate; every GPU the library runs on holds its own copy at its own address, which host
-// code learns from hipGetSymbolAddress (the array's name is not a device address in host code).
-// The arrival counters are zero when the module is loaded and every merge puts its counter
-// back to zero.  Launches on one GPU share the array: they must not overlap.
-constexpr size_t kScratchPartOBytes = 8u << 20;
-constexpr size_t kScratchPartMlBytes = 512u << 10;
-constexpr size_t kScratchCounterBytes = (size_t)kStreamMaxWgs * 4 * sizeof(uint32_t);
-constexpr size_t kScratchBytes = kScratchPartOBytes + kScratchPartMlBytes + kScratchCounterBytes;
+// Scratch memory of the tile-balanced decode kernel: the split-K partials (one slot per
+// workgroup, tagged words that say by themselves whether they were written in the current
+// launch, so nothing has to be cleared between launches), the replay word of captured passes,
+// and, in probe builds, the time stamps.  A file-scope device array, so that no entry point
+// that uses it has to allocate; every GPU the library runs on holds its own copy at its own
+// address, which host code learns from hipGetSymbolAddress (the array's name is not a device
+// address in host code).  Launches on one GPU share the array: they must not overlap.
+constexpr size_t kScratchProbeBytes = (size_t)kStreamMaxWgs * 256;
+constexpr size_t kScratchReplayWordOffset = kStreamPartBytes + kScratchProbeBytes;
+constexpr size_t kScratchBytes = kScratchReplayWordOffset + 256;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+// First launch of every captured pass: moves the replay word on, so that the decode launches of
+// this replay (whose arguments, tag included, are the same at every replay) use tags that the
+// replay before did not.
+__global__ void replay_word_kernel(uint32_t* word, uint32_t step) { *word += step; }
+constexpr uint32_t kReplayTagStep = 4096;   // decode launches of one captured pass, at most
 
 // Device copy of the flat page table (and, where the per-request arrays do not travel inside the
 // kernel arguments, of those arrays) as the tile-balanced decode kernel reads it; uploaded only
@@ -233,6 +239,14 @@ struct Ctx {
     char last_kernel[96] = "";   // kernel variant of the last decode launch (for benchmarks)
     int n_cu = 256;
     unsigned char* scratch_ptr = nullptr;   // device address of `scratch` on g.device
+    uint32_t next_tag = 0;                  // tag of the last tile-balanced decode launch (never zero)
+    // One word of pinned host memory that the decode kernel sets (through its device address) when a
+    // merge gives up waiting for another workgroup's partial; looked at wherever the host has
+    // waited for the stream.
+    volatile uint32_t* fault_host = nullptr;
+    uint32_t* fault_dev = nullptr;
+    long opt_spin_limit = 200000;           // rounds a merge polls before it gives up (about 0.1 s)
+    long opt_test_flags = 0;                // bit 0: workgroups do not publish their partials (tests of the give-up path)
     StreamTables tables;
     long opt_decode_kernel = 0;     // 0 = automatic (tile-balanced where it applies), 1 = planned items, 2 = tile-balanced
     long opt_wgs_per_cu = 0;        // tile-balanced kernel: workgroups per CU (0 = automatic)
@@ -260,6 +274,7 @@ struct Ctx {
         size_t B = 0, H = 0, Hkv = 0, D = 0, P = 0;
         int causal = 0;
         bool carried_kv = false;             // ... and does the step's KV write
+        size_t n_decode = 0;                 // tile-balanced decode launches of the pass
         const void* ids_dev = nullptr;       // device copy of the KV write's page ids and slots
         size_t ids_batch = 0;
     };
@@ -293,6 +308,18 @@ bool init_once() {
         return false;
     }
     g.scratch_ptr = static_cast<unsigned char*>(sp);
+    {
+        void* fh = nullptr;
+        void* fd = nullptr;
+        if (hipHostMalloc(&fh, 64, hipHostMallocMapped) != hipSuccess || !fh ||
+            hipHostGetDevicePointer(&fd, fh, 0) != hipSuccess || !fd) {
+            g_err = "hipHostMalloc(fault word) failed";
+            return false;
+        }
+        g.fault_host = static_cast<volatile uint32_t*>(fh);
+        *g.fault_host = 0;
+        g.fault_dev = static_cast<uint32_t*>(fd);
+    }
     if (hipStreamCreateWithFlags(&g.stream, hipStreamNonBlocking) != hipSuccess) return false;
     if (hipEventCreate(&g.ev0) != hipSuccess || hipEventCreate(&g.ev1) != hipSuccess) return false;
     g.available = true;
@@ -519,12 +546,23 @@ void rows_begin(const void* src, size_t batch, size_t len) {
     r.cur = src;
 }
 
+// After a wait for the stream: did a decode launch give up on a partial?
+int check_fault() {
+    if (g.fault_host && *g.fault_host) {
+        *g.fault_host = 0;
+        return fail("decode: a workgroup gave up waiting for another workgroup's partial result; the outputs of this "
+                    "pass are not valid (launches that share the library's scratch memory must not overlap)");
+    }
+    return 1;
+}
+
 int finish(int sync) {
     HIP_OK(hipGetLastError());
     if (sync) {
         NOT_WHILE_CAPTURING("a call with sync = 1");
         if (!settle()) return 0;
         HIP_OK(hipStreamSynchronize(g.stream));
+        return check_fault();
     }
     return 1;
 }
@@ -916,8 +954,8 @@ unsigned stream_grid(size_t G, size_t D, int nbuf, size_t dyn_lds) {
     size_t W = (size_t)g.n_cu * per_cu;
     if (g.opt_grid_wgs > 0) W = (size_t)g.opt_grid_wgs;
     W = std::min<size_t>(W, kStreamMaxWgs);
-    W = std::min<size_t>(W, kScratchPartOBytes / (2 * G * D * 4));
-    W = std::min<size_t>(W, kScratchPartMlBytes / (2 * G * 2 * 4));
+    int hpw = 1, nw = 1;
+    if (stream_variant(G, D, &hpw, &nw)) W = std::min<size_t>(W, kStreamPartBytes / stream_partial_bytes(G, D, (size_t)nw));
     return (unsigned)std::max<size_t>(W, 1);
 }
 
@@ -925,7 +963,7 @@ uint32_t stream_pair_cost(int nw, size_t G, size_t D) {
     if (g.opt_pair_cost >= 0) return (uint32_t)g.opt_pair_cost;
     (void)G;
     (void)D;
-    return nw == 4 ? 4u : 0u;
+    return nw == 4 ? 3u : 0u;
 }
 
 // Arithmetic mode of the tile-balanced kernel: 0 fp32 softmax weights, 1 fp16 weights on the vector
@@ -956,9 +994,20 @@ void stream_fill_common(StreamArgs& a, const void* q, const void* k_pages, const
     a.k_pages = static_cast<const uint4*>(k_pages);
     a.v_pages = static_cast<const uint4*>(v_pages);
     a.o = static_cast<float*>(o);
-    a.part_o = reinterpret_cast<float*>(g.scratch_ptr);
-    a.part_ml = reinterpret_cast<float*>(g.scratch_ptr + kScratchPartOBytes);
-    a.counters = reinterpret_cast<uint32_t*>(g.scratch_ptr + kScratchPartOBytes + kScratchPartMlBytes);
+    a.part = reinterpret_cast<uint64_t*>(g.scratch_ptr);
+    a.fault = g.fault_dev;
+    a.spin_limit = (uint32_t)g.opt_spin_limit;
+    a.test_flags = (uint32_t)g.opt_test_flags;
+    if (g_capturing) {
+        // the arguments of a captured launch are the same at every replay: its tag is its number in
+        // the pass plus the replay word, which the pass's first launch moves on by kReplayTagStep
+        a.tag = 0x80000000u | (uint32_t)g.cap.n_decode++;
+        a.tag_dev = reinterpret_cast<const uint32_t*>(g.scratch_ptr + kScratchReplayWordOffset);
+    } else {
+        if (++g.next_tag == 0) ++g.next_tag;   // (zero is what untouched memory holds)
+        a.tag = g.next_tag;
+        a.tag_dev = nullptr;
+    }
     a.batch = (uint32_t)B;
     a.num_heads = (uint32_t)H;
     a.kv_heads = (uint32_t)Hkv;
@@ -1087,7 +1136,7 @@ int mlc_hip_flush(void) {
     if (!g.pass_open) return 1;
     g.pass_open = false;
     HIP_OK(hipStreamSynchronize(g.stream));
-    return 1;
+    return check_fault();
 }
 
 int mlc_hip_has_open_pass(void) { return (g.inited && g.pass_open) ? 1 : 0; }
@@ -1206,7 +1255,9 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
         std::memcpy(meta3.data() + 2 * batch, page_table_offsets, batch * 4);
         // ... and the flat table with them when it fits behind them: then nothing is copied to the
         // device, however often the tables change
-        const bool embed_table = embed && 3 * batch + n_flat <= kStreamEmbWords;
+        // (up to 64 requests: the arrays sit at a fixed stride, see the kernel)
+        const size_t emb_stride = batch <= 64 ? kStreamSmallStride : batch;
+        const bool embed_table = embed && 3 * emb_stride + n_flat <= kStreamEmbWords;
         const uint32_t* d_flat = nullptr;
         const uint32_t* d_meta = nullptr;
         if (!embed_table && !tables_upload(embed ? nullptr : meta3.data(), batch, &d_flat, &d_meta)) return 0;
@@ -1229,8 +1280,8 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
         }
         a.meta_stride = (uint32_t)batch;
         if (embed) {
-            std::memcpy(a.emb, meta3.data(), 3 * batch * 4);
-            if (embed_table && n_flat) std::memcpy(a.emb + 3 * batch, page_tables_flat, n_flat * 4);
+            for (int i = 0; i < 3; ++i) std::memcpy(a.emb + i * emb_stride, meta3.data() + i * batch, batch * 4);
+            if (embed_table && n_flat) std::memcpy(a.emb + 3 * emb_stride, page_tables_flat, n_flat * 4);
         } else {
             a.meta = d_meta;
         }
@@ -1240,6 +1291,8 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
             a.new_ids = g.kv.d_ids;
             a.new_slots = g.kv.d_slots;
         }
+        if (g_capturing && g.cap.n_decode > kReplayTagStep)
+            return fail("capture: more decode launches in one pass than its tags can tell apart");
         if (!launch_stream_variant(head_dim, s_hpw, s_nw, nbuf, a, n_wg, dyn_lds, g.stream))
             return fail("decode: kernel variant not built");
         if (g_capturing) {
@@ -1389,9 +1442,10 @@ int mlc_hip_paged_attn_decode_noalloc(const void* q, const void* k_pages, const 
         if (pages != SIZE_MAX) a.capacity_pages = (uint32_t)std::min<size_t>(pages, 0xFFFFFFFFu);
     }
     a.meta_stride = (uint32_t)batch;
+    const size_t emb_stride = batch <= 64 ? kStreamSmallStride : batch;
     std::memcpy(a.emb, seq_lens, batch * 4);
-    std::memcpy(a.emb + batch, q_positions, batch * 4);
-    std::memcpy(a.emb + 2 * batch, page_table_offsets, batch * 4);
+    std::memcpy(a.emb + emb_stride, q_positions, batch * 4);
+    std::memcpy(a.emb + 2 * emb_stride, page_table_offsets, batch * 4);
     hipStream_t st = stream ? static_cast<hipStream_t>(stream) : g.stream;
     if (!launch_stream_variant(head_dim, hpw, nw, nbuf, a, n_wg, dyn_lds, st))
         return fail("decode: kernel variant not built");
@@ -2239,6 +2293,8 @@ int mlc_hip_capture_begin(void) {
     g_capture_failed = false;
     HIP_OK(hipStreamBeginCapture(g.stream, hipStreamCaptureModeThreadLocal));
     g_capturing = true;
+    hipLaunchKernelGGL(replay_word_kernel, dim3(1), dim3(1), 0, g.stream,
+                       reinterpret_cast<uint32_t*>(g.scratch_ptr + kScratchReplayWordOffset), kReplayTagStep);
     return 1;
 }
 
@@ -2270,9 +2326,9 @@ int mlc_hip_capture_end(void) {
         hipGraphNodeType type;
         ok = hipGraphNodeGetType(nodes[i], &type) == hipSuccess && type == hipGraphNodeTypeKernel;
     }
-    if (!ok || count == 0) {
+    if (!ok || count <= 1) {
         (void)hipGraphDestroy(graph);
-        return fail(count == 0 ? "capture: nothing was encoded" : "capture: the pass holds something other than kernel launches");
+        return fail(count <= 1 ? "capture: nothing was encoded" : "capture: the pass holds something other than kernel launches");
     }
     hipGraphExec_t exec = nullptr;
     if (hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0) != hipSuccess || !exec) {
@@ -2283,7 +2339,7 @@ int mlc_hip_capture_end(void) {
     Ctx::Captured c = g.cap;
     c.graph = graph;
     c.exec = exec;
-    c.n_nodes = count;
+    c.n_nodes = count - 1;   // (not counted: the library's own first launch, which moves the replay word on)
     const int handle = g.next_capture++;
     g.captures[handle] = c;
     return handle;
@@ -2414,7 +2470,7 @@ long mlc_hip_decode_table_uploads(void) { return g.table_uploads; }
 int mlc_hip_debug_probe(uint64_t* dst, size_t n_wg) {
     if (!init_once()) return 0;
     HIP_OK(hipStreamSynchronize(g.stream));
-    HIP_OK(hipMemcpy(dst, g.scratch_ptr + kScratchPartOBytes + 65536 * 4, n_wg * 256, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(dst, g.scratch_ptr + kStreamPartBytes, n_wg * 256, hipMemcpyDeviceToHost));
     return 1;
 }
 #endif
@@ -2461,6 +2517,16 @@ int mlc_hip_set_option(const char* name, long value) {
     if (!std::strcmp(name, "decode_pair_cost")) {
         if (value < -1 || value > 64) return 0;
         g.opt_pair_cost = value;
+        return 1;
+    }
+    if (!std::strcmp(name, "decode_spin_limit")) {
+        if (value < 1 || value > 0x7FFFFFFFl) return 0;
+        g.opt_spin_limit = value;
+        return 1;
+    }
+    if (!std::strcmp(name, "decode_test_flags")) {
+        if (value < 0 || value > 1) return 0;
+        g.opt_test_flags = value;
         return 1;
     }
     if (!std::strcmp(name, "decode_mfma")) {

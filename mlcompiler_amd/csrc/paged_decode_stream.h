@@ -14,23 +14,28 @@
 //     softmax state is kept across the tiles of a pair and finalised when the pair (or the
 //     range) ends.
 //   * A pair that lies inside one range is written to O directly.  A pair cut by range
-//     boundaries is published as partials by the workgroups that share it (at most two
-//     partials per workgroup: the first and the last pair of its range); the last of them
-//     to arrive merges.  Which workgroups share a pair follows from the numbering, so
+//     boundaries is summed up by the workgroup that holds its last tile, from the partials
+//     the other workgroups that share it leave behind (one per workgroup: the pair that goes
+//     on behind its range).  Which workgroups share a pair follows from the numbering, so
 //     nobody needs a list.
 //   * The per-request arrays (lengths, query positions, page-table offsets) either travel
-//     inside the kernel arguments or are read from device memory; the flat page table is
-//     always in device memory.  Nothing is planned on the host.
+//     inside the kernel arguments or are read from device memory, and so does the flat page
+//     table.  Nothing is planned on the host.
 #pragma once
 
 #include "paged_decode_kernels.h"
 
 namespace mlc_hip {
 
+static constexpr uint32_t kStreamSmallStride = 64;  // stride of the embedded arrays of up to 64 requests
 static constexpr uint32_t kStreamEmbBatch = 256;    // requests whose arrays fit the kernel arguments
 static constexpr uint32_t kStreamEmbWords = 960;    // words of the kernel arguments that carry tables
 static constexpr uint32_t kStreamMaxBatch = 4096;   // 64-ary search over the tile prefix in two levels
 static constexpr uint32_t kStreamMaxWgs = 2048;     // workgroups per launch, at most
+static constexpr size_t kStreamPartBytes = 8u << 20;  // the partial buffer
+static constexpr size_t kStreamProbeWord = kStreamPartBytes / 8;  // probe builds: time stamps behind the partials
+// Words per lane of a workgroup's partial (see the kernel): NW waves x (OPL + 1) words.
+constexpr size_t stream_partial_bytes(size_t G, size_t D, size_t NW) { return (G * D + 64 * NW) * 8; }
 
 struct StreamArgs {
     const float* q;             // [B][H][D]
@@ -39,10 +44,12 @@ struct StreamArgs {
     float* o;                   // [B][H][D]
     const uint32_t* pt_flat;    // device copy of page_tables_flat; null: the table is in emb, behind the arrays
     const uint32_t* meta;       // device [3][meta_stride]: seq_lens, q_positions, page_table_offsets;
-                                // null: the arrays are in emb (same layout)
-    float* part_o;              // [2 * n_wg][G][D] un-normalised partial outputs
-    float* part_ml;             // [2 * n_wg][G][2] (m in log2 units, l)
-    uint32_t* counters;         // [n_wg][NW] arrival counters, zero between launches
+                                // null: the arrays are in emb
+    uint64_t* part;             // [n_wg][NW][OPL + 1][64] tagged words {value, launch tag}: one partial per
+                                // workgroup (OPL = query heads per wave * D / 64)
+    const uint32_t* tag_dev;    // null, or a device word that is added to `tag` (captured passes: the
+                                // arguments are the same at every replay, the word is not)
+    uint32_t* fault;            // host-visible word, set when a merge gave up waiting for a partial
     uint32_t batch;
     uint32_t num_heads;
     uint32_t kv_heads;
@@ -52,6 +59,10 @@ struct StreamArgs {
     uint32_t meta_stride;
     float scale_log2e;          // log2(e) / sqrt(D)
     uint32_t pair_cost;         // units a pair's end counts for when the ranges are cut (0: tiles only)
+    uint32_t tag;               // this launch's tag: differs from that of every earlier launch whose
+                                // partials may still lie in `part`
+    uint32_t spin_limit;        // rounds a merge polls for its partials before it gives up
+    uint32_t test_flags;        // bit 0: partials are not published (tests of the give-up path)
     // The step's KV write done by this launch (null: none), as in DecodeArgs: the workgroup
     // that owns a pair's last tile writes that pair's slice of the new rows before it loads
     // anything.
@@ -59,8 +70,9 @@ struct StreamArgs {
     const uint4* new_v;
     const uint32_t* new_ids;
     const uint32_t* new_slots;
-    // seq_lens | q_positions | page_table_offsets (meta_stride words each) and, where it fits as
-    // well, the flat page table: a call whose tables travel here copies nothing to the device
+    // seq_lens | q_positions | page_table_offsets (at a stride of 64 words for up to 64 requests,
+    // of meta_stride words above) and, where it fits as well, the flat page table behind them: a
+    // call whose tables travel here copies nothing to the device
     uint32_t emb[kStreamEmbWords];
 };
 static_assert(sizeof(StreamArgs) <= 4096, "kernel arguments are limited to 4 KiB");
@@ -82,7 +94,7 @@ inline size_t stream_dynamic_lds_bytes(size_t batch) { return (4 * batch + 2) * 
 #define MLC_PROBE(i)                                                                                   \
     do {                                                                                               \
         if (threadIdx.x == 0)                                                                          \
-            reinterpret_cast<uint64_t*>(a.part_ml + 65536)[blockIdx.x * 32 + (i)] = __builtin_amdgcn_s_memrealtime(); \
+            (a.part + kStreamProbeWord)[blockIdx.x * 32 + (i)] = __builtin_amdgcn_s_memrealtime(); \
     } while (0)
 #else
 #define MLC_PROBE(i)
@@ -117,6 +129,15 @@ __device__ __forceinline__ void sd_wait_vmcnt() {
 // Workgroup barrier that orders LDS traffic only (global -> LDS loads stay in flight across it).
 __device__ __forceinline__ void sd_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// A word of a partial: {value, tag}, written and read whole (64-bit relaxed atomics at device
+// scope: the store is written through to memory, the load bypasses the per-XCD L2 caches).
+__device__ __forceinline__ void st_tagged(uint64_t* p, uint64_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint64_t ld_tagged(const uint64_t* p) {
+    return __hip_atomic_load(const_cast<uint64_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // exclusive-to-inclusive prefix sum over the 64 lanes in six DPP steps (no LDS traffic)
@@ -172,19 +193,31 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     uint32_t* s_nzb = s_off + B;           // [B + 1] requests with tiles before r
 
     MLC_PROBE(0);
+    // The embedded per-request arrays of a small batch are requested before anything else: their
+    // address is the argument segment's, which a wave knows when it starts.
+    uint32_t e_seq = 0, e_qp = 0, e_off = 0;
+    if constexpr (SMALL) {
+        const uint32_t l0 = threadIdx.x % 64;
+        e_seq = a.emb[l0];
+        e_qp = a.emb[kStreamSmallStride + l0];
+        e_off = a.emb[2 * kStreamSmallStride + l0];
+        __builtin_amdgcn_sched_barrier(0);
+    }
     // Everything the prologue needs from the kernel arguments is requested now, in one go: left
     // to the compiler, each would be fetched where it is first used, one memory round trip after
     // the other on the way to the first tile load.
     {
         const uint64_t p0 = (uint64_t)a.q, p1 = (uint64_t)a.k_pages, p2 = (uint64_t)a.v_pages, p3 = (uint64_t)a.pt_flat,
-                       p4 = (uint64_t)a.new_k;
+                       p4 = (uint64_t)a.new_k, p5 = (uint64_t)a.meta, p6 = (uint64_t)a.tag_dev;
         asm volatile("" ::"s"(a.batch), "s"(a.num_heads), "s"(a.kv_heads), "s"(a.page_size), "s"(a.causal),
                      "s"(a.capacity_pages), "s"(a.scale_log2e), "s"(p0), "s"(p1), "s"(p2), "s"(p3), "s"(p4),
-                     "s"(gridDim.x));
+                     "s"(p5), "s"(p6), "s"(a.pair_cost), "s"(a.meta_stride), "s"(gridDim.x));
     }
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const int lane = threadIdx.x % 64;
     const int hg = wave;  // head group of this wave
+    uint32_t tag_add = 0;   // (needed where the range ends; requested now)
+    if (a.tag_dev) tag_add = *a.tag_dev;
     const int c = lane % CPR;
     const int r_l = lane / CPR;
     const int c7 = c & 7;
@@ -201,7 +234,9 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         // The arrays inside the kernel arguments are read before anything else is known (their
         // address is the argument segment's, no pointer has to be fetched first); lanes past
         // the batch read other arguments and are masked.
-        uint32_t seq = a.emb[lane], qp = a.emb[a.meta_stride + lane], off = a.emb[2 * a.meta_stride + lane];
+        // (embedded arrays of up to 64 requests sit at a stride of 64 words, so that these loads go
+        // out before any argument has arrived)
+        uint32_t seq = e_seq, qp = e_qp, off = e_off;
         if (a.meta != nullptr && (uint32_t)lane < B) {
             seq = a.meta[lane];
             qp = a.meta[a.meta_stride + lane];
@@ -221,7 +256,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     } else {
         if (wave == 0) {
             const uint32_t* meta = a.meta ? a.meta : a.emb;
-            const uint32_t stride = a.meta_stride;
+            const uint32_t stride = a.meta_stride;   // (more than 64 requests: the arrays are packed)
             uint32_t carry = 0, carry_nz = 0;
             for (uint32_t b0 = 0; b0 < B; b0 += 64) {
                 const uint32_t i = b0 + lane;
@@ -387,7 +422,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     }
     ci = cc;
 
-    const uint32_t* pt_flat = a.pt_flat ? a.pt_flat : a.emb + 3u * a.meta_stride;
+    const uint32_t* pt_flat = a.pt_flat ? a.pt_flat : a.emb + 3u * (SMALL ? kStreamSmallStride : a.meta_stride);
     // Page ids of the issue side's request, 64 tiles at a time: lane i holds the page of tile
     // pv_win + i.  Refetched when the issue side enters another request or another window.
     uint32_t pv = 0, pv_win = 0, pv_req = 0xFFFFFFFFu;
@@ -435,6 +470,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     auto load_q = [&](const Cursor& cu) {
         if constexpr (MF) {
             const int hcol = n16 < G ? n16 : G - 1;
+            const float q_factor = n16 < G ? a.scale_log2e : 0.f;
             const float* qb = a.q + ((size_t)cu.r * a.num_heads + cu.kvh * G + hcol) * D + 8 * g4;
 #pragma unroll
             for (int ks = 0; ks < KST; ++ks) {
@@ -443,7 +479,10 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
                 const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    const float v = n16 < G ? x[i] * a.scale_log2e : 0.f;
+                    // (columns past the group: the loads are clamped onto the last head and the
+                    // factor is zero; a select on the loaded value would put the load under a
+                    // branch, and the wait for it there would be for every load in flight)
+                    const float v = x[i] * q_factor;
                     const _Float16 hi = (_Float16)v;
                     qh[ks][i] = hi;
                     ql[ks][i] = (_Float16)(v - (float)hi);
@@ -732,16 +771,24 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         }
     };
 
-    // ---- end of a pair's tiles inside this range.  The rows of lanes are summed; a pair that
-    // lay inside the range is written to O at once.  A pair cut by range boundaries becomes a
-    // partial, and nothing about a partial touches memory before the range has ended: a range's
-    // first pair that ends in mid-range is kept in registers (at most one per workgroup: a later
-    // pair that ends inside the range also started inside it), so that the stream never stops for
-    // the round trips of a publication.  At the end of the range the workgroup stores its
-    // partials (one or two), waits for them once, takes the arrival tickets together and merges
-    // where it arrived last.
+    // ---- end of a pair's tiles inside this range.  The rows of lanes are summed; a pair that lay
+    // inside the range is written to O at once.  A pair cut by range boundaries is shared by
+    // consecutive workgroups, and the one that holds its last tile (the highest-numbered sharer)
+    // sums it up: every other sharer leaves its (o, m, l) in its own slot of the partial buffer --
+    // a workgroup has one slot, because only the pair that goes on behind its range is published
+    // -- and is done.  A partial is a set of 64-bit words {value, tag}: the tag is this launch's,
+    // never seen in the buffer before, so every word says by itself whether it has been written
+    // in this launch.  Nothing else is needed: no order among the stores, no acknowledgement, no
+    // arrival counter.  The stores are relaxed device-scope atomics (written through to memory),
+    // the summing workgroup reads with relaxed device-scope loads until every word of every
+    // sharer's partial carries the tag, then folds them in workgroup order and its own part
+    // last, so the result does not depend on timing (runs are bit-identical).  It waits only for
+    // lower-numbered workgroups, which the hardware starts no later than itself; the wait is
+    // bounded all the same (spin_limit rounds, then the fault word is set and the pass fails on
+    // the host).  Nothing about a partial touches memory before the range has ended: a first
+    // pair that ends in mid-range waits in registers, so the stream never stops for it.
     struct PairOut {
-        uint32_t w_lo, n_splits, slot_first, my_slot;
+        uint32_t w_lo;   // first sharer
         float* orow;
     };
     // Brings the rows of lanes (the tokens a lane row owns) onto one reference and sums over
@@ -843,18 +890,12 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     auto out_row = [&](const Cursor& cu) {
         return a.o + ((size_t)cu.r * a.num_heads + cu.kvh * G + hg * HPW) * D;
     };
-    // who shares the pair [ps, pe) and where its partials go.  A workgroup's first pair uses
-    // slot 2w, a later (so: its last) pair slot 2w + 1.
-    auto pair_out = [&](const Cursor& cu, uint32_t ps, uint32_t pe) {
+    // who shares the pair whose first tile is ps
+    auto pair_out = [&](const Cursor& cu, uint32_t ps) {
         PairOut po;
         // the pair's tiles are consecutive units; the PC units in front of them stand for the
-        // end of the pair before, so the first sharer has no tile of that pair (the pair is its
-        // first) exactly when its range starts inside them or at the pair's first tile
-        const uint32_t ups = ps + PC * (Hkv * req_nzb(cu.r) + cu.kvh);
-        po.w_lo = wg_of_unit(ups);
-        po.n_splits = wg_of_unit(ups + (pe - ps) - 1u) - po.w_lo + 1u;
-        po.slot_first = 2u * po.w_lo + (unit_start(po.w_lo) + PC >= ups ? 0u : 1u);
-        po.my_slot = (ps <= g0) ? 2u * w : 2u * w + 1u;
+        // end of the pair before
+        po.w_lo = wg_of_unit(ps + PC * (Hkv * req_nzb(cu.r) + cu.kvh));
         po.orow = out_row(cu);
         return po;
     };
@@ -866,64 +907,28 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
             orow[(k / HPK) * D + dim0 + (k % HPK)] = o_un[k] * inv;
         }
     };
-    auto store_partial = [&](uint32_t my_slot, const float (&o_un)[OPL], const float (&m_all)[HPW],
-                             const float (&l_all)[HPW]) {
-        float* po = a.part_o + ((size_t)my_slot * G + hg * HPW) * D;
-        float* ml = a.part_ml + ((size_t)my_slot * G + hg * HPW) * 2;
+    // A wave's partial: PW tagged words per lane, word k of lane i at [k][i].  Words 0 .. OPL-1
+    // are the lane's un-normalised outputs, word OPL carries m of head i in lane i < HPW and l of
+    // head i - HPW in lanes HPW .. 2*HPW-1 (m in log2 units).
+    constexpr int PW = OPL + 1;
+    const uint32_t tag_sum = a.tag + tag_add;
+    const uint32_t tag = tag_sum ? tag_sum : 0x9E3779B9u;   // (zero is what untouched memory holds)
+    auto partial_of = [&](uint32_t wg) { return a.part + ((size_t)(wg * NW + (uint32_t)hg) * PW) * 64 + lane; };
+    auto publish = [&](const float (&o_un)[OPL], const float (&m_all)[HPW], const float (&l_all)[HPW]) {
+        uint64_t* dst = partial_of(w);
+        const uint64_t hi = (uint64_t)tag << 32;
 #pragma unroll
-        for (int k = 0; k < OPL; ++k) st_dev(po + k * 64 + lane, o_un[k]);
-        if (lane < HPW) {
-            float mh = m_all[0], lh = l_all[0];
+        for (int k = 0; k < OPL; ++k) st_tagged(dst + k * 64, hi | __float_as_uint(o_un[k]));
+        float x = 0.f;
 #pragma unroll
-            for (int hh = 1; hh < HPW; ++hh) {
-                mh = (lane == hh) ? m_all[hh] : mh;
-                lh = (lane == hh) ? l_all[hh] : lh;
-            }
-            st_dev(ml + lane * 2, mh);
-            st_dev(ml + lane * 2 + 1, lh);
-        }
+        for (int h = 0; h < HPW; ++h) x = lane == h ? m_all[h] : lane == HPW + h ? l_all[h] : x;
+        st_tagged(dst + OPL * 64, hi | __float_as_uint(x));
     };
-    // Merge of a pair's partials by the wave that arrived last, in the order of their slots (so
-    // the result does not depend on who arrived last).  64 partials at a time: lane s holds the
-    // (m, l) of partial s for every head; the partial outputs are loaded eight at a time.  The
-    // loads of the first round -- the (m, l) pairs and the first eight outputs, nearly always all
-    // there is -- are a step of their own (merge_fetch), so that a wave that merges two pairs
-    // has both pairs' loads in flight together: one memory round trip in all.
+    // Sums up the pair this workgroup ends: the partials of workgroups po.w_lo .. w-1, eight at a
+    // time, then this workgroup's own part.
     constexpr int MUNR = 8;
-    struct MergeLoads {
-        float pvv[MUNR][OPL];
-        float ms[HPW], ls[HPW];
-    };
-    auto merge_slot = [&](const PairOut& po, uint32_t i) { return i == 0 ? po.slot_first : 2u * (po.w_lo + i); };
-    auto merge_fetch_outputs = [&](const PairOut& po, uint32_t first, uint32_t cnt, float (&pvv)[MUNR][OPL]) {
-#pragma unroll
-        for (int u = 0; u < MUNR; ++u) {
-            const float* src = a.part_o + ((size_t)merge_slot(po, first + u) * G + hg * HPW) * D;
-#pragma unroll
-            for (int k = 0; k < OPL; ++k) {
-                pvv[u][k] = 0.f;
-                if ((uint32_t)u < cnt) pvv[u][k] = ld_dev(src + k * 64 + lane);
-            }
-        }
-    };
-    auto merge_fetch_ml = [&](const PairOut& po, uint32_t s0, uint32_t cnt, float (&ms)[HPW], float (&ls)[HPW]) {
-        const float* ml = a.part_ml + ((size_t)merge_slot(po, s0 + (uint32_t)lane) * G + hg * HPW) * 2;
-#pragma unroll
-        for (int h = 0; h < HPW; ++h) {
-            ms[h] = kNegBig;
-            ls[h] = 0.f;
-            if ((uint32_t)lane < cnt) {
-                ms[h] = ld_dev(ml + h * 2);
-                ls[h] = ld_dev(ml + h * 2 + 1);
-            }
-        }
-    };
-    auto merge_fetch = [&](const PairOut& po, MergeLoads& ld) {
-        const uint32_t cnt = min(64u, po.n_splits);
-        merge_fetch_outputs(po, 0, cnt, ld.pvv);
-        merge_fetch_ml(po, 0, cnt, ld.ms, ld.ls);
-    };
-    auto merge = [&](const PairOut& po, MergeLoads& ld) {
+    auto merge_pair = [&](const PairOut& po, const float (&own_o)[OPL], const float (&own_m)[HPW],
+                          const float (&own_l)[HPW]) {
         float acc_o[OPL], m_run[HPW], l_run[HPW];
 #pragma unroll
         for (int k = 0; k < OPL; ++k) acc_o[k] = 0.f;
@@ -932,35 +937,63 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
             m_run[h] = kNegBig;
             l_run[h] = 0.f;
         }
-        for (uint32_t s0 = 0; s0 < po.n_splits; s0 += 64) {
-            const uint32_t cnt = min(64u, po.n_splits - s0);
-            if (s0) {
-                merge_fetch_outputs(po, s0, cnt, ld.pvv);
-                merge_fetch_ml(po, s0, cnt, ld.ms, ld.ls);
-            }
-            float wgt[HPW];
+        auto fold = [&](const float (&o)[OPL], const float (&m)[HPW], const float (&l)[HPW]) {
 #pragma unroll
             for (int h = 0; h < HPW; ++h) {
-                const float m_new = max_nn(m_run[h], wave_max(ld.ms[h]));
+                const float m_new = max_nn(m_run[h], m[h]);
                 const float keep = fast_exp2(m_run[h] - m_new);
-                wgt[h] = fast_exp2(ld.ms[h] - m_new);  // lanes >= cnt: exp2(-1e30 - m) = 0
-                l_run[h] = l_run[h] * keep + __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(
-                                                 int, wave_sum(wgt[h] * ld.ls[h]))));
+                const float wgt = fast_exp2(m[h] - m_new);
+                l_run[h] = l_run[h] * keep + l[h] * wgt;
                 m_run[h] = m_new;
 #pragma unroll
-                for (int kk = 0; kk < HPK; ++kk) acc_o[h * HPK + kk] *= keep;
+                for (int kk = 0; kk < HPK; ++kk) acc_o[h * HPK + kk] = acc_o[h * HPK + kk] * keep + o[h * HPK + kk] * wgt;
             }
-            for (uint32_t u0 = 0; u0 < cnt; u0 += MUNR) {
-                if (u0) merge_fetch_outputs(po, s0 + u0, cnt - u0, ld.pvv);
+        };
+        const uint32_t n_others = w - po.w_lo;
+        uint32_t spins = 0;
+        for (uint32_t s0 = 0; s0 < n_others; s0 += MUNR) {
+            const uint32_t cnt = min((uint32_t)MUNR, n_others - s0);
+            uint64_t wd[MUNR][PW];
+            for (;;) {
+                bool ok = true;
 #pragma unroll
                 for (int u = 0; u < MUNR; ++u) {
-                    if (u0 + u < cnt) {
+                    if ((uint32_t)u < cnt) {
+                        const uint64_t* src = partial_of(po.w_lo + s0 + (uint32_t)u);
 #pragma unroll
-                        for (int k = 0; k < OPL; ++k) acc_o[k] += __shfl(wgt[k / HPK], (int)(u0 + u)) * ld.pvv[u][k];
+                        for (int k = 0; k < PW; ++k) wd[u][k] = ld_tagged(src + k * 64);
                     }
+                }
+#pragma unroll
+                for (int u = 0; u < MUNR; ++u) {
+                    if ((uint32_t)u < cnt) {
+#pragma unroll
+                        for (int k = 0; k < PW; ++k) ok = ok && (uint32_t)(wd[u][k] >> 32) == tag;
+                    }
+                }
+                if (__all(ok)) break;
+                if (++spins >= a.spin_limit) {   // a sharer never wrote: give up, tell the host
+                    if (lane == 0) __hip_atomic_store(a.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    break;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < MUNR; ++u) {
+                if ((uint32_t)u < cnt) {
+                    float o[OPL], m[HPW], l[HPW];
+#pragma unroll
+                    for (int k = 0; k < OPL; ++k) o[k] = __uint_as_float((uint32_t)wd[u][k]);
+                    const int x = (int)(uint32_t)wd[u][OPL];
+#pragma unroll
+                    for (int h = 0; h < HPW; ++h) {
+                        m[h] = __int_as_float(__builtin_amdgcn_readlane(x, h));
+                        l[h] = __int_as_float(__builtin_amdgcn_readlane(x, HPW + h));
+                    }
+                    fold(o, m, l);
                 }
             }
         }
+        fold(own_o, own_m, own_l);
         store_direct(po.orow, acc_o, l_run);
     };
 
@@ -1016,9 +1049,9 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         sd_wait_vmcnt<0>();  // the rows have left this wave before any wave of the workgroup loads them
         sd_barrier();
     }
-    load_q(cc);
     uint32_t issued = 1;
     issue_tile(ci, 0);
+    load_q(cc);   // (behind the tile's request: q is a memory round trip of its own)
     if (!kv_first) {
         g1 = tiles_before(u1);
         n = g1 - g0;
@@ -1030,7 +1063,8 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     uint32_t seg_first = g0;  // first tile consumed for the pair under cc
     bool drain = false;       // stores are in flight: they do not complete in order with loads
     uint32_t slot = 0;        // stage of tile k
-    bool kept = false;        // the range's first pair waits in registers for the end of the range
+    bool kept = false;        // the range's first pair, which this workgroup sums up, waits in registers
+                              // for the end of the range
     PairOut kept_po{};
     float kept_o[OPL], kept_m[HPW], kept_l[HPW];
     for (uint32_t k = 0; k < n; ++k) {
@@ -1067,65 +1101,42 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
             float o_un[OPL], m_all[HPW], l_all[HPW];
             reduce_rows(o_un, m_all, l_all);
             const uint32_t ps = req_start(cc.r) * Hkv + cc.kvh * cc.tiles;  // pair's first tile
-            const uint32_t pe = ps + cc.tiles;
-            const bool whole = seg_first == ps && g0 + k + 1u == pe;
-            bool cur = false;  // this pair is a partial to publish now (only at the end of the range)
+            const bool starts_here = seg_first == ps;                 // no workgroup before this one has tiles of the pair
+            const bool ends_here = g0 + k + 1u == ps + cc.tiles;      // ... none behind it
+            bool cur = false;  // this pair is summed up by this workgroup, now
             PairOut cur_po{};
-            if (whole) {
+            if (starts_here && ends_here) {
                 store_direct(out_row(cc), o_un, l_all);
                 drain = true;
-            } else if (!range_done) {
-                kept = true;
-                kept_po = pair_out(cc, ps, pe);
+            } else if (ends_here) {
+                if (range_done) {
+                    cur = true;
+                    cur_po = pair_out(cc, ps);
+                } else {
+                    kept = true;
+                    kept_po = pair_out(cc, ps);
 #pragma unroll
-                for (int i = 0; i < OPL; ++i) kept_o[i] = o_un[i];
+                    for (int i = 0; i < OPL; ++i) kept_o[i] = o_un[i];
 #pragma unroll
-                for (int h = 0; h < HPW; ++h) {
-                    kept_m[h] = m_all[h];
-                    kept_l[h] = l_all[h];
+                    for (int h = 0; h < HPW; ++h) {
+                        kept_m[h] = m_all[h];
+                        kept_l[h] = l_all[h];
+                    }
                 }
             } else {
-                cur = true;
-                cur_po = pair_out(cc, ps, pe);
-            }
-#ifdef MLC_NO_TAIL
-            if (false) {
-#else
-            if (range_done && (kept || cur)) {
+#ifndef MLC_NO_TAIL
+                // (the pair goes on in the next workgroup: the range ends here)
+                if (!(a.test_flags & 1u)) publish(o_un, m_all, l_all);
 #endif
-                if (kept) store_partial(kept_po.my_slot, kept_o, kept_m, kept_l);
-                if (cur) store_partial(cur_po.my_slot, o_un, m_all, l_all);
-                // The partials must have reached memory before an arrival counter is bumped: the
-                // write-through stores are complete once this wave's memory counter is zero.
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-                sd_wait_vmcnt<0>();
                 MLC_PROBE(26);
-                uint32_t t_kept = 0, t_cur = 0;
-                uint32_t* c_kept = &a.counters[(size_t)kept_po.w_lo * NW + hg];
-                uint32_t* c_cur = &a.counters[(size_t)cur_po.w_lo * NW + hg];
-                if (lane == 0) {  // both tickets travel together
-                    if (kept) t_kept = __hip_atomic_fetch_add(c_kept, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    if (cur) t_cur = __hip_atomic_fetch_add(c_cur, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
-                t_kept = __shfl(t_kept, 0);
-                t_cur = __shfl(t_cur, 0);
-                MLC_PROBE(27);
-                const bool last_kept = kept && t_kept == kept_po.n_splits - 1u;
-                const bool last_cur = cur && t_cur == cur_po.n_splits - 1u;
-                if (last_kept || last_cur) {
-                    MLC_PROBE(28);
-                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-                    if (lane == 0) {  // ready for the next launch
-                        if (last_kept) __hip_atomic_store(c_kept, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        if (last_cur) __hip_atomic_store(c_cur, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    }
-                    MergeLoads ld_kept, ld_cur;
-                    if (last_kept) merge_fetch(kept_po, ld_kept);
-                    if (last_cur) merge_fetch(cur_po, ld_cur);
-                    if (last_kept) merge(kept_po, ld_kept);
-                    if (last_cur) merge(cur_po, ld_cur);
-                }
             }
+#ifndef MLC_NO_TAIL
+            if (range_done && (kept || cur)) {
+                MLC_PROBE(28);
+                if (kept) merge_pair(kept_po, kept_o, kept_m, kept_l);
+                else merge_pair(cur_po, o_un, m_all, l_all);
+            }
+#endif
             reset_state();
             seg_first = g0 + k + 1u;
         }
@@ -1138,9 +1149,9 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     MLC_PROBE(5);
 #ifdef MLC_STREAM_PROBE
     if (threadIdx.x == 0) {
-        reinterpret_cast<uint64_t*>(a.part_ml + 65536)[blockIdx.x * 32 + 6] = n;
+        (a.part + kStreamProbeWord)[blockIdx.x * 32 + 6] = n;
         const uint64_t hw = __builtin_amdgcn_s_getreg((31 << 11) | 4), xcc = __builtin_amdgcn_s_getreg((31 << 11) | 20);
-        reinterpret_cast<uint64_t*>(a.part_ml + 65536)[blockIdx.x * 32 + 7] = hw | (xcc << 32);
+        (a.part + kStreamProbeWord)[blockIdx.x * 32 + 7] = hw | (xcc << 32);
     }
 #endif
 }
