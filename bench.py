@@ -511,6 +511,8 @@ def probe_timeline(n_wg: int) -> dict:
     if not lib.mlc_hip_debug_probe(buf.ctypes.data, n_wg):
         raise RuntimeError("mlc_hip_debug_probe failed")
     t = buf.astype(np.int64)
+    if os.environ.get("MLC_PROBE_RAW"):   # the raw stamps, for offline analysis
+        np.save(os.environ["MLC_PROBE_RAW"], t)
     us = lambda x: (x - t[:, 0].min()) / 100.0
 
     def st(x):
@@ -523,6 +525,9 @@ def probe_timeline(n_wg: int) -> dict:
     out = {"workgroups": n_wg, "tiles_per_workgroup": sorted(set(int(v) for v in t[:, 6]))}
     for i, nm in enumerate(names):
         out[nm] = st(us(t[:, i]))
+    xcc = (t[:, 7] >> 32) & 0xF
+    out["workgroups_not_on_xcd_blockidx_mod_8"] = int((xcc != (np.arange(n_wg) % 8)).sum())
+    out["xcd_of_first_16_workgroups"] = [int(v) for v in xcc[:16]]
     lastc, ex = us(t[:, 4]), us(t[:, 5])
     pub = (t[:, 26] >= t[:, 0]) & (t[:, 26] <= t[:, 5])
     mer = (t[:, 28] >= t[:, 0]) & (t[:, 28] <= t[:, 5])

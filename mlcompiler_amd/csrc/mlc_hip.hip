@@ -963,7 +963,7 @@ uint32_t stream_pair_cost(int nw, size_t G, size_t D) {
     if (g.opt_pair_cost >= 0) return (uint32_t)g.opt_pair_cost;
     (void)G;
     (void)D;
-    return nw == 4 ? 3u : 0u;
+    return nw == 4 ? 2u : 0u;
 }
 
 // Arithmetic mode of the tile-balanced kernel: 0 fp32 softmax weights, 1 fp16 weights on the vector

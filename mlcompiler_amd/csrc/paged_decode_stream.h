@@ -23,6 +23,8 @@
 //     table.  Nothing is planned on the host.
 #pragma once
 
+#include <cstddef>
+
 #include "paged_decode_kernels.h"
 
 namespace mlc_hip {
@@ -422,16 +424,41 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     }
     ci = cc;
 
-    const uint32_t* pt_flat = a.pt_flat ? a.pt_flat : a.emb + 3u * (SMALL ? kStreamSmallStride : a.meta_stride);
+    // (the embedded table is addressed as global memory, which the argument segment is: through
+    // the constant address space the choice between the two would make every page-id load a flat
+    // one, and the compiler waits for all loads in flight around those)
+    typedef const __attribute__((address_space(1))) uint32_t* global_u32_ptr;
+    const uint32_t* emb_table = (const uint32_t*)(global_u32_ptr)(uintptr_t)__builtin_amdgcn_kernarg_segment_ptr() +
+                                offsetof(StreamArgs, emb) / 4 + 3u * (SMALL ? kStreamSmallStride : a.meta_stride);
+    const uint32_t* pt_flat = a.pt_flat ? a.pt_flat : emb_table;
     // Page ids of the issue side's request, 64 tiles at a time: lane i holds the page of tile
     // pv_win + i.  Refetched when the issue side enters another request or another window.
     uint32_t pv = 0, pv_win = 0, pv_req = 0xFFFFFFFFu;
+    // ... and of the first 64 tiles of the request behind it, requested when the issue side enters a
+    // request, so that the step into the next request finds them in a register
+    uint32_t pv_nx = 0, pv_nx_req = 0xFFFFFFFFu;
+    auto prefetch_next_pages = [&](uint32_t r) {
+        pv_nx_req = 0xFFFFFFFFu;
+        do {
+            ++r;
+        } while (r < B && req_tiles(r) == 0);
+        if (r >= B) return;
+        pv_nx_req = r;
+        const uint32_t idx = min((uint32_t)lane, req_tiles(r) - 1u) / tpp;   // (lanes past the end repeat the last id)
+        pv_nx = pt_flat[req_off(r) + idx];
+    };
     auto fetch_pages = [&](const Cursor& cu) {
-        pv_req = cu.r;
-        pv_win = cu.t & ~63u;
-        const uint32_t t = pv_win + (uint32_t)lane;
-        pv = 0;
-        if (t < cu.tiles) pv = pt_flat[cu.off + t / tpp];
+        if (pv_nx_req == cu.r && cu.t < 64u) {
+            pv = pv_nx;
+            pv_req = cu.r;
+            pv_win = 0;
+        } else {
+            pv_req = cu.r;
+            pv_win = cu.t & ~63u;
+            const uint32_t t = pv_win + (uint32_t)lane;
+            pv = 0;
+            if (t < cu.tiles) pv = pt_flat[cu.off + t / tpp];
+        }
         // The ids are waited for here, inside whatever branch fetches them: left pending, the
         // compiler would wait at every later join of the control flow, and as it does not know
         // of the tile loads, that wait would be for all of them.
@@ -467,27 +494,43 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     }
     // q of this wave's heads, dims c*8 .. c*8+7, scaled
     float qv[HPW][8];
+    // matrix-pipe mode: q is fetched as it lies in memory (q_raw) and split into the two fp16
+    // operands when the consume side reaches the pair.  With two stages the issue side is exactly
+    // one tile ahead, so it fetches the next pair's q together with that pair's first tile and the
+    // pair's end finds it in registers.
+    constexpr bool Q_AHEAD = MF && NBUF == 2;
+    float4 q_raw[MF ? 2 * KST : 1];
+    auto fetch_q = [&](const Cursor& cu) {
+        // (columns past the group: the loads are clamped onto the last head and the factor below is
+        // zero; a select on the loaded value would put the load under a branch, and the wait for it
+        // there would be for every load in flight)
+        const int hcol = n16 < G ? n16 : G - 1;
+        const float* qb = a.q + ((size_t)cu.r * a.num_heads + cu.kvh * G + hcol) * D + 8 * g4;
+#pragma unroll
+        for (int ks = 0; ks < (MF ? KST : 0); ++ks) {
+            q_raw[2 * ks] = *reinterpret_cast<const float4*>(qb + 32 * ks);
+            q_raw[2 * ks + 1] = *reinterpret_cast<const float4*>(qb + 32 * ks + 4);
+        }
+    };
+    auto split_q = [&]() {
+        const float q_factor = n16 < G ? a.scale_log2e : 0.f;
+#pragma unroll
+        for (int ks = 0; ks < (MF ? KST : 0); ++ks) {
+            const float4 x0 = q_raw[2 * ks], x1 = q_raw[2 * ks + 1];
+            const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float v = x[i] * q_factor;
+                const _Float16 hi = (_Float16)v;
+                qh[ks][i] = hi;
+                ql[ks][i] = (_Float16)(v - (float)hi);
+            }
+        }
+    };
     auto load_q = [&](const Cursor& cu) {
         if constexpr (MF) {
-            const int hcol = n16 < G ? n16 : G - 1;
-            const float q_factor = n16 < G ? a.scale_log2e : 0.f;
-            const float* qb = a.q + ((size_t)cu.r * a.num_heads + cu.kvh * G + hcol) * D + 8 * g4;
-#pragma unroll
-            for (int ks = 0; ks < KST; ++ks) {
-                const float4 x0 = *reinterpret_cast<const float4*>(qb + 32 * ks);
-                const float4 x1 = *reinterpret_cast<const float4*>(qb + 32 * ks + 4);
-                const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    // (columns past the group: the loads are clamped onto the last head and the
-                    // factor is zero; a select on the loaded value would put the load under a
-                    // branch, and the wait for it there would be for every load in flight)
-                    const float v = x[i] * q_factor;
-                    const _Float16 hi = (_Float16)v;
-                    qh[ks][i] = hi;
-                    ql[ks][i] = (_Float16)(v - (float)hi);
-                }
-            }
+            fetch_q(cu);
+            split_q();
             return;
         }
         const float* qbase = a.q + ((size_t)cu.r * a.num_heads + cu.kvh * G + hg * HPW) * D + c * 8;
@@ -1052,6 +1095,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     uint32_t issued = 1;
     issue_tile(ci, 0);
     load_q(cc);   // (behind the tile's request: q is a memory round trip of its own)
+    if (pv_win == 0) prefetch_next_pages(ci.r);
     if (!kv_first) {
         g1 = tiles_before(u1);
         n = g1 - g0;
@@ -1086,9 +1130,17 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         // (all stages requested at once would make every workgroup wait for the whole burst)
         while (issued < n && issued < k + (uint32_t)NBUF) {
             advance(ci);
-            if (!pages_ready(ci)) fetch_pages(ci);
+            // (order: whatever the compiler waits for -- the page ids it takes over, registers of q it
+            // believes busy -- comes while nothing is in flight; the next request's ids are asked for
+            // last and are not waited for before the step into that request)
+            const bool new_pages = !pages_ready(ci);
+            if (new_pages) fetch_pages(ci);
+            if constexpr (Q_AHEAD) {
+                if (ci.t == 0) fetch_q(ci);   // first tile of the next pair: its q with it
+            }
             issue_tile(ci, issued % (uint32_t)NBUF);
             ++issued;
+            if (new_pages && pv_win == 0) prefetch_next_pages(ci.r);
         }
 #ifndef MLC_NO_COMPUTE
         consume_tile(slot, cc.t, cc.lim);
@@ -1142,7 +1194,10 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         }
         if (!range_done) {
             advance(cc);
-            if (pair_done) load_q(cc);
+            if (pair_done) {
+                if constexpr (Q_AHEAD) split_q();
+                else load_q(cc);
+            }
         }
         slot = slot + 1u == (uint32_t)NBUF ? 0u : slot + 1u;
     }
