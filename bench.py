@@ -671,13 +671,14 @@ def run_decode(args, name: str, steps: int, warmup: int, cpu_budget: float, full
             r[key] = {"wall": round((time.perf_counter() - tb) / n_b * 1e6, 3), "events": round(ev / n_b * 1e3, 3),
                       "steps": n_b}
 
-        # ---- fp32 softmax weights for P.V (decode_pv_fp16 = 0: meets the reference's 1e-5 gate)
+        # ---- softmax weights rounded to fp16 for P.V (option decode_pv_fp16 = 1; the default keeps them
+        # fp32-grade and meets the reference's 1e-5 stress gate)
         n_x = max(steps, 500)
-        assert exe.setOption("decode_pv_fp16", 0)
-        native_loop(2 * n_layers)
-        ev32, _ = native_loop(n_x)
         assert exe.setOption("decode_pv_fp16", 1)
-        r["pv_fp32_us"] = ev32 / n_x * 1e3
+        native_loop(2 * n_layers)
+        ev16, _ = native_loop(n_x)
+        assert exe.setOption("decode_pv_fp16", 0)
+        r["pv_fp16_us"] = ev16 / n_x * 1e3
 
         # ---- products on the vector pipe (decode_mfma = 0), fp16 softmax weights as in the default
         if any(kv.startswith("decode_mfma=") for kv in args.opt):
@@ -883,9 +884,6 @@ def main() -> int:
     ap.add_argument("--copy-mib", type=int, default=32, help="size of the calibration copy")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU baseline work")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--target-items", type=int, default=0)
-    ap.add_argument("--decode-kernel", type=int, default=0,
-                    help="0 = automatic (tile-balanced kernel), 1 = planned split-K items")
     ap.add_argument("--wgs-per-cu", type=int, default=0, help="tile-balanced kernel: workgroups per CU (0 = automatic)")
     ap.add_argument("--stages", type=int, default=0, help="tile-balanced kernel: LDS stages (0 = automatic)")
     ap.add_argument("--read-sweep", action="store_true",
@@ -925,10 +923,6 @@ def main() -> int:
     from mlcompiler_amd import HipExecutor
     exe = HipExecutor.Instance()
     exe.requireAvailable()
-    if args.target_items:
-        exe.setOption("decode_target_items", args.target_items)
-    if args.decode_kernel:
-        assert exe.setOption("decode_kernel", args.decode_kernel)
     if args.wgs_per_cu:
         assert exe.setOption("decode_wgs_per_cu", args.wgs_per_cu)
     if args.stages:
@@ -956,10 +950,10 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32 accumulate and output (fp16 K/V storage; products on f16 MFMA: fp32 q enters as the sum of "
-                 "two fp16 numbers, softmax weights are rounded to fp16 for P.V; option decode_pv_fp16 = 0: fp32 "
-                 "weights on the vector pipe, us_per_layer_pv_fp32 is its time; option decode_mfma = 0: every product on the "
-                 "vector pipe with fp32 q, us_per_layer_vector_pipe is its time)",
+        "dtype": "f32 (fp16 K/V storage, fp32 q, accumulate and output; fp32-grade products, no operand rounded: on "
+                 "the f16 MFMA q and the softmax weights enter as sums of two fp16 numbers; option decode_pv_fp16 = 1 "
+                 "rounds the weights to fp16, us_per_layer_pv_fp16 is its time; option decode_mfma = 0: every product "
+                 "on the vector pipe, us_per_layer_vector_pipe is its time)",
         "data": "synthetic",
         "config": {
             "workload": workload_text(c, r["n_layers"]),
@@ -971,7 +965,7 @@ def main() -> int:
             "kernels_per_step": r["launches"],
             "kernel": r["kernel"],
             "work_items": r["items"],
-            "us_per_layer_pv_fp32": round(r["pv_fp32_us"], 3),
+            "us_per_layer_pv_fp16": round(r["pv_fp16_us"], 3),
             "us_per_layer_vector_pipe": None if r["vector_pipe_us"] != r["vector_pipe_us"] else round(r["vector_pipe_us"], 3),
             "us_per_layer_tables_change": r["tables_change_us"],
             "us_per_layer_page_table_changes": r["page_table_changes_us"],

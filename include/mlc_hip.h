@@ -325,12 +325,12 @@ int   mlc_hip_timer_start(void);
 float mlc_hip_timer_stop(void);
 
 /* Number of kernels the last mlc_hip_paged_attn_decode call launched and the
- * number of split-K work items it planned (for benchmarks and tests). */
+ * number of workgroups that took part of the work (for benchmarks and tests). */
 int mlc_hip_last_decode_launches(void);
 int mlc_hip_last_decode_work_items(void);
 /* Name of the kernel variant the last decode call launched, with its template arguments, e.g.
- * "stream<64,2,4,pv16,regs,2>" (head_dim, query heads per wave, waves per group, softmax-weight
- * type, where the per-request figures live, LDS stages), "planned<...>" or "generic". */
+ * "stream<64,2,4,mfma-p32,regs,2>" (head_dim, query heads per wave, waves per group, arithmetic mode,
+ * where the per-request figures live, LDS stages) or "generic". */
 const char* mlc_hip_last_decode_kernel(void);
 /* Number of KV writes so far that went out fused with a neighbour: a batched K scatter with its
  * V twin, or split + RoPE + cast with the scatters of its fp16 rows (for tests). */
@@ -348,20 +348,18 @@ long mlc_hip_row_program_launches(void);
 long mlc_hip_decode_table_uploads(void);
 
 /* Tunables (0 selects the automatic choice where noted):
- *   "decode_kernel"         0 = automatic: the tile-balanced kernel (fixed grid, work derived from
- *                           the tables inside the kernel) wherever it applies; 1 = the planned
- *                           kernel (host-built split-K work items); 2 = same as 0
  *   "decode_wgs_per_cu"     workgroups per CU of the tile-balanced kernel's grid (0 = automatic)
  *   "decode_stages"         2, 3 or 4 K/V tiles staged in LDS per workgroup of the tile-balanced kernel
  *                           (0 = automatic: 2; batches above 64 requests take 3 at most)
  *   "decode_grid_wgs"       exact grid size of the tile-balanced kernel (0 = from the above; for tests)
- *   "decode_target_items"   planned kernel: split-K work items aimed for per launch (0 = automatic)
  *   "decode_heads_per_wave" 1, 2, 4 or 8: the most query heads one wavefront handles;
  *                           the GQA group is spread over group/that many waves (0 = automatic)
- *   "decode_tile_rows"      1 or 2: wave rows of a workgroup that share an item's tiles
- *   "decode_buffers"        1 or 2 LDS staging buffers per workgroup (0 = automatic)
- *   "decode_pv_fp16"        1 = softmax weights rounded to fp16 for the P.V product
- *                           (fp32 accumulate), 0 = fp32 weights (vector pipe only)
+ *   "decode_spin_limit"     rounds a workgroup that sums up a split pair polls for the other workgroups'
+ *                           partials before it gives up and the pass fails (default 200000, about 0.1 s)
+ *   "decode_test_flags"     bit 0: partials are not published (tests of the give-up path)
+ *   "decode_pv_fp16"        0 (default) = fp32-grade softmax weights: fp32 on the vector pipe, the sum
+ *                           of two fp16 numbers on the matrix pipe; 1 = weights rounded to fp16
+ *                           for the P.V product (fp32 accumulate)
  *   "decode_force_generic"  1 = always use the shape-agnostic kernel
  *   "q4_force_generic"      1 = Q4_0 matmul always on the scalar kernel
  *   "q4_ksplit"             K slices of the Q4_0 MFMA matmul (0 = automatic)
@@ -380,10 +378,10 @@ long mlc_hip_decode_table_uploads(void);
  *   "decode_pair_cost"      0..64: the tile-balanced decode kernel gives every workgroup the same
  *                           number of units, a KV tile counting one and the end of a (request,
  *                           KV head) pair this many; 0 = the same number of tiles; -1 (default) =
- *                           4 for GQA ratios of 4 and more (workgroups of four waves), 0 below
+ *                           2 for GQA ratios of 4 and more (workgroups of four waves), 0 below
  *   "decode_mfma"           1 (default) = the tile-balanced decode kernel does a tile's arithmetic
  *                           on the matrix pipe where the shape allows it (4 to 16 query heads per
- *                           KV head in 4 waves, fp16 softmax weights); 0 = on the vector pipe
+ *                           KV head in 4 waves); 0 = on the vector pipe
  *   "prefill_stages"        2, 4, 6 or 8 K/V tiles staged in LDS by the prefill kernel (0 = automatic:
  *                           6); with 8 the kernel with 64 rows per wave lets its waves meet only
  *                           after every second tile

@@ -30,10 +30,6 @@
 
 namespace mlc_hip {
 // Defined in paged_decode_inst.hip, one object per (head_dim, heads-per-wave).
-#define MLC_DECL(d, h) bool launch_decode_fast_##d##_##h(int, int, int, bool, const DecodeArgs&, hipStream_t);
-MLC_DECL(64, 1) MLC_DECL(64, 2) MLC_DECL(64, 4) MLC_DECL(64, 8)
-MLC_DECL(128, 1) MLC_DECL(128, 2) MLC_DECL(128, 4) MLC_DECL(128, 8)
-#undef MLC_DECL
 #define MLC_DECL(d, h) bool launch_decode_stream_##d##_##h(int, int, int, const StreamArgs&, unsigned, size_t, hipStream_t);
 MLC_DECL(64, 1) MLC_DECL(64, 2) MLC_DECL(64, 4) MLC_DECL(64, 8)
 MLC_DECL(128, 1) MLC_DECL(128, 2) MLC_DECL(128, 4) MLC_DECL(128, 8)
@@ -118,18 +114,17 @@ struct StreamTables {
     std::vector<uint32_t> last_meta;  // seq_lens | q_positions | offsets of the last decode call (host copy)
 };
 
+// What the shape-agnostic decode kernel reads: the flat page table, the page-table offsets and the
+// visible length of every request, in one device blob that is re-uploaded only when the tables
+// change (the walker passes the same tables for every layer of a step).
 struct DecodePlan {
     bool valid = false;
     // key
     std::vector<uint32_t> pt_flat, pt_off, seq_lens, q_pos;
-    size_t B = 0, H = 0, Hkv = 0, D = 0, P = 0;
+    size_t B = 0;
     int causal = 0;
-    long target_items = 0, force_generic = 0, hpw_max = 0, tile_rows = 0, buffers = 0;
     // result
-    bool fast = false;
-    int hpw = 0, nw = 0, ns = 0, nbuf = 2;
-    uint32_t n_items = 0, n_part = 0;
-    size_t off_items = 0, off_ptoff = 0, off_limits = 0;  // byte offsets in blob
+    size_t off_ptoff = 0, off_limits = 0;  // byte offsets in blob
     int slot = -1;
 };
 
@@ -221,19 +216,12 @@ struct Ctx {
     MetaSlot plan_slots[4];
     int plan_next = 0;
     DecodePlan plan;
-    float* part_o = nullptr;
-    float* part_ml = nullptr;
-    uint32_t* counters = nullptr;
-    size_t part_o_cap = 0, part_ml_cap = 0, counters_cap = 0;  // in elements
-    long opt_target_items = 0;                                 // 0 = automatic
     long opt_force_generic = 0;
     long opt_hpw_max = 0;                                      // query heads per wave, at most (0 = automatic)
-    long opt_buffers = 0;                                      // LDS staging buffers per workgroup (1, 2; 0 = automatic)
-    long opt_tile_rows = 1;                                    // wave rows that share an item's tiles
     long opt_prefill_stages = 0;                               // LDS pipeline depth of the prefill kernel (0 = automatic)
     long opt_decode_mfma = 1;                                  // tile-balanced decode kernel: tile arithmetic on the matrix pipe
     long opt_prefill_rows64 = 1;                               // prefill: 64 chunk rows per wave where the GQA ratio allows it
-    long opt_pv_fp16 = 1;                                      // softmax weights rounded to fp16 for P.V
+    long opt_pv_fp16 = 0;                                      // 1 = softmax weights rounded to fp16 for P.V (default: fp32-grade)
     int last_launches = 0;
     int last_items = 0;
     char last_kernel[96] = "";   // kernel variant of the last decode launch (for benchmarks)
@@ -248,7 +236,6 @@ struct Ctx {
     long opt_spin_limit = 200000;           // rounds a merge polls before it gives up (about 0.1 s)
     long opt_test_flags = 0;                // bit 0: workgroups do not publish their partials (tests of the give-up path)
     StreamTables tables;
-    long opt_decode_kernel = 0;     // 0 = automatic (tile-balanced where it applies), 1 = planned items, 2 = tile-balanced
     long opt_wgs_per_cu = 0;        // tile-balanced kernel: workgroups per CU (0 = automatic)
     long opt_stream_stages = 0;     // tile-balanced kernel: LDS stages per workgroup (0 = automatic)
     long opt_grid_wgs = 0;          // tile-balanced kernel: exact grid size (0 = from workgroups per CU)
@@ -582,16 +569,11 @@ const void* resident_ids(const uint32_t* page_ids, const uint32_t* slots, size_t
     return dev;
 }
 
-// ---------------------------------------------------------------- decode plan
+// ---------------------------------------------------------------- tables of the shape-agnostic decode kernel
 
 bool plan_matches(const DecodePlan& p, const uint32_t* flat, size_t n_flat, const uint32_t* off,
-                  const uint32_t* seq, const uint32_t* qpos, size_t B, size_t H, size_t Hkv,
-                  size_t D, size_t P, int causal) {
-    if (!p.valid || p.B != B || p.H != H || p.Hkv != Hkv || p.D != D || p.P != P ||
-        p.causal != causal || p.target_items != g.opt_target_items ||
-        p.force_generic != g.opt_force_generic || p.hpw_max != g.opt_hpw_max ||
-        p.tile_rows != g.opt_tile_rows || p.buffers != g.opt_buffers)
-        return false;
+                  const uint32_t* seq, const uint32_t* qpos, size_t B, int causal) {
+    if (!p.valid || p.B != B || p.causal != causal) return false;
     if (p.pt_flat.size() != n_flat) return false;
     if (n_flat && std::memcmp(p.pt_flat.data(), flat, n_flat * 4) != 0) return false;
     if (std::memcmp(p.pt_off.data(), off, (B + 1) * 4) != 0) return false;
@@ -600,205 +582,38 @@ bool plan_matches(const DecodePlan& p, const uint32_t* flat, size_t n_flat, cons
     return true;
 }
 
-// Builds (or reuses) the device-side metadata for one decode call: the page
-// tables and either the split-K work list of the fast kernel or the per-request
-// limits of the generic one.  The walker calls with byte-identical tables for
-// every layer of a step (compiler/runtime/batched_walker.cpp:316-325), so the
-// result is cached and re-uploaded only when the tables change.
+// Brings the tables of the shape-agnostic kernel onto the device (cached, see DecodePlan).
 int build_plan(const uint32_t* flat, size_t n_flat, const uint32_t* off, const uint32_t* seq,
-               const uint32_t* qpos, size_t B, size_t H, size_t Hkv, size_t D, size_t P,
-               int causal, bool pointers_aligned) {
+               const uint32_t* qpos, size_t B, int causal) {
     DecodePlan& p = g.plan;
-    if (plan_matches(p, flat, n_flat, off, seq, qpos, B, H, Hkv, D, P, causal)) return 1;
+    if (plan_matches(p, flat, n_flat, off, seq, qpos, B, causal)) return 1;
     p.valid = false;
     p.pt_flat.assign(flat, flat + n_flat);
     p.pt_off.assign(off, off + B + 1);
     p.seq_lens.assign(seq, seq + B);
     p.q_pos.assign(qpos, qpos + B);
-    p.B = B; p.H = H; p.Hkv = Hkv; p.D = D; p.P = P; p.causal = causal;
-    p.target_items = g.opt_target_items;
-    p.force_generic = g.opt_force_generic;
-    p.hpw_max = g.opt_hpw_max;
-    p.tile_rows = g.opt_tile_rows;
-    p.buffers = g.opt_buffers;
-
+    p.B = B;
+    p.causal = causal;
     std::vector<uint32_t> limits(B);
     for (size_t r = 0; r < B; ++r) {
         uint64_t lim = seq[r];
         if (causal && (uint64_t)qpos[r] + 1 < lim) lim = (uint64_t)qpos[r] + 1;  // :2286
         limits[r] = (uint32_t)lim;
     }
-
-    const size_t tile = (D == 64) ? 64 : 32;
-    p.fast = !g.opt_force_generic && pointers_aligned && (D == 64 || D == 128) && (P % tile) == 0;
-    const size_t G = H / Hkv;
-    if (p.fast) {
-        // query heads per wave (power of two dividing G), waves per workgroup = G / that
-        // Chosen by sweep on MI355X: a query-head group runs fastest spread over four waves
-        // (G / 4 heads each; one head per wave for groups of 4 and fewer): more waves hide the
-        // latency of the tile loads and of short items better than sharing the per-tile softmax
-        // and packing work over more heads saves.
-        const long hpw_cap = g.opt_hpw_max > 0 ? g.opt_hpw_max : std::max<long>(1, (long)G / 4);
-        int hpw = 8;
-        while (hpw > 1 && (hpw > hpw_cap || (G % (size_t)hpw) != 0)) hpw >>= 1;
-        size_t nw = G / (size_t)hpw;
-        if (nw > 4 || nw == 3) {  // too many / odd wave counts: use the widest wave
-            hpw = 8;
-            while (hpw > 1 && (G % (size_t)hpw) != 0) hpw >>= 1;
-            nw = G / (size_t)hpw;
-        }
-        if (nw > 4 || nw == 3) p.fast = false;
-        p.hpw = hpw;
-        p.nw = (int)nw;
-        // tile rows per workgroup, within the workgroup's LDS budget
-        int ns = (int)g.opt_tile_rows;
-        const int nbuf = g.opt_buffers > 0 ? (int)g.opt_buffers : 2;  // refined below
-        while (ns > 1 && decode_lds_bytes((int)D, hpw, (int)nw, ns, nbuf) > kMaxStaticLds) ns >>= 1;
-        if (decode_lds_bytes((int)D, hpw, (int)nw, ns, nbuf) > kMaxStaticLds) p.fast = false;
-        p.ns = ns;
-        p.nbuf = nbuf;
-    }
-    const size_t flat_bytes = align_up(n_flat * 4, 16);
-
-    std::vector<DecodeWorkItem> items;
-    p.n_part = 0;
-    if (p.fast) {
-        size_t total_tiles = 0;
-        for (size_t r = 0; r < B; ++r) total_tiles += (limits[r] + tile - 1) / tile;
-        total_tiles *= Hkv;
-        // About 8 tiles per item, but no fewer than 4 and no more than 16 items per CU
-        // (measured optimum on MI355X for 35 MB .. 1.2 GB of KV per call).
-        size_t target = std::min<size_t>(std::max<size_t>(total_tiles / 8, (size_t)g.n_cu * 4),
-                                         (size_t)g.n_cu * 16);
-        if (g.opt_target_items > 0) target = (size_t)g.opt_target_items;
-        size_t chunk = std::max<size_t>(1, (total_tiles + target - 1) / target);
-        // Short items cannot use a second buffer; one buffer lets twice the workgroups
-        // share a CU and hide each other's memory latency.
-        if (g.opt_buffers == 0) p.nbuf = (chunk >= 4 * (size_t)p.ns) ? 2 : 1;
-        for (size_t r = 0; r < B; ++r) {  // the merge handles at most kMaxSplits partials
-            const size_t tiles_r = (limits[r] + tile - 1) / tile;
-            chunk = std::max(chunk, (tiles_r + kMaxSplits - 1) / kMaxSplits);
-        }
-        for (size_t r = 0; r < B; ++r) {
-            const size_t tiles_r = (limits[r] + tile - 1) / tile;
-            const size_t ns = std::max<size_t>(1, (tiles_r + chunk - 1) / chunk);
-            const size_t per = (tiles_r + ns - 1) / ns;
-            size_t ns_eff = tiles_r == 0 ? 1 : (tiles_r + per - 1) / per;
-            if (ns_eff > kMaxSplits) return fail("decode: too many splits");
-            // Many splits are merged in two levels: groups of about sqrt(splits), a multiple of
-            // the eight partials one round of the merge loads, then the groups' results, which
-            // take n_groups more partial slots (and their arrival counters) behind the splits.
-            size_t group_size = 0, n_groups = 0;
-            if (ns_eff > kFlatMergeSplits) {
-                group_size = 8;
-                while (group_size * group_size < ns_eff) group_size += 8;
-                n_groups = (ns_eff + group_size - 1) / group_size;
-            }
-            for (size_t kvh = 0; kvh < Hkv; ++kvh) {
-                uint32_t first_part = kNoPartial;
-                if (ns_eff > 1) {
-                    first_part = p.n_part;
-                    p.n_part += (uint32_t)(ns_eff + n_groups);
-                }
-                for (size_t s = 0; s < ns_eff; ++s) {
-                    DecodeWorkItem it;
-                    it.req = (uint32_t)r;
-                    it.kv_head = (uint32_t)kvh;
-                    it.pt_base = off[r];
-                    it.tok_begin = (uint32_t)std::min<size_t>(s * per * tile, limits[r]);
-                    it.tok_end = (uint32_t)std::min<size_t>((s + 1) * per * tile, limits[r]);
-                    it.part_first = first_part;
-                    it.split = (uint32_t)s | ((uint32_t)ns_eff << 16);
-                    for (size_t i = 0; i < 4; ++i) {
-                        const size_t tok = (size_t)it.tok_begin + i * tile;
-                        it.first_pages[i] = tok < it.tok_end ? flat[off[r] + tok / P] : 0u;
-                    }
-                    it.group_size = (uint32_t)group_size;
-                    items.push_back(it);
-                }
-            }
-        }
-        // Longest first, so the tail of the launch is made of short items.
-        std::stable_sort(items.begin(), items.end(), [](const DecodeWorkItem& x,
-                                                        const DecodeWorkItem& y) {
-            return (x.tok_end - x.tok_begin) > (y.tok_end - y.tok_begin);
-        });
-        p.n_items = (uint32_t)items.size();
-        p.off_items = flat_bytes;
-        const size_t total = p.off_items + items.size() * sizeof(DecodeWorkItem);
-        MetaSlot& s = g.plan_slots[g.plan_next];
-        if (!slot_reserve(s, std::max<size_t>(total, 16))) return 0;
-        char* h = static_cast<char*>(s.host);
-        if (n_flat) std::memcpy(h, flat, n_flat * 4);
-        if (!items.empty()) std::memcpy(h + p.off_items, items.data(), items.size() * sizeof(DecodeWorkItem));
-        if (!slot_upload(s, std::max<size_t>(total, 16))) return 0;
-    } else {
-        p.hpw = 0;
-        p.nw = 0;
-        p.n_items = (uint32_t)(B * H);
-        p.off_ptoff = flat_bytes;
-        p.off_limits = p.off_ptoff + align_up(B * 4, 16);
-        const size_t total = p.off_limits + align_up(B * 4, 16);
-        MetaSlot& s = g.plan_slots[g.plan_next];
-        if (!slot_reserve(s, total)) return 0;
-        char* h = static_cast<char*>(s.host);
-        if (n_flat) std::memcpy(h, flat, n_flat * 4);
-        std::memcpy(h + p.off_ptoff, off, B * 4);
-        std::memcpy(h + p.off_limits, limits.data(), B * 4);
-        if (!slot_upload(s, total)) return 0;
-    }
+    p.off_ptoff = align_up(n_flat * 4, 16);
+    p.off_limits = p.off_ptoff + align_up(B * 4, 16);
+    const size_t total = p.off_limits + align_up(B * 4, 16);
+    MetaSlot& s = g.plan_slots[g.plan_next];
+    if (!slot_reserve(s, total)) return 0;
+    char* h = static_cast<char*>(s.host);
+    if (n_flat) std::memcpy(h, flat, n_flat * 4);
+    std::memcpy(h + p.off_ptoff, off, B * 4);
+    std::memcpy(h + p.off_limits, limits.data(), B * 4);
+    if (!slot_upload(s, total)) return 0;
     p.slot = g.plan_next;
     g.plan_next = (g.plan_next + 1) % 4;
     p.valid = true;
     return 1;
-}
-
-int ensure_partials(size_t n_part, size_t G, size_t D, size_t nw) {
-    const size_t need_o = n_part * G * D;
-    const size_t need_ml = n_part * G * 2;
-    const size_t need_c = n_part * nw;
-    if (need_o > g.part_o_cap || need_ml > g.part_ml_cap || need_c > g.counters_cap) {
-        NOT_WHILE_CAPTURING("growing the split-K partial buffers");
-        HIP_OK(hipStreamSynchronize(g.stream));
-        if (g.part_o) HIP_OK(hipFree(g.part_o));
-        if (g.part_ml) HIP_OK(hipFree(g.part_ml));
-        if (g.counters) HIP_OK(hipFree(g.counters));
-        g.part_o = nullptr;
-        g.part_ml = nullptr;
-        g.counters = nullptr;
-        g.part_o_cap = g.part_ml_cap = g.counters_cap = 0;
-        const size_t cap_o = std::max<size_t>(need_o * 2, 1 << 20);
-        const size_t cap_ml = std::max<size_t>(need_ml * 2, 1 << 14);
-        const size_t cap_c = std::max<size_t>(need_c * 2, 1 << 14);
-        HIP_OK(hipMalloc(reinterpret_cast<void**>(&g.part_o), cap_o * sizeof(float)));
-        HIP_OK(hipMalloc(reinterpret_cast<void**>(&g.part_ml), cap_ml * sizeof(float)));
-        HIP_OK(hipMalloc(reinterpret_cast<void**>(&g.counters), cap_c * sizeof(uint32_t)));
-        // Arrival counters start at zero; the last arriver of every group puts its counter
-        // back to zero, so they stay zero between launches.
-        HIP_OK(hipMemsetAsync(g.counters, 0, cap_c * sizeof(uint32_t), g.stream));
-        g.part_o_cap = cap_o;
-        g.part_ml_cap = cap_ml;
-        g.counters_cap = cap_c;
-    }
-    return 1;
-}
-
-bool launch_fast(size_t D, int hpw, int nw, int ns, int nbuf, const DecodeArgs& a) {
-    const bool pv16 = g.opt_pv_fp16 != 0;
-    if (D == 64) {
-        switch (hpw) {
-            case 8: return launch_decode_fast_64_8(nw, ns, nbuf, pv16, a, g.stream);
-            case 4: return launch_decode_fast_64_4(nw, ns, nbuf, pv16, a, g.stream);
-            case 2: return launch_decode_fast_64_2(nw, ns, nbuf, pv16, a, g.stream);
-            default: return launch_decode_fast_64_1(nw, ns, nbuf, pv16, a, g.stream);
-        }
-    }
-    switch (hpw) {
-        case 8: return launch_decode_fast_128_8(nw, ns, nbuf, pv16, a, g.stream);
-        case 4: return launch_decode_fast_128_4(nw, ns, nbuf, pv16, a, g.stream);
-        case 2: return launch_decode_fast_128_2(nw, ns, nbuf, pv16, a, g.stream);
-        default: return launch_decode_fast_128_1(nw, ns, nbuf, pv16, a, g.stream);
-    }
 }
 
 // Largest page id a request actually dereferences, for bounds checks against
@@ -947,7 +762,7 @@ int stream_stages(size_t batch) {
 // Grid of the tile-balanced kernel: as many workgroups as stay resident (LDS decides), within
 // what the scratch array holds.
 unsigned stream_grid(size_t G, size_t D, int nbuf, size_t dyn_lds) {
-    const bool matrix_pipe = g.opt_pv_fp16 && g.opt_decode_mfma && G >= 4 && G <= 16;
+    const bool matrix_pipe = g.opt_decode_mfma && G >= 4 && G <= 16;
     const size_t lds = stream_static_lds_bytes(nbuf, G, D, matrix_pipe) + dyn_lds;
     size_t per_cu = std::max<size_t>(1, std::min<size_t>(160 * 1024 / lds, 2));
     if (g.opt_wgs_per_cu > 0) per_cu = (size_t)g.opt_wgs_per_cu;
@@ -969,12 +784,13 @@ uint32_t stream_pair_cost(int nw, size_t G, size_t D) {
 // Arithmetic mode of the tile-balanced kernel: 0 fp32 softmax weights, 1 fp16 weights on the vector
 // pipe, 2 matrix pipe (4 waves per workgroup, at most 16 heads per KV head).
 int stream_pv_mode(int hpw, int nw) {
-    if (!g.opt_pv_fp16) return 0;
-    return (g.opt_decode_mfma && nw == 4 && hpw * nw <= 16) ? 2 : 1;
+    const bool matrix_pipe = g.opt_decode_mfma && nw == 4 && hpw * nw <= 16;
+    if (!g.opt_pv_fp16) return matrix_pipe ? 3 : 0;
+    return matrix_pipe ? 2 : 1;
 }
 const char* stream_pv_name(int hpw, int nw) {
     const int m = stream_pv_mode(hpw, nw);
-    return m == 2 ? "mfma" : m == 1 ? "pv16" : "pv32";
+    return m == 3 ? "mfma-p32" : m == 2 ? "mfma" : m == 1 ? "pv16" : "pv32";
 }
 
 bool launch_stream_variant(size_t D, int hpw, int nw, int nbuf, const StreamArgs& a, unsigned n_wg, size_t dyn_lds,
@@ -1203,7 +1019,7 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
 
     // ---- which kernel: the tile-balanced one wherever it applies
     int s_hpw = 0, s_nw = 0;
-    bool use_stream = g.opt_decode_kernel != 1 && !g.opt_force_generic && aligned &&
+    bool use_stream = !g.opt_force_generic && aligned &&
                       (page_size_tokens % tile) == 0 && batch <= kStreamMaxBatch &&
                       stream_variant(G, head_dim, &s_hpw, &s_nw);
     uint64_t total_tiles = 0;
@@ -1220,18 +1036,18 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
     const DecodePlan* plan = nullptr;
     if (!use_stream) {
         if (!build_plan(page_tables_flat, n_flat, page_table_offsets, seq_lens, q_positions, batch,
-                        num_heads, kv_heads, head_dim, page_size_tokens, apply_causal ? 1 : 0, aligned))
+                        apply_causal ? 1 : 0))
             return 0;
         plan = &g.plan;
     }
 
     if (carries_kv) {
-        // Only the tiled kernels write rows, and only rows that are every request's newest
+        // Only the tile-balanced kernel writes rows, and only rows that are every request's newest
         // visible position: then exactly one workgroup reads each of them, after writing it.
         // That also needs every page to belong to one request (and to appear once in its
         // table): with a repeated page id another workgroup could read the row while it is
         // being written, and the separate launches are the ones that give the order of the calls.
-        carries_kv = (use_stream || plan->fast) && g.tables.shared_pages == 0;
+        carries_kv = use_stream && g.tables.shared_pages == 0;
         for (size_t r = 0; carries_kv && r < batch; ++r) {
             const uint64_t S = seq_lens[r];
             const bool visible = !apply_causal || (uint64_t)q_positions[r] + 1 >= S;
@@ -1322,43 +1138,8 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
     MetaSlot& slot = g.plan_slots[p.slot];
     const char* dev = static_cast<const char*>(slot.dev);
     const float scale_log2e = (1.0f / std::sqrt(static_cast<float>(head_dim))) * 1.44269504088896340736f;
-    g.last_items = (int)p.n_items;
-    if (p.fast) {
-        if (p.n_part && !ensure_partials(p.n_part, G, head_dim, (size_t)p.nw))
-            return 0;
-        DecodeArgs a;
-        a.q = static_cast<const float*>(q);
-        a.k_pages = static_cast<const uint4*>(k_pages);
-        a.v_pages = static_cast<const uint4*>(v_pages);
-        a.o = static_cast<float*>(o);
-        a.pt_flat = reinterpret_cast<const uint32_t*>(dev);
-        a.items = reinterpret_cast<const DecodeWorkItem*>(dev + p.off_items);
-        a.part_o = g.part_o;
-        a.part_ml = g.part_ml;
-        a.counters = g.counters;
-        a.num_heads = (uint32_t)num_heads;
-        a.kv_heads = (uint32_t)kv_heads;
-        a.page_size = (uint32_t)page_size_tokens;
-        a.n_items = p.n_items;
-        a.scale_log2e = scale_log2e;
-        a.new_k = a.new_v = nullptr;
-        a.new_ids = a.new_slots = nullptr;
-        if (carries_kv) {
-            a.new_k = static_cast<const uint4*>(g.kv.src[0]);
-            a.new_v = static_cast<const uint4*>(g.kv.src[1]);
-            a.new_ids = g.kv.d_ids;
-            a.new_slots = g.kv.d_slots;
-        }
-        if (!launch_fast(head_dim, p.hpw, p.nw, p.ns, p.nbuf, a)) return fail("decode: kernel variant not built");
-        std::snprintf(g.last_kernel, sizeof g.last_kernel, "planned<%zu,%d,%d,%d,%d,%s>", head_dim, p.hpw, p.nw, p.ns,
-                      p.nbuf, g.opt_pv_fp16 ? "pv16" : "pv32");
-        if (carries_kv) {
-            g.kv.active = false;
-            ++g.kv_fused;
-            ++g.kv_in_decode;
-        }
-        ++g.last_launches;
-    } else {
+    g.last_items = (int)(batch * num_heads);
+    {
         GenericArgs a;
         a.q = static_cast<const float*>(q);
         a.k_pages = static_cast<const _Float16*>(k_pages);
@@ -2479,13 +2260,7 @@ int mlc_hip_set_option(const char* name, long value) {
     if (!name) return 0;
     if (g.inited && g.available && !settle()) return 0;
     if (!std::strcmp(name, "fuse_row_ops")) { g.opt_fuse_rows = value ? 1 : 0; return 1; }
-    if (!std::strcmp(name, "decode_target_items")) { g.opt_target_items = value; return 1; }
     if (!std::strcmp(name, "decode_force_generic")) { g.opt_force_generic = value; return 1; }
-    if (!std::strcmp(name, "decode_kernel")) {
-        if (value < 0 || value > 2) return 0;
-        g.opt_decode_kernel = value;
-        return 1;
-    }
     if (!std::strcmp(name, "decode_stages")) {
         if (value != 0 && (value < 2 || value > 4)) return 0;
         g.opt_stream_stages = value;
@@ -2537,16 +2312,6 @@ int mlc_hip_set_option(const char* name, long value) {
     if (!std::strcmp(name, "prefill_rows64")) {
         if (value != 0 && value != 1) return 0;
         g.opt_prefill_rows64 = value;
-        return 1;
-    }
-    if (!std::strcmp(name, "decode_buffers")) {
-        if (value != 0 && value != 1 && value != 2) return 0;
-        g.opt_buffers = value;
-        return 1;
-    }
-    if (!std::strcmp(name, "decode_tile_rows")) {
-        if (value != 1 && value != 2) return 0;
-        g.opt_tile_rows = value;
         return 1;
     }
     if (!std::strcmp(name, "decode_heads_per_wave")) {

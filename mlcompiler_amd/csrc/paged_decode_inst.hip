@@ -1,4 +1,4 @@
-// One translation unit per (head_dim, heads-per-wave) pair of the fast decode kernel:
+// One translation unit per (head_dim, heads-per-wave) pair of the tile-balanced decode kernel:
 // compiled with -DMLC_D=<64|128> -DMLC_HPW=<1|2|4|8>, so the variants build in parallel.
 #include "paged_decode_kernels.h"
 #include "paged_decode_stream.h"
@@ -7,47 +7,10 @@
 #error "compile with -DMLC_D=64|128 -DMLC_HPW=1|2|4|8"
 #endif
 
-#define MLC_CAT_(a, b, c) launch_decode_fast_##a##_##b
-#define MLC_CAT(a, b) MLC_CAT_(a, b, 0)
 #define MLC_SCAT_(a, b, c) launch_decode_stream_##a##_##b
 #define MLC_SCAT(a, b) MLC_SCAT_(a, b, 0)
 
 namespace mlc_hip {
-
-namespace {
-template <int NW, int NS, int NBUF>
-bool launch_buf(bool pv16, const DecodeArgs& a, hipStream_t stream) {
-    if constexpr (decode_lds_bytes(MLC_D, MLC_HPW, NW, NS, NBUF) <= kMaxStaticLds) {
-        const dim3 grid(a.n_items), block(64 * NW * NS);
-        if (pv16)
-            hipLaunchKernelGGL((paged_decode_fast_kernel<MLC_D, MLC_HPW, NW, NS, NBUF, true>), grid, block, 0, stream, a);
-        else
-            hipLaunchKernelGGL((paged_decode_fast_kernel<MLC_D, MLC_HPW, NW, NS, NBUF, false>), grid, block, 0, stream, a);
-        return true;
-    } else {
-        return false;
-    }
-}
-
-template <int NW, int NS>
-bool launch_one(int nbuf, bool pv16, const DecodeArgs& a, hipStream_t stream) {
-    return nbuf == 1 ? launch_buf<NW, NS, 1>(pv16, a, stream) : launch_buf<NW, NS, 2>(pv16, a, stream);
-}
-}  // namespace
-
-// nw = waves over the GQA group, ns = tile rows; returns false for an unbuilt combination.
-bool MLC_CAT(MLC_D, MLC_HPW)(int nw, int ns, int nbuf, bool pv16, const DecodeArgs& a, hipStream_t stream) {
-    const int key = nw * 10 + ns;
-    switch (key) {
-        case 11: return launch_one<1, 1>(nbuf, pv16, a, stream);
-        case 12: return launch_one<1, 2>(nbuf, pv16, a, stream);
-        case 21: return launch_one<2, 1>(nbuf, pv16, a, stream);
-        case 22: return launch_one<2, 2>(nbuf, pv16, a, stream);
-        case 41: return launch_one<4, 1>(nbuf, pv16, a, stream);
-        case 42: return launch_one<4, 2>(nbuf, pv16, a, stream);
-        default: return false;
-    }
-}
 
 namespace {
 template <int NW, bool SMALL, int NBUF>
@@ -58,8 +21,12 @@ void launch_stream_pv(int pvm, const StreamArgs& a, unsigned n_wg, size_t dyn_ld
             hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, 2, SMALL, NBUF>), grid, block, dyn_lds, stream, a);
             return;
         }
+        if (pvm == 3) {
+            hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, 3, SMALL, NBUF>), grid, block, dyn_lds, stream, a);
+            return;
+        }
     }
-    if (pvm)
+    if (pvm == 1 || pvm == 2)
         hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, 1, SMALL, NBUF>), grid, block, dyn_lds, stream, a);
     else
         hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, 0, SMALL, NBUF>), grid, block, dyn_lds, stream, a);
@@ -81,9 +48,9 @@ bool launch_stream(int nbuf, int pvm, const StreamArgs& a, unsigned n_wg, size_t
 }  // namespace
 
 // Tile-balanced kernel: nw = waves over the GQA group, nbuf = LDS stages (large batches: at most 3),
-// pvm = arithmetic mode (0 fp32 weights, 1 fp16 weights on the vector pipe, 2 matrix pipe where
-// built: 4 waves and at most 16 heads per KV head, else mode 1), n_wg = grid size; false for an
-// unbuilt combination.
+// pvm = arithmetic mode (0 fp32 weights, 1 fp16 weights on the vector pipe, 2 / 3 matrix pipe with
+// fp16 / split weights where built: 4 waves and at most 16 heads per KV head; the caller falls
+// back to 1 / 0 elsewhere), n_wg = grid size; false for an unbuilt combination.
 bool MLC_SCAT(MLC_D, MLC_HPW)(int nw, int nbuf, int pvm, const StreamArgs& a, unsigned n_wg, size_t dyn_lds, hipStream_t stream) {
     switch (nw) {
         case 1: return launch_stream<1>(nbuf, pvm, a, n_wg, dyn_lds, stream);

@@ -157,16 +157,18 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t x) {
 // nothing goes through LDS.  Otherwise they are kept in (dynamic) LDS.
 // NBUF: tiles staged in LDS per workgroup; tile k + NBUF - 1 is requested while tile k is consumed.
 // PVM: how a tile's arithmetic is done.  0: on the vector pipe with fp32 softmax weights; 1: on the
-// vector pipe, weights rounded to fp16 for P.V (v_dot2); 2: on the matrix pipe (4 waves, at most
+// vector pipe, weights rounded to fp16 for P.V (v_dot2); 2 and 3: on the matrix pipe (4 waves, at most
 // 16 query heads per KV head): every wave takes a quarter of the tile's tokens for all heads of
 // the group, S^T = K.q^T with v_mfma_f32_16x16x32_f16 (q as the sum of two fp16 numbers, so that
 // the products are as exact as with fp32 q), O^T += V^T.P^T with v_mfma_f32_16x16x16_f16 (fp16
-// weights as in mode 1), V^T through the transposing LDS read; the waves' results are combined
+// weights as in mode 1; mode 3: the weight as the sum of two fp16 numbers, two MFMAs per V block,
+// fp32-grade like mode 0), V^T through the transposing LDS read; the waves' results are combined
 // through LDS where a pair of (request, KV head) ends.
 template <int D, int HPW, int NW, int PVM, bool SMALL, int NBUF>
 __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const StreamArgs a) {
     constexpr bool PV16 = PVM == 1;
-    constexpr bool MF = PVM == 2;
+    constexpr bool MF = PVM == 2 || PVM == 3;
+    constexpr bool MF_SPLIT_P = PVM == 3;
     static_assert(!MF || (NW == 4 && HPW * NW <= 16), "matrix-pipe mode: 4 waves, at most 16 heads per KV head");
     static_assert(NBUF >= 2 && NBUF <= 4, "2 to 4 stages");
     static_assert(D == 64 || D == 128, "head_dim 64 and 128");
@@ -662,6 +664,24 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
                 for (int b = 0; b < DB; ++b) mf_o[b] *= alpha;
             }
             sd_half4 pb;
+            if constexpr (MF_SPLIT_P) {
+                // the weight enters as the sum of two fp16 numbers, like q: the products with the
+                // fp16 V are exact, only the order of the fp32 additions differs from the vector pipe
+                sd_half4 pl;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float pf = fast_exp2(s4[i] - mf_m);
+                    mf_l += pf;
+                    pb[i] = (_Float16)pf;
+                    pl[i] = (_Float16)(pf - (float)pb[i]);
+                }
+#pragma unroll
+                for (int b = 0; b < DB; ++b) {
+                    mf_o[b] = __builtin_amdgcn_mfma_f32_16x16x16f16(va[b], pb, mf_o[b], 0, 0, 0);
+                    mf_o[b] = __builtin_amdgcn_mfma_f32_16x16x16f16(va[b], pl, mf_o[b], 0, 0, 0);
+                }
+                return;
+            }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 pb[i] = (_Float16)fast_exp2(s4[i] - mf_m);

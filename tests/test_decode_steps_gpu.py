@@ -20,15 +20,14 @@ from test_kv_write_in_decode_gpu import _expect, _newest, _rows, _step
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("kernel", ["balanced", "planned"])
-def test_config3_full_size_step_every_request(exe, kernel):
+def test_config3_full_size_step_every_request(exe):
     case = baseline_config(3)
     assert case.batch == 64
     ids, slots = _newest(case)                 # (page_table.back(), (S - 1) % 64), some at slot 0 of a fresh page
     new_k, new_v = _rows(case, 303)
     want_k, want_v, want_o = _expect(case, ids, slots, new_k, new_v)
-    print(f"[case] config 3 full step, kernel {kernel}, KV bytes {case.kv_bytes}", flush=True)
-    out, kp, vp, carried = _step(exe, case, ids, slots, new_k, new_v, 1, kernel=kernel)
+    print(f"[case] config 3 full step, KV bytes {case.kv_bytes}", flush=True)
+    out, kp, vp, carried = _step(exe, case, ids, slots, new_k, new_v, 1)
     assert carried == 1
     assert np.array_equal(kp, want_k) and np.array_equal(vp, want_v)
     rep = assert_parity(out, want_o, case.head_dim, "config 3 step")

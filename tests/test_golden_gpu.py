@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("c", list(load_attention_cases()), ids=lambda c: f"H{c['H']}kv{c['Hkv']}D{c['D']}S{c['S']}")
-@pytest.mark.parametrize("kernel", ["balanced", "planned", "generic"])
+@pytest.mark.parametrize("kernel", ["balanced", "generic"])
 def test_decode_matches_golden_reference_outputs(exe, c, kernel):
     generic = 1 if kernel == "generic" else 0
     P, S = c["P"], c["S"]
@@ -24,14 +24,12 @@ def test_decode_matches_golden_reference_outputs(exe, c, kernel):
                       q=c["q"].reshape(1, c["H"], c["D"]), k_pages=c["k"], v_pages=c["v"])
     print(f"[golden] H={c['H']}/{c['Hkv']} D={c['D']} S={S} P={P} kernel={kernel}", flush=True)
     assert exe.setOption("decode_force_generic", generic)
-    assert exe.setOption("decode_kernel", 1 if kernel == "planned" else 0)
     dev = DeviceCase(exe, case)
     try:
         got = dev.run(sync=True)
     finally:
         dev.free()
         exe.setOption("decode_force_generic", 0)
-        exe.setOption("decode_kernel", 0)
     assert_parity(got.reshape(1, c["H"], c["D"]), c["o"].reshape(1, c["H"], c["D"]), c["D"], "golden")
 
 

@@ -22,13 +22,12 @@ def _newest(case):
     return ids, (last % case.page_size).astype(np.uint32)
 
 
-def _step(exe, case, ids, slots, new_k, new_v, fuse, *, only_k=False, target=0, kernel="balanced"):
+def _step(exe, case, ids, slots, new_k, new_v, fuse, *, only_k=False, target=0):
     """scatter K, scatter V, attention in one open pass -> (output, K pool, V pool, launches that carried the write)"""
     dev = DeviceCase(exe, case)
     nk, nv = (exe.allocateScratchBuffer(a.nbytes) for a in (new_k, new_v))
     assert exe.uploadToBuffer(nk, new_k) and exe.uploadToBuffer(nv, new_v)
-    split = "decode_target_items" if kernel == "planned" else "decode_grid_wgs"
-    assert exe.setOption("decode_kernel", 1 if kernel == "planned" else 0)
+    split = "decode_grid_wgs"
     assert exe.setOption("fuse_row_ops", fuse) and exe.setOption(split, target)
     before = exe.kvWritesInDecodeLaunches()
     c = case
@@ -48,7 +47,6 @@ def _step(exe, case, ids, slots, new_k, new_v, fuse, *, only_k=False, target=0, 
     finally:
         exe.setOption("fuse_row_ops", 1)
         exe.setOption(split, 0)
-        exe.setOption("decode_kernel", 0)
         dev.free()
         exe.releaseScratchBuffer(nk)
         exe.releaseScratchBuffer(nv)
@@ -70,11 +68,9 @@ def _rows(case, seed):
 
 
 @pytest.mark.parametrize("shape", [(8, 2, 64), (32, 4, 64), (32, 8, 128), (8, 8, 64)], ids=["g4d64", "g8d64", "g4d128", "mha"])
-@pytest.mark.parametrize("kernel,target", [("planned", 0), ("planned", 100000), ("planned", 1),
-                                           ("balanced", 0), ("balanced", 2048), ("balanced", 1), ("balanced", 5)],
-                         ids=["planned_auto", "planned_many_splits", "planned_no_splits", "balanced_auto",
-                              "balanced_many_splits", "balanced_one_workgroup", "balanced_five_workgroups"])
-def test_attention_launch_carries_the_kv_write(exe, shape, kernel, target):
+@pytest.mark.parametrize("target", [0, 2048, 1, 5],
+                         ids=["balanced_auto", "balanced_many_splits", "balanced_one_workgroup", "balanced_five_workgroups"])
+def test_attention_launch_carries_the_kv_write(exe, shape, target):
     h, hkv, d = shape
     lens = [1, 64, 65, 130, 700, 2000, 63, 128]     # newest position at page starts, page ends, mid-page
     case = make_case("kvstep", len(lens), h, hkv, d, 64, lens, seed=3 + d, capacity_pages=64)
@@ -82,8 +78,8 @@ def test_attention_launch_carries_the_kv_write(exe, shape, kernel, target):
     new_k, new_v = _rows(case, 17)
     want_k, want_v, want_o = _expect(case, ids, slots, new_k, new_v)
     print(f"[case] kv write in decode {shape} target={target}", flush=True)
-    plain = _step(exe, case, ids, slots, new_k, new_v, 0, target=target, kernel=kernel)
-    fused = _step(exe, case, ids, slots, new_k, new_v, 1, target=target, kernel=kernel)
+    plain = _step(exe, case, ids, slots, new_k, new_v, 0, target=target)
+    fused = _step(exe, case, ids, slots, new_k, new_v, 1, target=target)
     assert plain[3] == 0 and fused[3] == 1
     for got in (plain, fused):
         assert np.array_equal(got[1], want_k) and np.array_equal(got[2], want_v)
@@ -91,8 +87,7 @@ def test_attention_launch_carries_the_kv_write(exe, shape, kernel, target):
     assert np.array_equal(plain[0], fused[0])      # the same kernel did the arithmetic
 
 
-@pytest.mark.parametrize("kernel", ["balanced", "planned"])
-def test_other_rows_are_written_by_their_own_launch(exe, kernel):
+def test_other_rows_are_written_by_their_own_launch(exe):
     case = make_case("kvstep_other", 4, 8, 2, 64, 64, [70, 200, 64, 129], seed=9, capacity_pages=16)
     ids, slots = _newest(case)
     new_k, new_v = _rows(case, 5)
@@ -103,40 +98,38 @@ def test_other_rows_are_written_by_their_own_launch(exe, kernel):
     case_b = replace(case, q_positions=np.array([69, 199, 10, 128], np.uint32))
     for c, sl, only_k in ((case, slots_a, False), (case_b, slots, False), (case, slots, True)):
         want_k, want_v, want_o = _expect(c, ids, sl, new_k, new_v, only_k)
-        out, kp, vp, carried = _step(exe, c, ids, sl, new_k, new_v, 1, only_k=only_k, kernel=kernel)
+        out, kp, vp, carried = _step(exe, c, ids, sl, new_k, new_v, 1, only_k=only_k)
         assert carried == 0
         assert np.array_equal(kp, want_k) and np.array_equal(vp, want_v)
         assert_parity(out, want_o, 64, "kv step, separate launches")
 
 
-@pytest.mark.parametrize("opts", [{"decode_tile_rows": 2}, {"decode_buffers": 1}, {"decode_buffers": 2},
-                                  {"decode_heads_per_wave": 8}, {"decode_heads_per_wave": 1},
-                                  {"decode_tile_rows": 2, "decode_target_items": 100000}],
+@pytest.mark.parametrize("opts", [{"decode_heads_per_wave": 8}, {"decode_heads_per_wave": 1}, {"decode_stages": 3},
+                                  {"decode_mfma": 0}, {"decode_grid_wgs": 2048}],
                          ids=lambda o: ",".join(f"{k[7:]}={v}" for k, v in o.items()))
-def test_kv_write_and_two_level_merge_in_every_kernel_variant(exe, opts):
-    """The same step through the other shapes of the tiled kernel (two tile rows per workgroup,
-    one or two staging buffers, other head groupings), with one request long enough to be cut
-    into more splits than one wave merges at once."""
+def test_kv_write_and_many_splits_in_every_kernel_variant(exe, opts):
+    """The same step through the other shapes of the tile-balanced kernel (other head groupings,
+    three LDS stages, vector pipe, one tile per workgroup), with one request long enough to be
+    cut into more partials than one round of the merge loads."""
     lens = [1, 65, 700, 9000, 128]
     case = make_case("kvstep_variants", len(lens), 32, 8, 64, 64, lens, seed=21, capacity_pages=160)
     ids, slots = _newest(case)
     new_k, new_v = _rows(case, 23)
     want_k, want_v, want_o = _expect(case, ids, slots, new_k, new_v)
     for name, value in opts.items():
-        assert exe.setOption(name, value)
+        if name != "decode_grid_wgs":
+            assert exe.setOption(name, value)
     try:
-        out, kp, vp, carried = _step(exe, case, ids, slots, new_k, new_v, 1, target=opts.get("decode_target_items", 0),
-                                     kernel="planned")
+        out, kp, vp, carried = _step(exe, case, ids, slots, new_k, new_v, 1, target=opts.get("decode_grid_wgs", 0))
     finally:
         for name in opts:
-            exe.setOption(name, 1 if name == "decode_tile_rows" else 0)
+            exe.setOption(name, 1 if name == "decode_mfma" else 0)
     assert carried == 1
     assert np.array_equal(kp, want_k) and np.array_equal(vp, want_v)
     assert_parity(out, want_o, 64, f"kv step {opts}")
 
 
-@pytest.mark.parametrize("kernel", ["balanced", "planned"])
-def test_a_shared_page_keeps_the_launches_apart(exe, kernel):
+def test_a_shared_page_keeps_the_launches_apart(exe):
     """Two requests whose tables name the same physical page (the reference's allocator never
     does that, the interface does not forbid it): the row written for one request is then also
     read for the other, so the attention launch must not take the write; the three launches run
@@ -149,11 +142,11 @@ def test_a_shared_page_keeps_the_launches_apart(exe, kernel):
     ids, slots = _newest(case)
     new_k, new_v = _rows(case, 41)
     want_k, want_v, want_o = _expect(case, ids, slots, new_k, new_v)
-    out, kp, vp, carried = _step(exe, case, ids, slots, new_k, new_v, 1, kernel=kernel)
+    out, kp, vp, carried = _step(exe, case, ids, slots, new_k, new_v, 1)
     assert carried == 0
     assert np.array_equal(kp, want_k) and np.array_equal(vp, want_v)
     assert_parity(out, want_o, 64, "kv step, shared page")
     # the same tables without the repeated page: the attention launch takes the write again
     case2 = make_case("kvstep_unshared", 3, 8, 2, 64, 64, [130, 100, 70], seed=31, capacity_pages=16)
     ids2, slots2 = _newest(case2)
-    assert _step(exe, case2, ids2, slots2, new_k, new_v, 1, kernel=kernel)[3] == 1
+    assert _step(exe, case2, ids2, slots2, new_k, new_v, 1)[3] == 1
