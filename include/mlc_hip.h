@@ -235,8 +235,9 @@ int mlc_hip_matmul_q6_k_batched(const char* weight_name, const void* weights, si
  *   q  fp16 [batch][chunk][num_heads][head_dim]; row i of request r sits at
  *      absolute position q_start[r] + i and attends kv positions <= that and
  *      < seq_lens[r].   o  fp32, same shape as q.
- * page_table_offsets has batch entries; request r's table holds at least
- * ceil(seq_lens[r] / page_size_tokens) page ids from there on.
+ * page_table_offsets has batch + 1 entries (the last one is the number of page ids in use, as
+ * in the decode call, metal_runtime.mm:7747); request r's table holds at least
+ * ceil(seq_lens[r] / page_size_tokens) page ids from page_table_offsets[r] on.
  * sync as above (0 needs an open pass). */
 int mlc_hip_paged_attn_prefill(const void* q_f16, const void* k_pages, const void* v_pages,
                                void* o,
@@ -250,10 +251,11 @@ int mlc_hip_paged_attn_prefill(const void* q_f16, const void* k_pages, const voi
 /* Decode attention for callers that cannot allocate (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
  * Same result as mlc_hip_paged_attn_decode (same kernel), but the call itself allocates no device
- * or pinned memory and creates no stream or event: the kernel's scratch memory (split-K partial results and
- * arrival counters, 8.5 MiB) is a static device array that every GPU the library runs on holds
- * until the process ends; seq_lens, q_positions and page_table_offsets (HOST arrays, as above)
- * travel inside the kernel arguments; the flat page table is read where the caller keeps it:
+ * or pinned memory and creates no stream or event: the kernel's scratch memory (the split-K partial
+ * results, 8.5 MiB) is a static device array that every GPU the library runs on holds until the
+ * process ends; seq_lens [batch], q_positions [batch] and page_table_offsets [batch + 1] (HOST
+ * arrays, as in the decode call) travel inside the kernel arguments; the flat page table is read
+ * where the caller keeps it:
  *   page_tables_flat_device  DEVICE pointer to n_page_tables_flat uint32 page ids (4-byte aligned)
  *   stream                   hipStream_t to launch on; NULL = the library's stream
  * Limits, refused with an error otherwise: batch <= 256; head_dim 64 or 128; GQA ratio 1, 2, 4, 8,
@@ -261,8 +263,12 @@ int mlc_hip_paged_attn_prefill(const void* q_f16, const void* k_pages, const voi
  * pools 16-byte aligned.  mlc_hip_available() must have returned 1 before (set-up creates the
  * library's stream and looks up the scratch array's device address).  The call returns when the
  * kernel is enqueued (no synchronisation).  Every decode launch of this library on one GPU
- * uses the same scratch array: launches must not overlap (two streams without an ordering
- * between them race).  The page ids cannot be checked on the host; for pools obtained from
+ * uses the same scratch array, so they must follow each other: the library remembers the stream
+ * of the last one and puts a launch on another stream behind what that stream held at the time
+ * (events created at set-up); what the caller enqueues on its own streams by other means is the
+ * caller's to order.  Operators that earlier encode calls held back are launched first, on the
+ * library's stream, and a caller's stream is put behind them.  Not possible while a pass is
+ * being captured.  The page ids cannot be checked on the host; for pools obtained from
  * mlc_hip_alloc the kernel clamps them below the pool's size. */
 int mlc_hip_paged_attn_decode_noalloc(const void* q, const void* k_pages, const void* v_pages, void* o,
                                       const uint32_t* page_tables_flat_device, size_t n_page_tables_flat,
@@ -296,9 +302,12 @@ int mlc_hip_paged_attn_decode_noalloc(const void* q, const void* k_pages, const 
  * which moves a device word on by which the decode launches of one replay tell their split-K
  * partials from those of the replay before.
  *
- * mlc_hip_replay_update copies the step's tables over the device copies the captured launches
- * read (same addresses, ordered on the library's stream) and checks what the capture took for
- * granted: the same batch size; tables that cover their seq_lens; if the attention launch of the
+ * mlc_hip_replay_update copies the step's tables (seq_lens [batch], q_positions [batch],
+ * page_table_offsets [batch + 1], the flat table; page_ids / slots_in_page [batch]) over the
+ * device copies the captured launches read (same addresses, ordered on the library's stream) and
+ * checks what the capture took for granted: the same batch size; tables that cover their
+ * seq_lens; that no device buffer of the library which the pass may read (weights, norm vectors,
+ * named buffers, the tables' copy) was freed or moved since the capture; if the attention launch of the
  * captured pass does the step's KV write, that (page_ids, slots_in_page) are every request's newest
  * position on pages no two requests share.  It returns 0 when the step cannot be replayed (encode
  * it uncaptured; capture again if it said the copies had to move).  page_ids / slots_in_page may

@@ -228,6 +228,13 @@ struct Ctx {
     int n_cu = 256;
     unsigned char* scratch_ptr = nullptr;   // device address of `scratch` on g.device
     uint32_t next_tag = 0;                  // tag of the last tile-balanced decode launch (never zero)
+    // Every decode launch on this GPU uses the one scratch array, so launches on different
+    // streams must follow each other: the stream of the last launch is remembered, and a launch
+    // on another stream first waits for that one (one event, created at set-up; launches that
+    // stay on the library's stream cost nothing).
+    hipStream_t scratch_stream = nullptr;
+    bool scratch_in_use = false;
+    hipEvent_t scratch_ev = nullptr;
     // One word of pinned host memory that the decode kernel sets (through its device address) when a
     // merge gives up waiting for another workgroup's partial; looked at wherever the host has
     // waited for the stream.
@@ -262,10 +269,14 @@ struct Ctx {
         int causal = 0;
         bool carried_kv = false;             // ... and does the step's KV write
         size_t n_decode = 0;                 // tile-balanced decode launches of the pass
+        uint64_t buffer_generation = 0;      // Ctx::buffer_generation when the pass was captured
         const void* ids_dev = nullptr;       // device copy of the KV write's page ids and slots
         size_t ids_batch = 0;
     };
     std::map<int, Captured> captures;
+    // Counts the times a device buffer that the library owns (and a captured launch may have its
+    // address baked in) was freed or moved: a capture taken at another count is stale.
+    uint64_t buffer_generation = 0;
     int next_capture = 1;
     Captured cap;                            // the pass being captured
 };
@@ -309,6 +320,7 @@ bool init_once() {
     }
     if (hipStreamCreateWithFlags(&g.stream, hipStreamNonBlocking) != hipSuccess) return false;
     if (hipEventCreate(&g.ev0) != hipSuccess || hipEventCreate(&g.ev1) != hipSuccess) return false;
+    if (hipEventCreateWithFlags(&g.scratch_ev, hipEventDisableTiming) != hipSuccess) return false;
     g.available = true;
     return true;
 }
@@ -354,7 +366,8 @@ size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 const void* resident_blob(int kind, const void* key, const void* blob, size_t bytes) {
     // A caller that never repeats itself: start over -- but only while no held-back operator
     // refers to one of the copies (their launches come later).
-    if (g.resident.size() > 1024 && !g.rows.active && !g.kv.active && !g.gemm.active && !g_capturing) {
+    if (g.resident.size() > 1024 && !g.rows.active && !g.kv.active && !g.gemm.active && !g_capturing &&
+        g.captures.empty()) {   // (a captured pass keeps the addresses of the copies it read)
         if (hipStreamSynchronize(g.stream) != hipSuccess) { fail("resident: synchronize failed"); return nullptr; }
         for (auto& kv : g.resident)
             if (kv.second.dev) (void)hipFree(kv.second.dev);
@@ -365,6 +378,7 @@ const void* resident_blob(int kind, const void* key, const void* blob, size_t by
     if (bytes > r.cap) {
         if (g_capturing) { fail("capture: a small host array is not on the device yet (run the pass once uncaptured first)"); return nullptr; }
         if (r.dev && hipFree(r.dev) != hipSuccess) { fail("resident: hipFree failed"); return nullptr; }
+        if (r.dev) ++g.buffer_generation;
         r.dev = nullptr;
         r.cap = 0;
         const size_t cap = std::max<size_t>(256, align_up(bytes, 256));
@@ -651,26 +665,16 @@ void tables_refresh(const uint32_t* flat, size_t n_flat, const uint32_t* off, si
     }
     t.off.assign(off, off + B + 1);
     // duplicates among the entries the requests own ([off[r], off[r+1]), a superset of what a
-    // call dereferences): generation-stamped array over the page ids
-    static thread_local std::vector<uint32_t> stamp;
-    static thread_local uint32_t generation = 0;
-    if (stamp.size() <= t.max_page) stamp.assign((size_t)t.max_page + 1, 0);
-    if (++generation == 0) {
-        std::fill(stamp.begin(), stamp.end(), 0u);
-        generation = 1;
+    // call dereferences): the owned ids, sorted.  (No table indexed by page id: an id may be any
+    // 32-bit number -- padding, or a corrupt entry that the bounds checks refuse afterwards.)
+    static thread_local std::vector<uint32_t> owned;
+    owned.clear();
+    for (size_t r = 0; r < B; ++r) {
+        const size_t b0 = std::min<size_t>(off[r], n_flat), e = std::min<size_t>(off[r + 1], n_flat);
+        if (e > b0) owned.insert(owned.end(), flat + b0, flat + e);
     }
-    t.shared_pages = 0;
-    for (size_t r = 0; r < B && !t.shared_pages; ++r) {
-        const size_t e = std::min<size_t>(off[r + 1], n_flat);
-        for (size_t i = off[r]; i < e; ++i) {
-            uint32_t& st = stamp[flat[i]];
-            if (st == generation) {
-                t.shared_pages = 1;
-                break;
-            }
-            st = generation;
-        }
-    }
+    std::sort(owned.begin(), owned.end());
+    t.shared_pages = std::adjacent_find(owned.begin(), owned.end()) != owned.end() ? 1 : 0;
 }
 
 // Makes the device copy of the flat table (and of the per-request arrays when `meta3` is
@@ -694,6 +698,7 @@ int tables_upload(const uint32_t* meta3, size_t B, const uint32_t** d_flat, cons
         if (total > t.cap) {
             HIP_OK(hipStreamSynchronize(g.stream));
             if (t.dev) HIP_OK(hipFree(t.dev));
+            if (t.dev) ++g.buffer_generation;
             t.dev = nullptr;
             t.cap = 0;
             HIP_OK(hipMalloc(&t.dev, total));
@@ -793,15 +798,38 @@ const char* stream_pv_name(int hpw, int nw) {
     return m == 3 ? "mfma-p32" : m == 2 ? "mfma" : m == 1 ? "pv16" : "pv32";
 }
 
+// Orders a launch that uses the scratch array on `stream` behind the last one that did (see
+// Ctx::scratch_stream).  The library's own stream lives as long as the library, so the event that
+// marks its last launch is recorded only when another stream shows up; a caller's stream may be
+// gone by then, so the event is recorded right behind a launch on one.  A captured pass runs on
+// the library's stream, where its replays are ordered like any other launch there.
+int scratch_follow(hipStream_t stream) {
+    if (g_capturing) return 1;
+    if (g.scratch_in_use && g.scratch_stream != stream) {
+        if (g.scratch_stream == g.stream) HIP_OK(hipEventRecord(g.scratch_ev, g.stream));
+        HIP_OK(hipStreamWaitEvent(stream, g.scratch_ev, 0));
+    }
+    return 1;
+}
+int scratch_launched(hipStream_t stream) {
+    if (g_capturing) return 1;
+    g.scratch_stream = stream;
+    g.scratch_in_use = true;
+    if (stream != g.stream) HIP_OK(hipEventRecord(g.scratch_ev, stream));
+    return 1;
+}
+
 bool launch_stream_variant(size_t D, int hpw, int nw, int nbuf, const StreamArgs& a, unsigned n_wg, size_t dyn_lds,
                            hipStream_t stream) {
+    if (!scratch_follow(stream)) return false;
     const int pvm = stream_pv_mode(hpw, nw);
+    bool launched = false;
 #define MLC_CASE(d, h) \
-    if (D == d && hpw == h) return launch_decode_stream_##d##_##h(nw, nbuf, pvm, a, n_wg, dyn_lds, stream);
+    if (D == d && hpw == h) launched = launch_decode_stream_##d##_##h(nw, nbuf, pvm, a, n_wg, dyn_lds, stream);
     MLC_CASE(64, 1) MLC_CASE(64, 2) MLC_CASE(64, 4) MLC_CASE(64, 8)
     MLC_CASE(128, 1) MLC_CASE(128, 2) MLC_CASE(128, 4) MLC_CASE(128, 8)
 #undef MLC_CASE
-    return false;
+    return launched && scratch_launched(stream);
 }
 
 void stream_fill_common(StreamArgs& a, const void* q, const void* k_pages, const void* v_pages, void* o,
@@ -881,6 +909,7 @@ void* cached_buffer(const char* name, size_t bytes) {
         (void)hipStreamSynchronize(g.stream);
         g.allocs.erase(it->second.first);
         (void)hipFree(it->second.first);
+        ++g.buffer_generation;
         g.cached.erase(it);
     }
     void* p = nullptr;
@@ -1174,7 +1203,18 @@ int mlc_hip_paged_attn_decode_noalloc(const void* q, const void* k_pages, const 
     // the file-scope device array whose address init_once() looked up; the per-request arrays travel
     // inside the kernel arguments and the page table stays where the caller keeps it.
     if (!g.inited || !g.available) return fail("decode (no allocation): call mlc_hip_available() once at set-up");
-    if (!settle()) return 0;  // operators held back by earlier encode calls are launched (kernel launches only)
+    if (g_capturing) return fail("decode (no allocation): not while a pass is being captured (the captured launch would keep this call's lengths)");
+    hipStream_t st = stream ? static_cast<hipStream_t>(stream) : g.stream;
+    {
+        // operators held back by earlier encode calls are launched now, on the library's stream
+        // (kernel launches only); a caller's stream of its own is put behind them
+        const bool pending = g.rows.active || g.kv.active || g.gemm.active;
+        if (!settle()) return 0;
+        if (pending && st != g.stream) {
+            HIP_OK(hipEventRecord(g.scratch_ev, g.stream));
+            HIP_OK(hipStreamWaitEvent(st, g.scratch_ev, 0));
+        }
+    }
     if (!q || !k_pages || !v_pages || !o) return fail("decode: null buffer");  // metal_runtime.mm:7742-7750
     if (batch == 0 || num_heads == 0 || head_dim == 0 || page_size_tokens == 0) return fail("decode: zero dimension");
     if (kv_heads == 0 || (num_heads % kv_heads) != 0) return fail("decode: heads % kv_heads != 0");
@@ -1227,7 +1267,6 @@ int mlc_hip_paged_attn_decode_noalloc(const void* q, const void* k_pages, const 
     std::memcpy(a.emb, seq_lens, batch * 4);
     std::memcpy(a.emb + emb_stride, q_positions, batch * 4);
     std::memcpy(a.emb + 2 * emb_stride, page_table_offsets, batch * 4);
-    hipStream_t st = stream ? static_cast<hipStream_t>(stream) : g.stream;
     if (!launch_stream_variant(head_dim, hpw, nw, nbuf, a, n_wg, dyn_lds, st))
         return fail("decode: kernel variant not built");
     HIP_OK(hipGetLastError());
@@ -1716,7 +1755,7 @@ Ctx::Q4Weight* q4_weight(const char* name, const uint8_t* host, size_t bytes, si
     if (g_capturing) { fail("q4 matmul: the weights are not on the device yet (run the pass once uncaptured first)"); return nullptr; }
     (void)hipStreamSynchronize(g.stream);
     for (void** p : {&w.raw, &w.qs, &w.d})
-        if (*p) { (void)hipFree(*p); *p = nullptr; }
+        if (*p) { (void)hipFree(*p); *p = nullptr; ++g.buffer_generation; }
     w = Ctx::Q4Weight{};
     void* raw = nullptr;
     if (hipMalloc(&raw, bytes) != hipSuccess) { (void)hipGetLastError(); fail("q4 matmul: hipMalloc failed"); return nullptr; }
@@ -1874,7 +1913,7 @@ Ctx::Q6KWeight* q6k_weight(const char* name, const uint8_t* host, size_t bytes, 
     if (g_capturing) { fail("q6_k matmul: the weights are not on the device yet (run the pass once uncaptured first)"); return nullptr; }
     (void)hipStreamSynchronize(g.stream);
     for (void** p : {&w.raw, &w.qa, &w.sc, &w.d})
-        if (*p) { (void)hipFree(*p); *p = nullptr; }
+        if (*p) { (void)hipFree(*p); *p = nullptr; ++g.buffer_generation; }
     w = Ctx::Q6KWeight{};
     void* raw = nullptr;
     if (hipMalloc(&raw, bytes) != hipSuccess) { (void)hipGetLastError(); fail("q6_k matmul: hipMalloc failed"); return nullptr; }
@@ -2118,6 +2157,7 @@ int mlc_hip_capture_end(void) {
         return fail("capture: hipGraphInstantiate failed");
     }
     Ctx::Captured c = g.cap;
+    c.buffer_generation = g.buffer_generation;
     c.graph = graph;
     c.exec = exec;
     c.n_nodes = count - 1;   // (not counted: the library's own first launch, which moves the replay word on)
@@ -2140,6 +2180,8 @@ int mlc_hip_replay_update(int handle, const uint32_t* page_tables_flat, size_t n
     auto it = g.captures.find(handle);
     if (it == g.captures.end()) return fail("replay: unknown handle");
     const Ctx::Captured& c = it->second;
+    if (c.buffer_generation != g.buffer_generation)
+        return fail("replay: a device buffer of the library was freed or moved since the capture (capture again)");
     if (!settle()) return 0;
     if (c.used_tables) {
         if (!page_table_offsets || !seq_lens || !q_positions || (n_flat && !page_tables_flat))
@@ -2155,7 +2197,9 @@ int mlc_hip_replay_update(int handle, const uint32_t* page_tables_flat, size_t n
             if (c.causal && (uint64_t)q_positions[r] + 1 < lim) lim = (uint64_t)q_positions[r] + 1;
             total_tiles += (lim + tile - 1) / tile;
         }
-        if (total_tiles * c.Hkv >= 0x7FFFFFFFull) return fail("replay: too many KV tiles for the captured kernel");
+        // (the same bound as the encode path: the kernel counts in units, tiles plus at most 64 per pair)
+        if (total_tiles * c.Hkv + 64ull * batch * c.Hkv >= 0x7FFFFFFFull)
+            return fail("replay: too many KV tiles for the captured kernel");
         tables_refresh(page_tables_flat, n_flat, page_table_offsets, batch);
         static thread_local std::vector<uint32_t> meta3;
         meta3.resize(3 * batch);
@@ -2198,8 +2242,12 @@ int mlc_hip_replay(int handle) {
     NOT_WHILE_CAPTURING("replay");
     auto it = g.captures.find(handle);
     if (it == g.captures.end()) return fail("replay: unknown handle");
+    if (it->second.buffer_generation != g.buffer_generation)
+        return fail("replay: a device buffer of the library was freed or moved since the capture (capture again)");
     if (!settle()) return 0;
+    if (it->second.n_decode && !scratch_follow(g.stream)) return 0;
     HIP_OK(hipGraphLaunch(it->second.exec, g.stream));
+    if (it->second.n_decode && !scratch_launched(g.stream)) return 0;
     return 1;
 }
 

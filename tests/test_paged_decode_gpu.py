@@ -353,3 +353,42 @@ def test_baseline_config4_full_size(exe, decode_kernel):
         want = oracle_decode(sub)
         assert want is not None
         assert_parity(got[r:r + 1], want, case.head_dim, f"cfg4 request {r}")
+
+
+def test_a_merge_that_never_sees_its_partials_gives_up_and_the_pass_fails(exe):
+    """Forced from the host: workgroups do not publish their partials (a test switch of the kernel)
+    and the wait is cut to a few rounds, so every workgroup that sums up a split pair gives up,
+    sets the fault word and leaves; the kernel ends normally, the synchronous call reports the
+    failure, and the next call is served as usual."""
+    case = baseline_config(2, batch=6)
+    dev = DeviceCase(exe, case)
+    try:
+        assert exe.setOption("decode_test_flags", 1) and exe.setOption("decode_spin_limit", 3)
+        args = (dev.q_buf, dev.k_buf, dev.v_buf, dev.o_buf, case.page_tables_flat, case.page_table_offsets,
+                case.seq_lens, case.q_positions, case.batch, case.num_heads, case.kv_heads, case.head_dim,
+                case.page_size, case.apply_causal)
+        assert not exe.runPagedFlashAttention(*args)
+        assert "gave up" in exe.lastError()
+        assert exe.setOption("decode_test_flags", 0) and exe.setOption("decode_spin_limit", 200000)
+        got = dev.run()
+    finally:
+        exe.setOption("decode_test_flags", 0)
+        exe.setOption("decode_spin_limit", 200000)
+        dev.free()
+    assert_parity(got, oracle_decode(case), 64, "after a failed pass")
+
+
+def test_page_table_padded_with_all_ones_is_served(exe):
+    """A flat table with entries no request uses (0xFFFFFFFF padding between the requests' slices):
+    the host checks look only at the entries in use, and no host table is sized by the largest id."""
+    import dataclasses
+    case = make_case("padded", 3, 8, 2, 64, 64, [300, 70, 129], capacity_pages=16, seed=5)
+    off = case.page_table_offsets
+    flat, new_off = [], [0]
+    for r in range(3):
+        flat += list(case.page_tables_flat[off[r]:off[r + 1]]) + [0xFFFFFFFF] * 3
+        new_off.append(len(flat))
+    # every request's slice now ends with three unused entries; its used entries are unchanged
+    padded = dataclasses.replace(case, page_tables_flat=np.array(flat, np.uint32),
+                                 page_table_offsets=np.array([new_off[0], new_off[1], new_off[2], new_off[3]], np.uint32))
+    _check(exe, padded)

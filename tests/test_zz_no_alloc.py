@@ -3,8 +3,10 @@
 Both run the same tile-balanced kernel; the one under test takes the flat page table as a device
 pointer, the per-request arrays inside the kernel arguments and its scratch memory from the
 library's static device array.  Called twice in a row, the second time with a smaller batch, so
-that whatever the first call left in the shared scratch array (partials, arrival counters) must not
-leak into the second."""
+that whatever the first call left in the shared scratch array (the partials) must not leak into
+the second.  Also on a stream of the caller's own, between launches on the library's stream (the
+library orders the launches that share its scratch array), and with the device's free memory
+read before and after the calls."""
 import ctypes as C
 
 import numpy as np
@@ -96,3 +98,70 @@ def test_noalloc_refuses_what_it_cannot_serve():
         assert b"256" in lib.mlc_hip_last_error()
     finally:
         exe.releaseScratchBuffer(buf)
+
+
+def _hip():
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipStreamCreate.argtypes = [C.POINTER(C.c_void_p)]
+    hip.hipStreamSynchronize.argtypes = [C.c_void_p]
+    hip.hipStreamDestroy.argtypes = [C.c_void_p]
+    hip.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+    return hip
+
+
+def test_noalloc_on_a_second_stream_between_launches_on_the_library_stream():
+    """Launches on the library's stream and on a stream of the caller's alternate, all of them using
+    the one scratch array, none of them waited for in between: every output must be what the
+    ordinary entry point gives, and the no-allocation calls must leave the device's free memory
+    as it was."""
+    exe = HipExecutor.Instance()
+    exe.requireAvailable()
+    lib = load()
+    hip = _hip()
+    stream = C.c_void_p()
+    assert hip.hipStreamCreate(C.byref(stream)) == 0
+    c = baseline_config(2)
+    rounds = 6
+    nbytes = c.q.nbytes
+    q, k, v = (exe.allocateScratchBuffer(n) for n in (nbytes, c.k_pages.nbytes, c.v_pages.nbytes))
+    outs_lib = [exe.allocateScratchBuffer(nbytes) for _ in range(rounds)]
+    outs_own = [exe.allocateScratchBuffer(nbytes) for _ in range(rounds)]
+    flat = np.ascontiguousarray(c.page_tables_flat, dtype=np.uint32)
+    d_flat = exe.allocateScratchBuffer(flat.nbytes)
+    off, seq, qpos = (np.ascontiguousarray(a, dtype=np.uint32) for a in (c.page_table_offsets, c.seq_lens, c.q_positions))
+    try:
+        exe.uploadToBuffer(q, c.q)
+        exe.uploadToBuffer(k, c.k_pages)
+        exe.uploadToBuffer(v, c.v_pages)
+        exe.uploadToBuffer(d_flat, flat)
+        want = np.empty_like(c.q)
+        assert exe.runPagedFlashAttention(q, k, v, outs_lib[0], c.page_tables_flat, c.page_table_offsets, c.seq_lens,
+                                          c.q_positions, c.batch, c.num_heads, c.kv_heads, c.head_dim, c.page_size,
+                                          c.apply_causal), exe.lastError()
+        exe.downloadFromBuffer(outs_lib[0], want)
+        for o in outs_lib + outs_own:
+            exe.zeroBuffer(o, nbytes)
+        assert exe.flushForwardPassCB()
+        free0, total = C.c_size_t(), C.c_size_t()
+        assert hip.hipMemGetInfo(C.byref(free0), C.byref(total)) == 0
+        assert exe.beginForwardPassCB()
+        for i in range(rounds):
+            assert exe.encodePagedFlashAttention(q, k, v, outs_lib[i], c.page_tables_flat, c.page_table_offsets, c.seq_lens,
+                                                 c.q_positions, c.batch, c.num_heads, c.kv_heads, c.head_dim, c.page_size,
+                                                 c.apply_causal), exe.lastError()
+            assert lib.mlc_hip_paged_attn_decode_noalloc(q, k, v, outs_own[i], d_flat, flat.size, _u32p(off), _u32p(seq),
+                                                         _u32p(qpos), c.batch, c.num_heads, c.kv_heads, c.head_dim,
+                                                         c.page_size, int(c.apply_causal), stream), exe.lastError()
+        assert hip.hipStreamSynchronize(stream) == 0
+        assert exe.flushForwardPassCB(), exe.lastError()
+        free1 = C.c_size_t()
+        assert hip.hipMemGetInfo(C.byref(free1), C.byref(total)) == 0
+        assert free1.value == free0.value, (free0.value, free1.value)
+        got = np.empty_like(c.q)
+        for o in outs_lib + outs_own:
+            exe.downloadFromBuffer(o, got)
+            assert np.array_equal(got, want), float(np.abs(got - want).max())
+    finally:
+        for buf in [q, k, v, d_flat] + outs_lib + outs_own:
+            exe.releaseScratchBuffer(buf)
+        hip.hipStreamDestroy(stream)
