@@ -31,7 +31,6 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
-sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
@@ -84,7 +83,7 @@ def bench_prefill(args) -> dict:
 
     from mlcompiler_amd import HipExecutor
     from mlcompiler_amd.build import BENCH_LIB_PATH
-    from test_paged_prefill_gpu import make_prefill, oracle
+    from mlcompiler_amd.workloads import make_prefill
     exe = HipExecutor.Instance()
     exe.requireAvailable()
     if args.prefill_stages and not exe.setOption("prefill_stages", args.prefill_stages):
@@ -145,7 +144,8 @@ def bench_prefill(args) -> dict:
         sub["C"] = rows
         sub["q"] = np.ascontiguousarray(w["q"].reshape(B, Cc, H * D)[0, :rows]).ravel()
         t0 = time.perf_counter()
-        want = oracle(sub, n_threads=1)
+        want = po.paged_attention_prefill(sub["q"], sub["k"], sub["v"], sub["flat"], sub["off"], sub["seq"],
+                                          sub["q_start"], 1, rows, H, Hkv, D, P, 1)
         dt = time.perf_counter() - t0
         f_s = 4 * D * H * sum(ctx + i + 1 for i in range(rows))
         got = np.empty((B, Cc, H, D), np.float32)
@@ -159,16 +159,18 @@ def bench_prefill(args) -> dict:
     return result
 
 
-def bench_layer(args) -> int:
+def bench_layer(args, workload=None, steps=None) -> dict:
     """One whole decoder layer per step (TinyLlama-1.1B shape, Q4_0 weights) around the paged
     decode attention of configuration 2: the eleven operators of the reference's layer loop
     (compiler/runtime/batched_walker.cpp:246-405) enqueued through the C ABI with no host wait
     between them.  Reports the algorithmic bytes (Q4_0 weights + KV read) per second."""
     import ctypes as C
 
-    import layer_case as lc
     from mlcompiler_amd import HipExecutor
+    from mlcompiler_amd import workloads as lc
     from mlcompiler_amd.build import BENCH_LIB_PATH
+    workload = workload or args.workload
+    steps = steps or args.steps
     exe = HipExecutor.Instance()
     exe.requireAvailable()
     if args.q4_ksplit:
@@ -188,19 +190,25 @@ def bench_layer(args) -> int:
                          for r in range(B)], np.uint32)
     slots = (qpos % c.page_size).astype(np.uint32)
 
-    keep = []
+    keep, held = [], []
 
     def up(a):
         a = np.ascontiguousarray(a)
         b = exe.allocateScratchBuffer(a.nbytes)
         assert b and exe.uploadToBuffer(b, a), "out of device memory"
         keep.append(a)
+        held.append(b)
         return b
 
     def dev(n_floats):
         b = exe.allocateScratchBuffer(n_floats * 4)
         assert b
+        held.append(b)
         return b
+
+    def release():
+        while held:
+            exe.releaseScratchBuffer(held.pop())
 
     k_bufs = [up(c.k_pages) for _ in range(n_layers)]
     v_bufs = [up(c.v_pages) for _ in range(n_layers)]
@@ -244,12 +252,10 @@ def bench_layer(args) -> int:
     enqueue_s = C.c_double()
     L.enqueue_s = C.pointer(enqueue_s)
 
-    whole_step = args.workload == "step"
-    VOCAB = 32000
+    whole_step = workload == "step"
+    VOCAB = lc.VOCAB
     if whole_step:   # final RMSNorm + Q6_K lm_head after every 22nd layer: one decode step of the model
-        from oracle import paged_oracle as po
-        head_norm = rng.uniform(0.5, 1.5, lc.HID).astype(np.float32)
-        w_head = po.quantize_q6_k((rng.standard_normal((VOCAB, lc.HID)) * 0.03).astype(np.float32))
+        head_norm, w_head = lc.make_head_weights(rng)
         keep.extend([head_norm, w_head])
         L.head_norm_w = head_norm.ctypes.data_as(f32p)
         L.head_w, L.head_bytes, L.head_rows = w_head.ctypes.data, w_head.nbytes, VOCAB
@@ -271,14 +277,18 @@ def bench_layer(args) -> int:
     # residual add of one layer and the RMSNorm of the next are neighbours in the pass)
     L.out2 = dev(B * lc.HID)
     if whole_step:
-        return finish_step(args, exe, L, loop, lc, c, w, x, cos, sin, page_ids, slots, qpos, n_layers,
-                           VOCAB, head_norm, w_head)
-    ev_ms, wall = loop(args.steps)
-    host_encode_us = enqueue_s.value / args.steps * 1e6
+        try:
+            return finish_step(args, steps, exe, L, loop, lc, c, w, x, cos, sin, page_ids, slots, qpos,
+                               n_layers, VOCAB, head_norm, w_head)
+        finally:
+            release()
+    enqueue_s.value = 0.0
+    ev_ms, wall = loop(steps)
+    host_encode_us = enqueue_s.value / steps * 1e6
     graph_us = graph_nodes = None
     if args.graph:   # the same n_layers launches captured once into a HIP graph and replayed
         g_ms, g_nodes = C.c_float(), C.c_size_t()
-        replays = max(1, args.steps // n_layers)
+        replays = max(1, steps // n_layers)
         loop(n_layers)                   # the same pass launched call by call: the replays must reproduce it
         eager_out = np.empty((B, lc.HID), np.float32)
         exe.downloadFromBuffer(L.out2, eager_out)
@@ -299,13 +309,13 @@ def bench_layer(args) -> int:
 
     w_bytes = lc.weight_bytes(w)
     alg_bytes = w_bytes + c.kv_bytes
-    us = wall / args.steps * 1e6
-    ev_us = ev_ms / args.steps * 1e3
-    value = alg_bytes / (wall / args.steps) / 1e9
+    us = wall / steps * 1e6
+    ev_us = ev_ms / steps * 1e3
+    value = alg_bytes / (wall / steps) / 1e9
     ach = alg_bytes / (ev_us * 1e-6) / 1e9
     result = {
         "metric": "decoder layer (Q4_0 weights + KV read) GB/s & us/layer, TinyLlama shape B=32",
-        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": steps,
         "warmup": max(args.warmup, n_layers), "ms_per_step": round(us / 1e3, 6),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32 (Q4_0 weights, fp16 K/V storage; matmuls on split-fp16 MFMA with fp32 accumulate)",
@@ -329,11 +339,12 @@ def bench_layer(args) -> int:
     }
     if not args.no_cpu:
         from oracle import paged_oracle as po
+        from oracle.layer_chain import oracle_chain
         nb = 8   # bounded sample: the first 8 requests of the batch, one thread
         off = c.page_table_offsets
         flat = c.page_tables_flat[:off[nb]]
         t0 = time.perf_counter()
-        ref = lc.oracle_chain(w, x[:nb], cos[:nb], sin[:nb], c.k_pages, c.v_pages, page_ids[:nb],
+        ref = oracle_chain(w, x[:nb], cos[:nb], sin[:nb], c.k_pages, c.v_pages, page_ids[:nb],
                               slots[:nb], flat, off[:nb + 1], c.seq_lens[:nb], qpos[:nb], n_threads=1)
         dt = time.perf_counter() - t0
         # the CPU reads the weights once per request: bytes that count are per request
@@ -348,17 +359,16 @@ def bench_layer(args) -> int:
         result["parity_vs_cpu_baseline"] = {"cosine": round(po.cosine(got.ravel(), ref["out"].ravel()), 8),
                                             "max_abs_over_max": float(f"{rel:.3e}"),
                                             "requests_checked": nb}
-    print(json.dumps(result))
-    return 0
+    release()
+    return result
 
 
-def finish_step(args, exe, L, loop, lc, c, w, x, cos, sin, page_ids, slots, qpos, n_layers, VOCAB,
-                head_norm, w_head) -> int:
+def finish_step(args, steps, exe, L, loop, lc, c, w, x, cos, sin, page_ids, slots, qpos, n_layers, VOCAB,
+                head_norm, w_head) -> dict:
     """--workload step: times whole decode steps of a TinyLlama-1.1B-shape model (22 decoder
     layers, final RMSNorm, Q6_K lm_head) and checks the logits of one step against the CPU chain."""
-    from oracle import paged_oracle as po
     B = c.batch
-    steps = max(1, min(args.steps, 200))
+    steps = max(1, min(steps, 200))
     loop(n_layers)                                  # first use of the lm_head: upload and repack
     ev_ms, wall = loop(steps * n_layers)
     loop(n_layers)                                  # one step from the known input, for the parity check
@@ -391,14 +401,16 @@ def finish_step(args, exe, L, loop, lc, c, w, x, cos, sin, page_ids, slots, qpos
                              "weights once + the K/V of all layers"},
     }
     if not args.no_cpu:
-        nb = 16   # bounded sample: the first 16 requests through all 22 layers and the head, 8 threads
-        off = c.page_table_offsets
+        from oracle import paged_oracle as po
+        from oracle.layer_chain import oracle_chain
+        nb = 16 if args.workload == "step" else 4   # bounded sample: the first requests of the batch through all
+        off = c.page_table_offsets                    # 22 layers and the head, 8 threads
         flat = c.page_tables_flat[:off[nb]]
         n_thr = min(os.cpu_count() or 1, 8)
         t0 = time.perf_counter()
         h = x[:nb]
         for _ in range(n_layers):
-            h = lc.oracle_chain(w, h, cos[:nb], sin[:nb], c.k_pages, c.v_pages, page_ids[:nb], slots[:nb],
+            h = oracle_chain(w, h, cos[:nb], sin[:nb], c.k_pages, c.v_pages, page_ids[:nb], slots[:nb],
                                 flat, off[:nb + 1], c.seq_lens[:nb], qpos[:nb], n_threads=n_thr)["out"]
         hn = po.rms_norm_batched(h, head_norm, 1e-5, nb, lc.HID)
         want = po.matmul_q6_k_batched(w_head, hn, nb, VOCAB, lc.HID, n_threads=n_thr)
@@ -411,12 +423,11 @@ def finish_step(args, exe, L, loop, lc, c, w, x, cos, sin, page_ids, slots, qpos
             "max_abs_over_max": float(f"{float(np.max(np.abs(got - want)) / np.max(np.abs(want))):.3e}"),
             "argmax_agree": int(np.sum(np.argmax(got, axis=1) == np.argmax(want, axis=1))),
             "requests_checked": nb}
-    print(json.dumps(result))
-    return 0
+    return result
 
 
 def build_workload(name: str):
-    from paged_cases import baseline_config
+    from mlcompiler_amd.workloads import baseline_config
     idx = {"cfg1": 1, "cfg2": 2, "cfg3": 3, "cfg4": 4}[name]
     case = baseline_config(idx)
     layers = {"cfg1": 22, "cfg2": 22, "cfg3": 8, "cfg4": 1}[name]
@@ -822,14 +833,14 @@ def per_config_entry(name: str, r: dict) -> dict:
     return e
 
 
-def bench_refbench(args) -> int:
+def bench_refbench(args) -> dict:
     """The reference's own micro-benchmark grid (tools/paged_flash_bench.cpp:29-34, 206-226):
     32 query heads, 4 KV heads, head_dim 64, one 64-token page per request, batch 1, 2, 4, 8;
     3 warm-up calls, then 200 synchronous runPagedFlashAttention calls timed one by one on the
     host clock (as the reference's harness does, :55-76), median / p10 / p90 in microseconds; beside
     it the same calls timed with a HIP event pair on the stream."""
     from mlcompiler_amd import HipExecutor
-    from paged_cases import DeviceCase, make_case
+    from mlcompiler_amd.workloads import DeviceCase, make_case
     exe = HipExecutor.Instance()
     exe.requireAvailable()
     rows = []
@@ -861,14 +872,13 @@ def bench_refbench(args) -> int:
         pick = lambda v: {"median": round(v[len(v) // 2], 2), "p10": round(v[len(v) // 10], 2),
                           "p90": round(v[len(v) * 9 // 10], 2)}
         rows.append({"batch": b, "host_sync_call_us": pick(host), "stream_event_us": pick(dev), "n": len(host)})
-    print(json.dumps({"metric": "paged flash attention micro-benchmark of the reference (median us per call)",
+    return ({"metric": "paged flash attention micro-benchmark of the reference (median us per call)",
                       "value": rows[-1]["host_sync_call_us"]["median"], "unit": "us", "n_gpus": 1, "steps": 200,
                       "warmup": 3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
                       "dtype": "f32 (fp16 K/V storage, fp32 q, accumulate and output)", "data": "synthetic",
                       "config": {"workload": "tools/paged_flash_bench.cpp grid: 32q/4kv heads, head_dim 64, one "
                                              "64-token page per request, batch 1/2/4/8, uniform(-0.5, 0.5) inputs",
-                                 "rows": rows}}))
-    return 0
+                                 "rows": rows}})
 
 
 def main() -> int:
@@ -916,9 +926,11 @@ def main() -> int:
     if args.workload == "copy":
         return bench_copy(args)
     if args.workload == "refbench":
-        return bench_refbench(args)
+        print(json.dumps(bench_refbench(args)))
+        return 0
     if args.workload in ("layer", "step"):
-        return bench_layer(args)
+        print(json.dumps(bench_layer(args)))
+        return 0
 
     from mlcompiler_amd import HipExecutor
     exe = HipExecutor.Instance()
@@ -1013,6 +1025,18 @@ def main() -> int:
                       "us_per_step": p5["roofline"]["us_per_launch"], "TFLOPs": p5["roofline"]["achieved"],
                       "frac_of_mfma_f16_peak": p5["roofline"]["frac"], "traffic": p5["roofline"]["traffic"],
                       **{k: p5[k] for k in ("cpu_baseline", "parity_vs_cpu_baseline") if k in p5}}
+        # the reference's own micro-benchmark grid, one decoder layer and one whole decode step
+        rb = bench_refbench(args)
+        pc["refbench"] = {"workload": rb["config"]["workload"], "calls_per_batch": 200, "rows": rb["config"]["rows"]}
+        for name, st in (("layer", 2000), ("step", 100)):
+            sub = bench_layer(args, name, st)
+            pc[name] = {"workload": sub["config"]["workload"], "steps": sub["steps"], "metric": sub["metric"],
+                        "value": sub["value"], "unit": sub["unit"], "us_per_step": round(sub["ms_per_step"] * 1e3, 2),
+                        **{k: sub["config"][k] for k in ("weight_bytes_per_step", "kv_bytes_per_step", "us_per_layer",
+                                                        "host_encode_us_per_layer", "tokens_per_s_at_22_layers")
+                           if k in sub["config"]},
+                        "frac_of_hbm_peak": sub["roofline"]["frac"],
+                        **{k: sub[k] for k in ("cpu_baseline", "parity_vs_cpu_baseline") if k in sub}}
         result["config"]["per_config"] = pc
     print(json.dumps(result))
     return 0

@@ -697,3 +697,35 @@ def test_q6_k_bit_exact_with_reference_build():
             for r in range(4):
                 want = R.ref_dot_q6_k(q[r].ctypes.data, cols, x[b].ctypes.data_as(po._f32p))
                 assert np.float32(want).view(np.uint32) == got[b, r].view(np.uint32)
+
+
+def test_numpy_q4_0_encoder_is_bit_identical_to_the_oracle_quantiser():
+    """The workload module's vectorised Q4_0 encoder against the oracle's restatement of
+    quantizeRowQ4_0, including all-zero blocks and blocks whose extreme value is negative."""
+    from mlcompiler_amd import workloads as wl
+    rng = np.random.default_rng(5)
+    w = (rng.standard_normal((37, 256)) * 0.05).astype(np.float32)
+    w[3, 32:64] = 0.0
+    w[5, :32] = -np.abs(w[5, :32])
+    w[6, :32] = np.abs(w[6, :32])
+    assert np.array_equal(wl.quantize_q4_0(w), po.quantize_q4_0(w))
+
+
+def test_numpy_q6_k_encoder_decodes_within_half_a_step():
+    """The workload module's Q6_K encoder is a plain round-to-nearest one (not the reference's
+    scale search): what it writes must decode, through the oracle's dequantizeRowQ6_K, to within
+    half a quantisation step of the input, and all-zero super-blocks must decode to zero."""
+    from mlcompiler_amd import workloads as wl
+    rng = np.random.default_rng(6)
+    w = (rng.standard_normal((9, 1024)) * 0.03).astype(np.float32)
+    w[2, 256:512] = 0.0
+    enc = wl.quantize_q6_k(w)
+    assert enc.shape == (9, po.q6_k_row_bytes(1024))
+    back = po.dequantize_q6_k(enc, 1024)
+    assert np.all(back[2, 256:512] == 0.0)
+    step = np.abs(w).reshape(9, 64, 16).max(axis=2, keepdims=True) / 31.0
+    err = np.abs(back - w).reshape(9, 64, 16)
+    assert np.all(err <= 0.75 * step + 1e-7), float((err / (step + 1e-12)).max())
+    # and it is about as good as the reference's quantiser on the same input
+    ref = po.dequantize_q6_k(po.quantize_q6_k(w), 1024)
+    assert np.abs(back - w).mean() <= 1.5 * np.abs(ref - w).mean()

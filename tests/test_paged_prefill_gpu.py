@@ -5,27 +5,10 @@ import numpy as np
 import pytest
 
 from oracle import paged_oracle as po
+from mlcompiler_amd.workloads import make_prefill
 from paged_cases import MAX_ABS, MIN_COSINE
 
 pytestmark = pytest.mark.gpu
-
-
-def make_prefill(B, C, H, Hkv, D, P, ctx, seed=0, scale_k=0.0):
-    """ctx[r] cached tokens, then a chunk of C new tokens (already written to the cache)."""
-    rng = np.random.default_rng(seed)
-    ctx = np.asarray(ctx, np.int64)
-    seq = (ctx + C).astype(np.uint32)
-    pages = (seq.astype(np.int64) + P - 1) // P
-    cap = int(pages.sum()) + 3
-    ids = rng.permutation(cap).astype(np.uint32)
-    flat = ids[:int(pages.sum())]
-    off = np.zeros(B + 1, np.uint32)
-    off[1:] = np.cumsum(pages)
-    q = rng.standard_normal((B, C, H, D), dtype=np.float32).astype(np.float16)
-    k = rng.standard_normal(cap * P * Hkv * D, dtype=np.float32).astype(np.float16)
-    v = rng.standard_normal(cap * P * Hkv * D, dtype=np.float32).astype(np.float16)
-    return dict(B=B, C=C, H=H, Hkv=Hkv, D=D, P=P, seq=seq, q_start=ctx.astype(np.uint32), flat=flat,
-                off=off, q=q.view(np.uint16), k=k.view(np.uint16), v=v.view(np.uint16))
 
 
 def run_gpu(exe, w, sync=True):
