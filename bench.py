@@ -1016,8 +1016,8 @@ def main() -> int:
         pc = {}
         # (their own step counts, stated in each entry and independent of --steps: a 20-step region
         # of a 7 us kernel would mostly measure its first launches)
-        for name, st in (("cfg1", 2000), ("cfg3", 500), ("cfg4", 100)):
-            sub = run_decode(args, name, st, 20, 4.0, full=False)
+        for name, st, wu in (("cfg1", 2000, 20), ("cfg3", 500, 20), ("cfg4", 300, 50)):
+            sub = run_decode(args, name, st, wu, 4.0, full=False)
             pc[name] = per_config_entry(name, sub)
         p5 = bench_prefill(args)
         pc["cfg5"] = {"workload": p5["config"]["workload"], "steps": p5["steps"],

@@ -393,7 +393,9 @@ long mlc_hip_decode_table_uploads(void);
  *                           KV head in 4 waves); 0 = on the vector pipe
  *   "prefill_stages"        2, 4, 6 or 8 K/V tiles staged in LDS by the prefill kernel (0 = automatic:
  *                           6); with 8 the kernel with 64 rows per wave lets its waves meet only
- *                           after every second tile
+ *                           after every second tile;
+ *                           the kernel with 64 rows per wave has no 2-stage build and runs 4
+ *                           stages when 2 is asked for
  *   "prefill_rows64"        1 (default) = heads/kv_heads up to 4 run the prefill kernel with 64
  *                           chunk rows per wave; 0 = the kernel with 32 rows per wave for every
  *                           ratio (ratio 8 always runs it)

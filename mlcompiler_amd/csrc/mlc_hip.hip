@@ -247,12 +247,10 @@ struct Ctx {
     long opt_stream_stages = 0;     // tile-balanced kernel: LDS stages per workgroup (0 = automatic)
     long opt_grid_wgs = 0;          // tile-balanced kernel: exact grid size (0 = from workgroups per CU)
     // tile-balanced kernel: units the end of a (request, KV head) pair counts for when the ranges are
-    // cut (a tile is one unit).  -1 = automatic: 4 for workgroups of four waves (swept 0..6 on
-    // MI355X at GQA ratios 4, 8 and 16, head_dim 64 and 128: 3 or 4 was fastest, up to a quarter
-    // faster than 0; 4 is as fast as 3 for the attention alone at the TinyLlama shape and 0.8 us
-    // faster where the launch also carries the step's KV write, and 3 us faster for 16 heads of
-    // 128), 0 for the one- and two-wave workgroups of GQA ratios 1 and 2, whose pair ends are cheap
-    // (there 3 was 1 to 5 % slower than 0).
+    // cut (a tile is one unit).  -1 = automatic: 2 for workgroups of four waves (swept 0..4 on
+    // MI355X at the TinyLlama shape: batch 32 14.3 / 13.5 / 13.4 / 13.5 / 14.1 us, with the step's
+    // KV write carried 15.5 / 14.8 / 13.9 / 14.1 / 14.6 us), 0 for the one- and two-wave workgroups
+    // of GQA ratios 1 and 2, whose pair ends are cheap (there any cost was 1 to 5 % slower than 0).
     long opt_pair_cost = -1;
     long table_uploads = 0;         // page-table uploads of the tile-balanced path (for tests)
     // A captured pass: the kernel launches of the encode calls between mlc_hip_capture_begin and
