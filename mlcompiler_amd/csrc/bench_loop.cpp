@@ -2,6 +2,7 @@
 // the reference (compiler-side harness that calls the executor in a tight loop), so that
 // the measured rate is the GPU's and not the Python interpreter's call overhead.
 // It only calls entry points of include/mlc_hip.h; it adds no kernels of its own.
+#include <algorithm>
 #include <chrono>
 #include <string>
 #include <vector>
@@ -292,7 +293,8 @@ struct MlcBenchLayer {
     // when head_w is set: after every n_layers-th layer the final RMSNorm and the Q6_K lm_head
     // (batched_walker.cpp:415-431), i.e. n_layers steps are one decode step of the model
     const float* head_norm_w; const void* head_w; size_t head_bytes; size_t head_rows; void* logits;
-    double* enqueue_s;        // when set: receives the host time spent encoding (before the wait)
+    double* enqueue_s;        // when set: receives the host time spent encoding (before the wait),
+                              // measured over the first 256 steps and scaled to the loop's steps
 };
 
 // Weight-cache names of layer l's four matrices.
@@ -351,9 +353,15 @@ int mlc_bench_layer_loop(const MlcBenchLayer* L, void* const* k_pools, void* con
     if (!mlc_hip_begin()) return 0;
     const auto t0 = std::chrono::steady_clock::now();
     if (!mlc_hip_timer_start()) return 0;
-    for (size_t i = 0; i < steps; ++i)
+    // (host time of encoding: taken over the first 256 steps and scaled to all of them -- further on
+    // the host is so far ahead of the GPU that the queue is full and encode calls wait for room)
+    const size_t enq_steps = std::min<size_t>(steps, 256);
+    double enq_s = 0.0;
+    for (size_t i = 0; i < steps; ++i) {
         if (!encode_layer_step(L, names, k_pools, v_pools, n_layers, i)) return 0;
-    if (L->enqueue_s) *L->enqueue_s = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+        if (i + 1 == enq_steps) enq_s = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    }
+    if (L->enqueue_s) *L->enqueue_s = enq_s * (double)steps / (double)enq_steps;
     const float ms = mlc_hip_timer_stop();
     if (ms < 0.f) return 0;
     if (!mlc_hip_flush()) return 0;
