@@ -1,6 +1,6 @@
 """Writes tests/golden/walker_tiny_llama.npz: the logits of the reference's own single-stream CPU
 runner (DecodeRunner, compiler/runtime/decode_runner.cpp) on the synthetic model that
-tests/integration/make_tiny_llama_gguf.py writes, for 4 requests x 8 steps -- what the reference's
+tests/integration/make_tiny_llama_gguf.py writes, for 4 requests x 8 steps and (the last steps of) 2 requests x 72 steps -- what the reference's
 walker test compares BatchedWalker::step against (tests/test_batched_walker_h1.cpp:62-180).
 
 Runs in the build container only (needs the reference checkout): it executes
@@ -25,6 +25,9 @@ ROOT = os.path.dirname(os.path.dirname(HERE))
 sys.path.insert(0, os.path.join(ROOT, "tests", "integration"))
 
 REQUESTS, STEPS = 4, 8
+# a second run long enough for every request to open a second 64-token page: 2 requests x 72 steps,
+# of which the last LONG_KEPT steps' logits are kept
+LONG_REQUESTS, LONG_STEPS, LONG_KEPT = 2, 72, 8
 
 
 def read_logits(path: str) -> np.ndarray:
@@ -43,9 +46,12 @@ def main() -> int:
             fh.write(blob)
         subprocess.check_call([exe, "reference", model, out, str(REQUESTS), str(STEPS)])
         logits = read_logits(out)
-    np.savez_compressed(os.path.join(HERE, "walker_tiny_llama.npz"), logits=logits,
+        subprocess.check_call([exe, "reference", model, out, str(LONG_REQUESTS), str(LONG_STEPS)])
+        long_logits = read_logits(out)[:, LONG_STEPS - LONG_KEPT:]
+    np.savez_compressed(os.path.join(HERE, "walker_tiny_llama.npz"), logits=logits, long_logits=long_logits,
                         gguf_sha256=np.array(hashlib.sha256(blob).hexdigest()))
-    print("wrote walker_tiny_llama.npz", logits.shape, "model sha256", hashlib.sha256(blob).hexdigest())
+    print("wrote walker_tiny_llama.npz", logits.shape, long_logits.shape, "model sha256",
+          hashlib.sha256(blob).hexdigest())
     return 0
 
 

@@ -36,13 +36,13 @@ def model(tmp_path_factory):
                     "(another numpy random stream?): run tests/golden/make_walker_golden.py")
     path = tmp_path_factory.mktemp("walker") / "tiny.gguf"
     path.write_bytes(blob)
-    return str(path), golden["logits"]
+    return str(path), golden["logits"], golden["long_logits"]
 
 
 @pytest.mark.parametrize("requests", [1, 2, 4])
 def test_walker_logits_match_the_single_stream_cpu_runner(model, requests, tmp_path):
     from make_walker_golden import STEPS, read_logits
-    path, want = model
+    path, want, _ = model
     if not os.path.exists(PROGRAM):
         pytest.fail(f"{PROGRAM} is not built (make -C tests/integration, needs the reference checkout)")
     out = str(tmp_path / "logits.bin")
@@ -55,6 +55,32 @@ def test_walker_logits_match_the_single_stream_cpu_runner(model, requests, tmp_p
     worst = 1.0
     for r in range(requests):
         for i in range(STEPS):
+            a, b = got[r, i].astype(np.float64), want[r, i].astype(np.float64)
+            cos = float(a @ b / np.sqrt((a @ a) * (b @ b)))
+            worst = min(worst, cos)
+            assert cos >= 0.999, (r, i, cos)
+            assert int(np.argmax(a)) == int(np.argmax(b)), (r, i)
+    print(f"[walker] worst cosine {worst:.7f}", flush=True)
+
+
+def test_walker_across_a_page_boundary(model, tmp_path):
+    """72 steps per request: the reference's PagePool hands every request a second 64-token page on
+    the way, the KV writes and the paged attention go on across it; the last steps' logits against the
+    single-stream CPU runner's."""
+    from make_walker_golden import LONG_KEPT, LONG_REQUESTS, LONG_STEPS, read_logits
+    path, _, want = model
+    if not os.path.exists(PROGRAM):
+        pytest.fail(f"{PROGRAM} is not built (make -C tests/integration, needs the reference checkout)")
+    out = str(tmp_path / "logits_long.bin")
+    print(f"[walker] {LONG_REQUESTS} requests x {LONG_STEPS} steps", flush=True)
+    proc = subprocess.run([PROGRAM, "walker", path, out, str(LONG_REQUESTS), str(LONG_STEPS)], stdout=subprocess.PIPE,
+                          stderr=subprocess.STDOUT, text=True, timeout=110)
+    assert proc.returncode == 0, proc.stdout
+    got = read_logits(out)[:, LONG_STEPS - LONG_KEPT:]
+    assert got.shape == want.shape
+    worst = 1.0
+    for r in range(LONG_REQUESTS):
+        for i in range(LONG_KEPT):
             a, b = got[r, i].astype(np.float64), want[r, i].astype(np.float64)
             cos = float(a @ b / np.sqrt((a @ a) * (b @ b)))
             worst = min(worst, cos)
