@@ -859,7 +859,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
     // values a lane keeps (v_permlane32_swap / v_permlane16_swap hand the other half to the
     // partner, the last step of head_dim 64 goes over lane ^ 8).  Lane (r, c) ends up with
     // dims c*8 + r*HPK + kk (kk < HPK) of every head, summed over all tokens of the wave.
-    auto reduce_rows = [&](float (&o_un)[OPL], float (&m_all)[HPW], float (&l_all)[HPW]) {
+    auto reduce_rows = [&](float (&o_un)[OPL], float (&m_all)[HPW], float (&l_all)[HPW], bool last_of_range) {
         if constexpr (MF) {
             // every wave leaves its (o, m, l) of all heads of the group in LDS; wave hg then
             // combines the four for its own heads, in the lane layout the code below expects
@@ -902,8 +902,9 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
 #pragma unroll
                 for (int kk = 0; kk < HPK; ++kk) o_un[h * HPK + kk] = o[kk];
             }
-            sd_barrier();   // the waves run on their own between pairs: nobody writes the next pair's
-                            // figures before everybody has read these
+            // the waves run on their own between pairs: nobody writes the next pair's figures before
+            // everybody has read these (at the range's end nobody writes them again)
+            if (!last_of_range) sd_barrier();
             return;
         }
 #pragma unroll
@@ -1171,7 +1172,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         if (range_done) MLC_PROBE(4);
         if (pair_done || range_done) {
             float o_un[OPL], m_all[HPW], l_all[HPW];
-            reduce_rows(o_un, m_all, l_all);
+            reduce_rows(o_un, m_all, l_all, range_done);
             const uint32_t ps = req_start(cc.r) * Hkv + cc.kvh * cc.tiles;  // pair's first tile
             const bool starts_here = seg_first == ps;                 // no workgroup before this one has tiles of the pair
             const bool ends_here = g0 + k + 1u == ps + cc.tiles;      // ... none behind it
