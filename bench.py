@@ -426,10 +426,12 @@ def finish_step(args, steps, exe, L, loop, lc, c, w, x, cos, sin, page_ids, slot
     return result
 
 
-def build_workload(name: str):
+def build_workload(name: str, batch=None):
+    """The benchmark configuration `name`; batch: another batch size of the same shape and length
+    distribution (cfg2 - cfg4; an experiment, not a benchmark configuration)."""
     from mlcompiler_amd.workloads import baseline_config
     idx = {"cfg1": 1, "cfg2": 2, "cfg3": 3, "cfg4": 4}[name]
-    case = baseline_config(idx)
+    case = baseline_config(idx, batch=batch) if batch and idx > 1 else baseline_config(idx)
     layers = {"cfg1": 22, "cfg2": 22, "cfg3": 8, "cfg4": 1}[name]
     return case, layers
 
@@ -571,7 +573,7 @@ def run_decode(args, name: str, steps: int, warmup: int, cpu_budget: float, full
     from mlcompiler_amd import HipExecutor
     from mlcompiler_amd.build import BENCH_LIB_PATH
     exe = HipExecutor.Instance()
-    case, n_layers = build_workload(name)
+    case, n_layers = build_workload(name, getattr(args, "batch", 0) if name == args.workload else None)
     c = case
     pool_bytes = c.k_pages.nbytes
     q_buf = exe.allocateScratchBuffer(c.q.nbytes)
@@ -891,6 +893,9 @@ def main() -> int:
     ap.add_argument("--per-config", type=int, default=-1,
                     help="1: add config.per_config (configurations 1, 3, 4 and 5, each with its own bounded CPU "
                          "baseline) to the line; default: only for the default workload")
+    ap.add_argument("--batch", type=int, default=0,
+                    help="cfg2 - cfg4: another batch size of the same shape (an experiment; the line then is not "
+                         "the benchmark configuration's)")
     ap.add_argument("--copy-mib", type=int, default=32, help="size of the calibration copy")
     ap.add_argument("--cpu-budget", type=float, default=15.0, help="seconds of CPU baseline work")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")

@@ -103,7 +103,8 @@ def baseline_config(idx: int, *, batch=None, seed=1234) -> DecodeCase:
     if idx == 2:
         b = batch or 32
         sl = rng.integers(128, 2049, size=b)
-        return make_case("cfg2_tinyllama_b32", b, 32, 4, 64, 64, sl, capacity_pages=1024, seed=seed)
+        cap = 1024 if b == 32 else int(((sl + 63) // 64).sum()) + 64
+        return make_case(f"cfg2_tinyllama_b{b}", b, 32, 4, 64, 64, sl, capacity_pages=cap, seed=seed)
     if idx == 3:
         b = batch or 64
         sl = rng.integers(256, 4097, size=b)
