@@ -771,7 +771,8 @@ def stream_read_sweep(bl, kp, vp, n_layers: int, each: int, n_cu: int, launches:
     """The practical ceiling of the memory system for a launch that reads `each` bytes of a K pool and
     of a V pool and does nothing else: the streaming-read kernels of csrc/bench_loop.cpp (loads into
     registers with 1..8 independent 16-byte loads per tensor in flight per lane, and global -> LDS
-    loads shaped like the decode kernel's tile loads) swept over 1, 2, 4 and 8 workgroups per CU,
+    loads shaped like the decode kernel's tile loads, each with ordinary and with non-temporal
+    loads) swept over 1, 2, 4 and 8 workgroups per CU,
     each timed like the decode loop (same pools, rotated, HIP events around `launches` launches).
     Reports the best average, the best block of a repeat run of that combination, and the untuned
     grid-stride kernel."""
@@ -787,15 +788,16 @@ def stream_read_sweep(bl, kp, vp, n_layers: int, each: int, n_cu: int, launches:
     assert bl.mlc_bench_read_loop(kp, vp, C.c_size_t(n_layers), C.c_size_t(each), C.c_size_t(launches), C.byref(ms))
     plain_us = ms.value / launches * 1e3
     rows = []
-    for kind, unrolls in ((0, (1, 2, 4, 8)), (1, (1, 2, 4))):
+    names = {0: "registers", 1: "global->LDS", 2: "registers, non-temporal", 3: "global->LDS, non-temporal"}
+    for kind, unrolls in ((0, (1, 2, 4, 8)), (1, (1, 2, 4)), (2, (1, 2, 4, 8)), (3, (1, 2, 4))):
         for u in unrolls:
             for per_cu in (1, 2, 4, 8):
-                if kind == 1 and per_cu * 2 * 2 * u * 4096 > 160 * 1024:
+                if kind % 2 == 1 and per_cu * 2 * 2 * u * 4096 > 160 * 1024:
                     continue   # the LDS stages of that many workgroups do not fit a CU
                 grid = n_cu * per_cu
                 if tuned(kind, u, grid, n_layers) is None:
                     continue
-                rows.append({"kind": "registers" if kind == 0 else "global->LDS", "loads_in_flight_per_lane": 2 * u * (1 if kind == 0 else 2),
+                rows.append({"kind": names[kind], "loads_in_flight_per_lane": 2 * u * (1 if kind % 2 == 0 else 2),
                              "wgs_per_cu": per_cu, "us": round(tuned(kind, u, grid, launches), 3),
                              "_k": kind, "_u": u, "_g": grid})
     best = min(rows, key=lambda x: x["us"])

@@ -35,12 +35,25 @@ __global__ __launch_bounds__(256) void mlc_bench_read_kernel(const uint4* __rest
     if (acc == 0x9E3779B9u && sink) sink[0] = acc;
 }
 
+// 16-byte load, ordinary or non-temporal.
+template <bool NT>
+__device__ __forceinline__ uint4 load16(const uint4* p) {
+    if constexpr (NT) {
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+        return make_uint4(v[0], v[1], v[2], v[3]);
+    } else {
+        return *p;
+    }
+}
+
 // Tuned streaming read, into registers: a workgroup takes 256 * U consecutive 16-byte units of each
 // tensor per trip, so every lane has 2 * U independent 16-byte loads in flight before it folds
 // any of them (the plain kernel above has two).  The grid is persistent (a few workgroups per CU)
 // and swept by the caller.  This is the yardstick for what the memory system delivers to a launch
-// of a given size with nothing else to do.
-template <int U>
+// of a given size with nothing else to do.  NT: non-temporal loads (the data is read once: it need
+// not stay in the L2).
+template <int U, bool NT>
 __global__ __launch_bounds__(256) void mlc_bench_read_unrolled_kernel(const uint4* __restrict__ a,
                                                                       const uint4* __restrict__ b, size_t n_each,
                                                                       uint32_t* sink) {
@@ -50,9 +63,9 @@ __global__ __launch_bounds__(256) void mlc_bench_read_unrolled_kernel(const uint
     for (; i + (size_t)(U - 1) * 256 < n_each; i += stride) {
         uint4 x[U], y[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) x[u] = a[i + (size_t)u * 256];
+        for (int u = 0; u < U; ++u) x[u] = load16<NT>(&a[i + (size_t)u * 256]);
 #pragma unroll
-        for (int u = 0; u < U; ++u) y[u] = b[i + (size_t)u * 256];
+        for (int u = 0; u < U; ++u) y[u] = load16<NT>(&b[i + (size_t)u * 256]);
 #pragma unroll
         for (int u = 0; u < U; ++u) acc ^= x[u].x ^ x[u].y ^ x[u].z ^ x[u].w ^ y[u].x ^ y[u].y ^ y[u].z ^ y[u].w;
     }
@@ -70,7 +83,7 @@ __global__ __launch_bounds__(256) void mlc_bench_read_unrolled_kernel(const uint
 // moves 1 KiB per instruction straight into LDS (no registers), U instructions per tensor and
 // trip, two trips in flight (the next trip is requested before the current one is waited for).
 // Units past the end are clamped onto the last one (in bounds, read twice).
-template <int U>
+template <int U, bool NT>
 __global__ __launch_bounds__(256) void mlc_bench_read_lds_kernel(const uint4* __restrict__ a, const uint4* __restrict__ b,
                                                                  size_t n_each, uint32_t* sink) {
     __shared__ __attribute__((aligned(16))) unsigned char stage[2][2 * U * 4096];
@@ -87,7 +100,10 @@ __global__ __launch_bounds__(256) void mlc_bench_read_lds_kernel(const uint4* __
                 size_t j = i + (size_t)u * 256;
                 j = j < n_each ? j : n_each - 1;
                 const uint32_t dst = __builtin_amdgcn_readfirstlane(base + buf * (2 * U * 4096) + (t * U + u) * 4096 + wave * 1024);
-                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(dst), "v"(src + j) : "memory", "m0");
+                if constexpr (NT)
+                    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt" : : "s"(dst), "v"(src + j) : "memory", "m0");
+                else
+                    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(dst), "v"(src + j) : "memory", "m0");
             }
         }
     };
@@ -132,7 +148,8 @@ int mlc_bench_read_loop(void* const* k_pools, void* const* v_pools, size_t n_lay
     return 1;
 }
 
-// The tuned reads: kind 0 = into registers, 1 = global -> LDS; unroll = 16-byte loads per tensor
+// The tuned reads: kind 0 = into registers, 1 = global -> LDS, 2 and 3 = the same with non-temporal
+// loads; unroll = 16-byte loads per tensor
 // and trip (1, 2, 4 or 8); grid = workgroups of 256 threads.  Same rotation over the pools and the
 // same timing as mlc_bench_read_loop.  Returns 0 for a combination that is not built.
 int mlc_bench_read_tuned_loop(void* const* k_pools, void* const* v_pools, size_t n_layers, size_t bytes_each,
@@ -143,11 +160,17 @@ int mlc_bench_read_tuned_loop(void* const* k_pools, void* const* v_pools, size_t
     if (!n) return 0;
     void (*kern)(const uint4*, const uint4*, size_t, uint32_t*) = nullptr;
     if (kind == 0) {
-        kern = unroll == 1 ? mlc_bench_read_unrolled_kernel<1> : unroll == 2 ? mlc_bench_read_unrolled_kernel<2>
-             : unroll == 4 ? mlc_bench_read_unrolled_kernel<4> : unroll == 8 ? mlc_bench_read_unrolled_kernel<8> : nullptr;
+        kern = unroll == 1 ? mlc_bench_read_unrolled_kernel<1, false> : unroll == 2 ? mlc_bench_read_unrolled_kernel<2, false>
+             : unroll == 4 ? mlc_bench_read_unrolled_kernel<4, false> : unroll == 8 ? mlc_bench_read_unrolled_kernel<8, false> : nullptr;
     } else if (kind == 1) {
-        kern = unroll == 1 ? mlc_bench_read_lds_kernel<1> : unroll == 2 ? mlc_bench_read_lds_kernel<2>
-             : unroll == 4 ? mlc_bench_read_lds_kernel<4> : nullptr;
+        kern = unroll == 1 ? mlc_bench_read_lds_kernel<1, false> : unroll == 2 ? mlc_bench_read_lds_kernel<2, false>
+             : unroll == 4 ? mlc_bench_read_lds_kernel<4, false> : nullptr;
+    } else if (kind == 2) {
+        kern = unroll == 1 ? mlc_bench_read_unrolled_kernel<1, true> : unroll == 2 ? mlc_bench_read_unrolled_kernel<2, true>
+             : unroll == 4 ? mlc_bench_read_unrolled_kernel<4, true> : unroll == 8 ? mlc_bench_read_unrolled_kernel<8, true> : nullptr;
+    } else if (kind == 3) {
+        kern = unroll == 1 ? mlc_bench_read_lds_kernel<1, true> : unroll == 2 ? mlc_bench_read_lds_kernel<2, true>
+             : unroll == 4 ? mlc_bench_read_lds_kernel<4, true> : nullptr;
     }
     if (!kern) return 0;
     if (!mlc_hip_timer_start()) return 0;

@@ -114,7 +114,21 @@ inline size_t stream_dynamic_lds_bytes(size_t batch) { return (4 * batch + 2) * 
 // LDS reads of another stage nor needs one array per stage; the ordering is explicit instead
 // (sd_wait_vmcnt, sd_barrier).
 __device__ __forceinline__ void sd_g2lds16(const void* g, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+    // (non-temporal: a K/V byte is read once per launch and need not stay in the L2, where it only
+    // pushes out what is read again -- page tables, q, partials -- and costs the allocation: measured
+    // 13.43 -> 12.88 us, 30.4 -> 27.7 us and 204.6 -> 192.2 us at configurations 2, 3 and 4)
+#if defined(MLC_TILE_LOAD_PLAIN)   // (timing experiments: the ordinary load, other cache policies)
+#define MLC_TILE_LOAD_BITS ""
+#elif MLC_TILE_LOAD_MODE == 4
+#define MLC_TILE_LOAD_BITS " sc0 sc1 nt"
+#elif MLC_TILE_LOAD_MODE == 5
+#define MLC_TILE_LOAD_BITS " sc1 nt"
+#elif MLC_TILE_LOAD_MODE == 6
+#define MLC_TILE_LOAD_BITS " sc0 nt"
+#else
+#define MLC_TILE_LOAD_BITS " nt"
+#endif
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" MLC_TILE_LOAD_BITS
                  :
                  : "s"(lds_base), "v"(g)
                  : "memory", "m0");

@@ -202,6 +202,13 @@ __device__ __forceinline__ void q4_rope_epilogue(const RopeArgs& p, const Q4Rope
     if (pool) pool[(size_t)f.page_row * rows + local] = h;
 }
 
+// 8-byte non-temporal load (data that is read once and need not displace anything in the L2).
+__device__ __forceinline__ uint2 q4_stream_u2(const uint2* p) {
+    typedef uint32_t q4_u32x2 __attribute__((ext_vector_type(2)));
+    const q4_u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const q4_u32x2*>(p));
+    return make_uint2(v[0], v[1]);
+}
+
 // (0x6400 | n) is the half 1024 + n: two nibbles -> half2 (n0 - 8, n1 - 8), exactly.
 __device__ __forceinline__ q4_half2 q4_pair(uint32_t bytes, uint32_t sel) {
     const uint32_t m = __builtin_amdgcn_perm(0x64646464u, bytes, sel);
@@ -274,8 +281,9 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
 #pragma unroll
         for (int r = 0; r < RT; ++r) {
             const size_t tb = (size_t)(tile0 + r) * a.nblocks + blk;
-            k.q[r] = a.qs[tb * 64 + lane];
-            k.d[r] = a.d[tb * 32 + l32];
+            // (non-temporal: a weight is read once per launch and need not stay in the L2)
+            k.q[r] = q4_stream_u2(a.qs + tb * 64 + lane);
+            k.d[r] = __builtin_nontemporal_load(a.d + tb * 32 + l32);
         }
 #pragma unroll
         for (int t = 0; t < NBT; ++t)

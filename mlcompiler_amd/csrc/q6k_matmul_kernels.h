@@ -117,9 +117,10 @@ __global__ __launch_bounds__(512) void q6_k_matmul_mfma_kernel(const Q6KArgs a) 
         for (int r = 0; r < RT; ++r) {
             const size_t tg = (size_t)(tile0 + r) * groups + gi;
 #pragma unroll
-            for (int pc = 0; pc < 3; ++pc) k.p[r][pc] = a.qa[(tg * 3 + pc) * 64 + lane];
-            k.sc[r] = a.sc[tg * 32 + l32];
-            k.d[r] = a.d[((size_t)(tile0 + r) * a.nblocks + blk) * 32 + l32];
+            // (non-temporal: a weight is read once per launch and need not stay in the L2)
+            for (int pc = 0; pc < 3; ++pc) k.p[r][pc] = q4_stream_u2(a.qa + (tg * 3 + pc) * 64 + lane);
+            k.sc[r] = __builtin_nontemporal_load(a.sc + tg * 32 + l32);
+            k.d[r] = __builtin_nontemporal_load(a.d + ((size_t)(tile0 + r) * a.nblocks + blk) * 32 + l32);
         }
 #pragma unroll
         for (int t = 0; t < NBT; ++t)
