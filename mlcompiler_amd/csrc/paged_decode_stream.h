@@ -113,25 +113,30 @@ inline size_t stream_dynamic_lds_bytes(size_t batch) { return (4 * batch + 2) * 
 // compiler then does not know of the load, so it neither waits for all loads in flight before
 // LDS reads of another stage nor needs one array per stage; the ordering is explicit instead
 // (sd_wait_vmcnt, sd_barrier).
+// NT: non-temporal.  A K/V byte is read once per launch and need not stay in the L2, where it only
+// pushes out what is read again (page tables, q, partials) and costs the allocation: measured
+// 13.43 -> 12.88 us, 30.4 -> 27.7 us and 204.6 -> 192.2 us at configurations 2, 3 and 4 -- where one
+// instruction fetches whole cache lines, as the matrix-pipe mode's loads do.  The vector mode's loads
+// spread the 16-byte chunks of a row over eight instructions (the swizzle of its row groups), and
+// non-temporal loads then fetch most lines more than once (FETCH_SIZE 1.6 times the bytes and
+// 222 -> 521 us at configuration 4): it keeps the ordinary load.
+template <bool NT>
 __device__ __forceinline__ void sd_g2lds16(const void* g, uint32_t lds_base) {
-    // (non-temporal: a K/V byte is read once per launch and need not stay in the L2, where it only
-    // pushes out what is read again -- page tables, q, partials -- and costs the allocation: measured
-    // 13.43 -> 12.88 us, 30.4 -> 27.7 us and 204.6 -> 192.2 us at configurations 2, 3 and 4)
-#if defined(MLC_TILE_LOAD_PLAIN)   // (timing experiments: the ordinary load, other cache policies)
-#define MLC_TILE_LOAD_BITS ""
-#elif MLC_TILE_LOAD_MODE == 4
-#define MLC_TILE_LOAD_BITS " sc0 sc1 nt"
-#elif MLC_TILE_LOAD_MODE == 5
-#define MLC_TILE_LOAD_BITS " sc1 nt"
-#elif MLC_TILE_LOAD_MODE == 6
-#define MLC_TILE_LOAD_BITS " sc0 nt"
+#ifdef MLC_TILE_LOAD_PLAIN   // (timing experiments)
+    constexpr bool kNt = false;
 #else
-#define MLC_TILE_LOAD_BITS " nt"
+    constexpr bool kNt = NT;
 #endif
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" MLC_TILE_LOAD_BITS
-                 :
-                 : "s"(lds_base), "v"(g)
-                 : "memory", "m0");
+    if constexpr (kNt)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt"
+                     :
+                     : "s"(lds_base), "v"(g)
+                     : "memory", "m0");
+    else
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                     :
+                     : "s"(lds_base), "v"(g)
+                     : "memory", "m0");
 }
 __device__ __forceinline__ uint32_t sd_lds_addr(const void* p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
@@ -597,7 +602,7 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
                 }
                 tr = tr < last ? tr : last;
 #ifndef MLC_NO_LOADS
-                sd_g2lds16(src + (size_t)tr * row_u4, dst + j * 1024);
+                sd_g2lds16<MF>(src + (size_t)tr * row_u4, dst + j * 1024);
 #else
                 asm volatile("" ::"v"(src + (size_t)tr * row_u4), "s"(dst + j * 1024));
 #endif
