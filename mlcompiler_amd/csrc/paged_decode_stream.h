@@ -694,6 +694,20 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
                     pb[i] = (_Float16)pf;
                     pl[i] = (_Float16)(pf - (float)pb[i]);
                 }
+                if constexpr (TW == 8) {
+                    // A wave has 8 tokens of the tile, the product sums over 16: the upper 8 places
+                    // (lanes 32 .. 63, whose own weights are masked to zero and whose V^T operand
+                    // repeats the rows of the lower ones, see mf_v_off) take the low parts of the 8
+                    // weights, so that hi and lo go through one instruction per V block.
+                    const uint2 lw = __builtin_bit_cast(uint2, pl);
+                    const auto s0 = __builtin_amdgcn_permlane32_swap(lw.x, lw.x, false, false);
+                    const auto s1 = __builtin_amdgcn_permlane32_swap(lw.y, lw.y, false, false);
+                    const sd_half4 up = __builtin_bit_cast(sd_half4, make_uint2(s0[0], s1[0]));
+                    const sd_half4 pboth = g4 < 2 ? pb : up;
+#pragma unroll
+                    for (int b = 0; b < DB; ++b) mf_o[b] = __builtin_amdgcn_mfma_f32_16x16x16f16(va[b], pboth, mf_o[b], 0, 0, 0);
+                    return;
+                }
 #pragma unroll
                 for (int b = 0; b < DB; ++b) {
                     mf_o[b] = __builtin_amdgcn_mfma_f32_16x16x16f16(va[b], pb, mf_o[b], 0, 0, 0);
