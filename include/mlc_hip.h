@@ -347,6 +347,11 @@ long mlc_hip_fused_kv_write_launches(void);
 /* Number of Q4_0 matmuls so far that went out with the split + RoPE + cast (and KV write) of
  * their output as epilogue (for tests). */
 long mlc_hip_fused_matmul_rope_launches(void);
+/* Number of Q4_0 matmuls so far that went out with the gate/up split + SiLU * up of their output
+ * as epilogue, and how many of those also wrote the activation fragments of the Q4_0 matmul
+ * that reads the products (for tests). */
+long mlc_hip_fused_matmul_silu_launches(void);
+long mlc_hip_fused_matmul_silu_split_launches(void);
 /* Number of decode attention launches so far that carried the step's KV write (a pair of
  * batched K / V scatters of every request's newest position encoded just before it). */
 long mlc_hip_kv_writes_in_decode_launches(void);

@@ -170,6 +170,10 @@ struct Ctx {
     // A Q4_0 matmul of the open pass whose launch is held back for one call: when that call is
     // the split + RoPE + cast of the matmul's output (the qkv projection of a layer), the
     // matmul's epilogue does it and the two -- with the KV scatters that join -- are one launch.
+    // When that call is the gate/up split + SiLU * up of the matmul's output (the gate/up
+    // projection), the epilogue does that instead and the matmul is held back for one call more:
+    // a Q4_0 matmul that reads the products (the down-projection) lets the epilogue also write
+    // its activation fragments.
     struct GemmPending {
         bool active = false;
         Q4Args a{};
@@ -177,8 +181,14 @@ struct Ctx {
         int nbt = 1, rt = 1;
         const void* out = nullptr;
         size_t batch = 0, rows = 0;
+        bool block_scales = false;       // the activations carry one scale per (request, block)
+        bool silu = false;               // the gate/up split + SiLU * up has joined
+        const void* silu_out = nullptr;
+        size_t ffn_inner = 0;
     } gemm;
     long gemm_rope_fused = 0;        // matmuls launched with the RoPE epilogue (for tests)
+    long gemm_silu_fused = 0;        // ... with the gate/up split + SiLU * up as epilogue
+    long gemm_silu_split_fused = 0;  // ... of which also wrote the next matmul's activation fragments
     long kv_fused = 0;               // KV writes that went out fused with a neighbour (for tests)
     long kv_in_decode = 0;           // ... of which inside the attention launch
     long opt_fuse_rows = 1;          // 0 = every operator is launched when it is encoded
@@ -394,6 +404,28 @@ void launch_q4_mfma(int nbt, int rt, dim3 grid, const Q4Args& a) {
 #undef MLC_Q4
 }
 
+// The same with activations that were split with one scale per (request, block): a.blk_exp.
+// Integer-operand arithmetic only.
+void launch_q4_mfma_block_scales(int nbt, int rt, dim3 grid, const Q4Args& a) {
+#define MLC_Q4(NBT, RT, WAVES) \
+    hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<NBT, RT, WAVES, true, true>), grid, dim3(WAVES * 64), 0, g.stream, a)
+    if (nbt == 1) {
+        if (rt == 1) { MLC_Q4(1, 1, 16); } else { MLC_Q4(1, 2, 16); }
+    } else {
+        if (rt == 1) { MLC_Q4(2, 1, 8); } else { MLC_Q4(2, 2, 8); }
+    }
+#undef MLC_Q4
+}
+
+// The gate/up projection with the gate/up split + SiLU * up (and, when a.split_frag is set, the
+// split of the products for the matmul that reads them) as epilogue: two row tiles per workgroup.
+void launch_q4_mfma_silu(int nbt, dim3 grid, const Q4Args& a) {
+    if (nbt == 1)
+        hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<1, 2, 16, true, false, true>), grid, dim3(16 * 64), 0, g.stream, a);
+    else
+        hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<2, 2, 8, true, false, true>), grid, dim3(8 * 64), 0, g.stream, a);
+}
+
 // Launches the held-back matmul, with the split + RoPE + cast of its output as epilogue when
 // `rope` is given.
 int settle_gemm(const RopeArgs* rope = nullptr) {
@@ -407,7 +439,18 @@ int settle_gemm(const RopeArgs* rope = nullptr) {
         ++g.gemm_rope_fused;
     }
     const dim3 grid(m.grid_x, 1);
-    launch_q4_mfma(m.nbt, m.rt, grid, a);
+    if (m.silu) {
+        m.silu = false;
+        ++g.gemm_silu_fused;
+        if (a.split_frag) ++g.gemm_silu_split_fused;
+        launch_q4_mfma_silu(m.nbt, grid, a);
+        HIP_OK(hipGetLastError());
+        return 1;
+    }
+    if (m.block_scales)
+        launch_q4_mfma_block_scales(m.nbt, m.rt, grid, a);
+    else
+        launch_q4_mfma(m.nbt, m.rt, grid, a);
     HIP_OK(hipGetLastError());
     return 1;
 }
@@ -416,7 +459,7 @@ int settle_gemm(const RopeArgs* rope = nullptr) {
 // call describes, so that the matmul's epilogue can do that call's work.
 bool gemm_feeds_rope(const void* qkv, size_t batch, size_t qkv_rows, size_t q_rows, size_t k_rows, size_t v_rows) {
     const Ctx::GemmPending& m = g.gemm;
-    return g.opt_fuse_rows && m.active && !g.kv.active && !g.rows.active && m.out == qkv && m.batch == batch &&
+    return g.opt_fuse_rows && m.active && !m.silu && !g.kv.active && !g.rows.active && m.out == qkv && m.batch == batch &&
            m.rows == qkv_rows && q_rows + k_rows + v_rows == qkv_rows;
 }
 

@@ -71,7 +71,13 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
     // replace a buffer the chain still refers to)
     const bool feeds = batch <= 64 && !g.opt_q4_force_generic && !(reinterpret_cast<uintptr_t>(out) & 15u) &&
                        q4_fast_shape(rows, cols, row_stride) && row_len_ok(cols) && rows_continue(in, batch, cols);
-    if (!feeds && !settle()) return 0;
+    // ... or is the input the SiLU * up product that the held-back gate/up projection's epilogue
+    // will write?  Then that epilogue also splits it, per (request, block of 32 columns).
+    const bool feeds_silu = !feeds && batch <= 64 && g.opt_fuse_rows && g.opt_q4_int_operand && !g.opt_q4_force_generic &&
+                            !(reinterpret_cast<uintptr_t>(out) & 15u) && q4_fast_shape(rows, cols, row_stride) &&
+                            g.gemm.active && g.gemm.silu && !g.rows.active && !g.kv.active && g.gemm.silu_out == in &&
+                            g.gemm.batch == batch && g.gemm.ffn_inner == cols;
+    if (!feeds && !feeds_silu && !settle()) return 0;
     Ctx::Q4Weight* w = q4_weight(weight_name, static_cast<const uint8_t*>(weights), weight_bytes, rows, cols, row_stride);
     if (!w) return 0;
 
@@ -101,12 +107,18 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
     for (size_t bo = 0; bo < batch; bo += 64) {
         const size_t bn = std::min<size_t>(64, batch - bo);
         const size_t bpad = (bn + 31) / 32 * 32;
-        _Float16* frag = static_cast<_Float16*>(cached_buffer("q4_x_fragments", bpad * cols * 4));
+        // (the held-back projection still reads "q4_x_fragments": its products go to a buffer of their own)
+        _Float16* frag = static_cast<_Float16*>(cached_buffer(feeds_silu ? "q4_x_fragments_silu" : "q4_x_fragments", bpad * cols * 4));
         float* inv = static_cast<float*>(cached_buffer("q4_x_inv_scale", 64 * 4));
-        if (!frag || !inv) return fail("q4 matmul: scratch allocation failed");
+        int8_t* blk_exp = feeds_silu ? static_cast<int8_t*>(cached_buffer("q4_x_block_exponents", bpad * nblocks)) : nullptr;
+        if (!frag || !inv || (feeds_silu && !blk_exp)) return fail("q4 matmul: scratch allocation failed");
         const float* xin = static_cast<const float*>(in) + bo * cols;
         float* o = static_cast<float*>(out) + bo * rows;
-        if (feeds) {  // the chain that produces the input also splits it (batch <= 64: one round)
+        if (feeds_silu) {
+            g.gemm.a.split_frag = frag;
+            g.gemm.a.split_blk_exp = blk_exp;
+            if (!settle()) return 0;
+        } else if (feeds) {  // the chain that produces the input also splits it (batch <= 64: one round)
             g.rows.p.frag = frag;
             g.rows.p.inv_scale = inv;
             g.rows.grid_rows = bpad;
@@ -118,8 +130,9 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
         // (the chain has been launched: its K-slice source may be replaced now)
         float* slices = ksplit > 1 ? static_cast<float*>(cached_buffer("q4_k_slices", ksplit * bn * rows * 4)) : nullptr;
         if (ksplit > 1 && !slices) return fail("q4 matmul: scratch allocation failed");
-        Q4Args a;
+        Q4Args a{};
         a.qs = static_cast<const uint2*>(w->qs);
+        a.blk_exp = blk_exp;
         a.d = static_cast<const _Float16*>(w->d);
         a.xfrag = frag;
         a.inv_scale = inv;
@@ -132,6 +145,8 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
             // held back for one call: a split + RoPE + cast of this output becomes the epilogue
             Ctx::GemmPending& m = g.gemm;
             m.active = true;
+            m.silu = false;
+            m.block_scales = feeds_silu;
             m.a = a;
             m.grid_x = (unsigned)wgs;
             m.nbt = bpad == 32 ? 1 : 2;
@@ -142,7 +157,10 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
             return finish(sync);
         }
         const dim3 grid((unsigned)wgs, (unsigned)ksplit);
-        launch_q4_mfma(bpad == 32 ? 1 : 2, row_tiles, grid, a);
+        if (feeds_silu)
+            launch_q4_mfma_block_scales(bpad == 32 ? 1 : 2, row_tiles, grid, a);
+        else
+            launch_q4_mfma(bpad == 32 ? 1 : 2, row_tiles, grid, a);
         if (ksplit > 1) {
             const uint32_t n = (uint32_t)(bn * rows);
             if (g.opt_fuse_rows && batch <= 64 && rows <= 2 * kRowMaxLen) {

@@ -108,6 +108,24 @@ int mlc_hip_gate_up_split_silu_mul(const void* gate_up, void* gate, void* up, vo
     const size_t kg = known_bytes(gate_up);
     if (kg && batch * ffn_gate_up_rows * 4 > kg) return fail("gate/up split: gate_up buffer too small");
     {
+        // The gate/up projection itself is still held back: the operator becomes its epilogue
+        // (workgroup j takes row tile j of the gate half and row tile j of the up half).
+        Ctx::GemmPending& m = g.gemm;
+        if (g.opt_fuse_rows && g.opt_q4_int_operand && !sync && m.active && !m.silu && !g.rows.active && !g.kv.active &&
+            m.rt == 2 && m.out == gate_up && m.batch == batch && m.rows == ffn_gate_up_rows &&
+            ffn_gate_up_rows == 2 * ffn_inner && ffn_inner % 32 == 0 && aligned16(gate) && aligned16(up) && aligned16(out)) {
+            m.silu = true;
+            m.silu_out = out;
+            m.ffn_inner = ffn_inner;
+            m.a.tile_stride = (uint32_t)(ffn_inner / 32);
+            m.a.ffn_inner = (uint32_t)ffn_inner;
+            m.a.gate = static_cast<float*>(gate);
+            m.a.up = static_cast<float*>(up);
+            m.a.silu_out = static_cast<float*>(out);
+            m.a.split_frag = nullptr;
+            m.a.split_blk_exp = nullptr;
+            return finish(sync);
+        }
         Ctx::RowPending& r = g.rows;
         const bool joins = ffn_gate_up_rows == 2 * ffn_inner && row_len_ok(ffn_inner) && aligned16(gate) &&
                            aligned16(up) && aligned16(out) && !r.p.silu && !r.p.addend && !r.p.rms &&

@@ -146,6 +146,26 @@ struct Q4Args {
     // request): the epilogue also does what qkv_split_rope_cast_kernel would do with that row.
     uint32_t rope_on;
     RopeArgs rope;
+    // Kernels built with BS: the activations were split with one power-of-two scale per (request,
+    // block of 32 columns) instead of one per request: x = (hi + lo) * 2^e.  blk_exp holds the
+    // exponents e as [batch tile of 32][nblocks][32 bytes], request c of the tile at byte
+    // ((c % 8) / 4) * 16 + (c / 8) * 4 + c % 4 -- the order in which a lane's 16 accumulator
+    // registers hold the requests, so that one 16-byte load per block brings a lane's 16 exponents;
+    // inv_scale is not read.
+    const int8_t* blk_exp;
+    // Kernels built with SILU (two row tiles per workgroup, ksplit == 1, rows = 2 * ffn_inner): the
+    // output is a fused gate/up row; workgroup j takes tile j of the gate half and tile j of the up
+    // half (tile_stride = ffn_inner / 32 apart) and its epilogue also does the gate/up split and
+    // SiLU(gate) * up of those 32 columns -> gate, up, silu_out ([batch][ffn_inner] each).  With
+    // split_frag set it goes on to split the 32 products of every request into the B-operand
+    // fragments of the matmul that consumes them (K = ffn_inner), scaled per (request, block):
+    // block j of that matmul is exactly this workgroup's 32 columns.
+    uint32_t tile_stride, ffn_inner;
+    float* gate;
+    float* up;
+    float* silu_out;
+    _Float16* split_frag;
+    int8_t* split_blk_exp;
 };
 
 // The split + RoPE + cast (+ paged write) of one element of a request's fused qkv row, by the
@@ -231,15 +251,23 @@ __device__ __forceinline__ q4_half2 q4_pair(uint32_t bytes, uint32_t sel) {
 // is one number per lane) and the activations the A operand; both fragment layouts serve either
 // role unchanged.  No product is rounded and no term is dropped: what remains is the fp32
 // rounding of the additions and of one multiply per block.
-template <int NBT, int RT, int WAVES, bool IOP>
+__device__ __forceinline__ float q4_silu_times(float g, float u) {  // walker_kernels.h: silu_times
+    const float silu = g / (1.0f + expf(-g));
+    return silu * u;
+}
+
+template <int NBT, int RT, int WAVES, bool IOP, bool BS = false, bool SILU = false>
 __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Args a) {
+    static_assert(!BS || IOP, "per-block activation scales: integer-operand arithmetic only");
+    static_assert(!SILU || (IOP && RT == 2), "SiLU epilogue: gate tile and up tile, integer-operand arithmetic");
     constexpr int PF = WAVES >= 16 ? 2 : 4;  // blocks in flight per wave
     constexpr int PITCH = 65;                // floats per accumulator register in LDS (bank spread)
     __shared__ float red[WAVES * RT * NBT * 16 * PITCH];
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const uint32_t lane = threadIdx.x % 64;
     const uint32_t l32 = lane % 32;
-    const uint32_t tile0 = blockIdx.x * RT;
+    const uint32_t tile0 = SILU ? blockIdx.x : blockIdx.x * RT;
+    const uint32_t tile_step = SILU ? a.tile_stride : 1u;   // row tile r of the workgroup: tile0 + r * tile_step
     const uint32_t slice = blockIdx.y;
     const uint32_t b0 = slice * a.blocks_per_slice;
     const uint32_t b1 = min(b0 + a.blocks_per_slice, a.nblocks);
@@ -270,6 +298,7 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
         uint2 q[RT];
         _Float16 d[RT];
         q4_half8 x[NBT][2][2];  // [batch tile][k step][hi, lo]
+        uint4 ex[BS ? NBT : 1];   // BS: scale exponents of the 16 batch columns in this lane's registers, a byte each
         bool real;               // false: a repeat past the end of the slice, multiplied with scale 0
     };
     auto load = [&](uint32_t blk_raw, Block& k) __attribute__((always_inline)) {
@@ -280,7 +309,7 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
         k.real = blk_raw < b1;
 #pragma unroll
         for (int r = 0; r < RT; ++r) {
-            const size_t tb = (size_t)(tile0 + r) * a.nblocks + blk;
+            const size_t tb = (size_t)(tile0 + r * tile_step) * a.nblocks + blk;
             // (non-temporal: a weight is read once per launch and need not stay in the L2)
             k.q[r] = q4_stream_u2(a.qs + tb * 64 + lane);
             k.d[r] = __builtin_nontemporal_load(a.d + tb * 32 + l32);
@@ -293,11 +322,20 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
                 for (int p = 0; p < 2; ++p)
                     k.x[t][ks][p] = *reinterpret_cast<const q4_half8*>(
                         a.xfrag + ((((size_t)t * ksteps + blk * 2 + ks) * 2 + p) * 64 + lane) * 8);
+        if constexpr (BS) {
+            // register i of the accumulator is batch column (i/4)*8 + (lane/32)*4 + i%4
+#pragma unroll
+            for (int t = 0; t < NBT; ++t)
+                k.ex[t] = *reinterpret_cast<const uint4*>(a.blk_exp + ((size_t)t * a.nblocks + blk) * 32 + (lane / 32) * 16);
+        }
     };
     auto multiply = [&](const Block& k) __attribute__((always_inline)) {
         if constexpr (IOP) {
 #pragma unroll
             for (int r = 0; r < RT; ++r) {
+                // (SILU: one row tile's products after the other, or the scheduler keeps three
+                // sets of 16 in flight and the loop no longer fits the 128 registers a wave has)
+                if constexpr (SILU) { if (r) __builtin_amdgcn_sched_barrier(0); }
                 const float d = k.real ? (float)k.d[r] : 0.0f;
                 q4_half8 w[2];
 #pragma unroll
@@ -318,8 +356,20 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
                         sblk = __builtin_amdgcn_mfma_f32_32x32x16_f16(k.x[t][ks][0], w[ks], sblk, 0, 0, 0);
                         sblk = __builtin_amdgcn_mfma_f32_32x32x16_f16(k.x[t][ks][1], w[ks], sblk, 0, 0, 0);
                     }
+                    if constexpr (BS) {
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) acc[r][t][i] = fmaf(d, sblk[i], acc[r][t][i]);
+                        for (int j = 0; j < 4; ++j) {
+                            const uint32_t e4 = j == 0 ? k.ex[t].x : j == 1 ? k.ex[t].y : j == 2 ? k.ex[t].z : k.ex[t].w;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const int ex = (int)(e4 << (24 - 8 * e)) >> 24;   // signed byte e
+                                acc[r][t][j * 4 + e] = fmaf(__builtin_ldexpf(d, ex), sblk[j * 4 + e], acc[r][t][j * 4 + e]);
+                            }
+                        }
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) acc[r][t][i] = fmaf(d, sblk[i], acc[r][t][i]);
+                    }
                 }
             }
             return;
@@ -382,6 +432,60 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
             for (int i = 0; i < 16; ++i)
                 red[(((wave * RT + r) * NBT + t) * 16 + i) * PITCH + lane] = acc[r][t][i];
     __syncthreads();
+    if constexpr (SILU) {
+        // thread -> (column rr of the workgroup's 32 ffn columns, request b); the 32 lanes of a half
+        // wave hold one request's 32 columns, which are one block of the consuming matmul's K
+        constexpr uint32_t B_PER_PASS = WAVES * 2, S_PASSES = 32 * NBT / B_PER_PASS;
+        const uint32_t rr = threadIdx.x % 32, bs = threadIdx.x / 32;
+        const uint32_t col = tile0 * 32 + rr;            // column of gate / up / silu_out
+        const uint32_t nblk_out = a.ffn_inner / 32, ksteps_out = a.ffn_inner / 16;
+#pragma unroll
+        for (uint32_t pass = 0; pass < S_PASSES; ++pass) {
+            const uint32_t b = pass * B_PER_PASS + bs;
+            const bool live = b < a.batch;
+            const uint32_t t = b / 32, in_reg = b % 32;
+            const uint32_t i = (in_reg / 8) * 4 + in_reg % 4, ln = ((in_reg % 8) / 4) * 32 + rr;
+            float sg = 0.f, su = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) {
+                sg += red[(((w * RT + 0) * NBT + t) * 16 + i) * PITCH + ln];
+                su += red[(((w * RT + 1) * NBT + t) * 16 + i) * PITCH + ln];
+            }
+            float prod = 0.f;
+            if (live) {
+                const float inv = a.inv_scale[b];
+                const float gv = sg * inv, uv = su * inv;
+                prod = q4_silu_times(gv, uv);
+                a.out[(size_t)b * a.rows + col] = gv;
+                a.out[(size_t)b * a.rows + a.ffn_inner + col] = uv;
+                a.gate[(size_t)b * a.ffn_inner + col] = gv;
+                a.up[(size_t)b * a.ffn_inner + col] = uv;
+                a.silu_out[(size_t)b * a.ffn_inner + col] = prod;
+            }
+            if (a.split_frag) {   // (uniform; requests past the batch are written as zeros)
+                float amax = fabsf(prod);
+#pragma unroll
+                for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+                int e = 0;
+                if (amax > 0.f && amax < INFINITY) (void)frexpf(amax, &e);
+                int se = 14 - e;
+                se = se > 100 ? 100 : (se < -100 ? -100 : se);
+                const float tv = prod * ldexpf(1.0f, se);
+                const _Float16 hi = (_Float16)tv;
+                const _Float16 lo = (_Float16)(tv - (float)hi);
+                const uint32_t k = col;
+                const size_t base = ((size_t)t * ksteps_out + k / 16) * 2;
+                const uint32_t fl = ((k % 16) / 8) * 32 + b % 32;
+                a.split_frag[((base + 0) * 64 + fl) * 8 + k % 8] = hi;
+                a.split_frag[((base + 1) * 64 + fl) * 8 + k % 8] = lo;
+                if (rr == 0) {
+                    const uint32_t c = b % 32;
+                    a.split_blk_exp[((size_t)t * nblk_out + tile0) * 32 + ((c % 8) / 4) * 16 + (c / 8) * 4 + c % 4] = (int8_t)(-se);
+                }
+            }
+        }
+        return;
+    }
     const uint32_t r = row / 32, rr = row % 32;
     float* out = a.out + (size_t)slice * a.batch * a.rows;
 #pragma unroll
@@ -394,7 +498,7 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
         float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) sum += red[(((w * RT + r) * NBT + t) * 16 + i) * PITCH + ln];
-        const float val = sum * a.inv_scale[b];
+        const float val = BS ? sum : sum * a.inv_scale[b];
         out[(size_t)b * a.rows + tile0 * 32 + row] = val;
         if (a.rope_on)  // (the lanes of a pair share b)
             q4_rope_epilogue(a.rope, ROPE_AHEAD ? rope_pre[ROPE_AHEAD ? pass : 0] : q4_rope_prefetch(a.rope, b, tile0 * 32 + row),

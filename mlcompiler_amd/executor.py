@@ -296,6 +296,14 @@ class HipExecutor:
         """Q4_0 matmuls so far launched with the split + RoPE + cast of their output as epilogue."""
         return int(self._lib.mlc_hip_fused_matmul_rope_launches())
 
+    def fusedMatmulSiluLaunches(self) -> int:
+        """Q4_0 matmuls so far launched with the gate/up split + SiLU * up of their output as epilogue."""
+        return int(self._lib.mlc_hip_fused_matmul_silu_launches())
+
+    def fusedMatmulSiluSplitLaunches(self) -> int:
+        """... of which also wrote the activation fragments of the matmul that reads the products."""
+        return int(self._lib.mlc_hip_fused_matmul_silu_split_launches())
+
     def rowProgramLaunches(self) -> int:
         """Fused row-operator launches so far (option "fuse_row_ops")."""
         return int(self._lib.mlc_hip_row_program_launches())
