@@ -186,6 +186,22 @@ struct Ctx {
         const void* silu_out = nullptr;
         size_t ffn_inner = 0;
     } gemm;
+    // The tile-balanced decode attention launch of the open pass, held back for one call: when that
+    // call is a Q4_0 matmul that reads the attention's output (the out-projection), the kernel
+    // that writes a row of the output also writes it as that matmul's split-fp16 activations, one
+    // scale exponent per (request, block of 32 columns), and the split kernel's launch goes away.
+    // Everything about the call (tables, tags, the KV write it carries) was settled when it was
+    // encoded; only the launch waits.
+    struct DecodePending {
+        bool active = false;
+        StreamArgs a{};
+        size_t head_dim = 0, dyn_lds = 0;
+        int hpw = 0, nw = 0, nbuf = 0;
+        unsigned n_wg = 0;
+        const void* o = nullptr;
+        size_t batch = 0, cols = 0;
+    } dec;
+    long decode_split_fused = 0;     // decode launches that also wrote the next matmul's activation fragments (for tests)
     long gemm_rope_fused = 0;        // matmuls launched with the RoPE epilogue (for tests)
     long gemm_silu_fused = 0;        // ... with the gate/up split + SiLU * up as epilogue
     long gemm_silu_split_fused = 0;  // ... of which also wrote the next matmul's activation fragments
@@ -344,7 +360,7 @@ size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 const void* resident_blob(int kind, const void* key, const void* blob, size_t bytes) {
     // A caller that never repeats itself: start over -- but only while no held-back operator
     // refers to one of the copies (their launches come later).
-    if (g.resident.size() > 1024 && !g.rows.active && !g.kv.active && !g.gemm.active && !g_capturing &&
+    if (g.resident.size() > 1024 && !g.rows.active && !g.kv.active && !g.gemm.active && !g.dec.active && !g_capturing &&
         g.captures.empty()) {   // (a captured pass keeps the addresses of the copies it read)
         if (hipStreamSynchronize(g.stream) != hipSuccess) { fail("resident: synchronize failed"); return nullptr; }
         for (auto& kv : g.resident)
@@ -463,6 +479,21 @@ bool gemm_feeds_rope(const void* qkv, size_t batch, size_t qkv_rows, size_t q_ro
            m.rows == qkv_rows && q_rows + k_rows + v_rows == qkv_rows;
 }
 
+bool launch_stream_variant(size_t D, int hpw, int nw, int nbuf, const StreamArgs& a, unsigned n_wg, size_t dyn_lds,
+                           hipStream_t stream);
+
+// Launches the held-back decode attention.
+int settle_decode() {
+    Ctx::DecodePending& d = g.dec;
+    if (!d.active) return 1;
+    d.active = false;
+    if (d.a.split_frag) ++g.decode_split_fused;
+    if (!launch_stream_variant(d.head_dim, d.hpw, d.nw, d.nbuf, d.a, d.n_wg, d.dyn_lds, g.stream))
+        return fail("decode: kernel variant not built");
+    HIP_OK(hipGetLastError());
+    return 1;
+}
+
 // Launches the pending KV write.
 int settle_kv() {
     Ctx::KvPending& kv = g.kv;
@@ -498,6 +529,9 @@ int settle_kv() {
 // than a pending chain (whatever starts the KV write launches the chain first, and a scatter
 // only joins while no chain is pending).
 int settle() {
+    // a held-back attention launch is older than anything else: whatever was pending when it was
+    // encoded has been launched, and nothing joins a chain behind it before it is launched
+    if (!settle_decode()) return 0;
     // a held-back matmul is older than anything else pending, unless the pending KV write is
     // its own epilogue
     if (g.gemm.active && !(g.kv.active && g.kv.rope && g.kv.from_gemm) && !settle_gemm()) return 0;

@@ -157,8 +157,23 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
         }
         if (g_capturing && g.cap.n_decode > kReplayTagStep)
             return fail("capture: more decode launches in one pass than its tags can tell apart");
-        if (!launch_stream_variant(head_dim, s_hpw, s_nw, nbuf, a, n_wg, dyn_lds, g.stream))
+        // Held back for one call where a Q4_0 matmul reading o could take its activations from
+        // this launch (see Ctx::DecodePending); launched now otherwise.
+        const size_t o_cols = num_heads * head_dim;
+        if (g.opt_fuse_rows && g.opt_q4_int_operand && !g.opt_q4_force_generic && !sync && batch <= 64 &&
+            nbuf == 2 && o_cols % 32 == 0 && o_cols >= 64) {
+            Ctx::DecodePending& d = g.dec;
+            d.active = true;
+            d.a = a;
+            d.head_dim = head_dim; d.dyn_lds = dyn_lds;
+            d.hpw = s_hpw; d.nw = s_nw; d.nbuf = nbuf;
+            d.n_wg = n_wg;
+            d.o = o;
+            d.batch = batch;
+            d.cols = o_cols;
+        } else if (!launch_stream_variant(head_dim, s_hpw, s_nw, nbuf, a, n_wg, dyn_lds, g.stream)) {
             return fail("decode: kernel variant not built");
+        }
         if (g_capturing) {
             Ctx::Captured& c = g.cap;
             if (c.used_tables && (c.B != batch || c.tables_flat != d_flat || c.tables_meta != d_meta))
@@ -227,7 +242,7 @@ int mlc_hip_paged_attn_decode_noalloc(const void* q, const void* k_pages, const 
     {
         // operators held back by earlier encode calls are launched now, on the library's stream
         // (kernel launches only); a caller's stream of its own is put behind them
-        const bool pending = g.rows.active || g.kv.active || g.gemm.active;
+        const bool pending = g.rows.active || g.kv.active || g.gemm.active || g.dec.active;
         if (!settle()) return 0;
         if (pending && st != g.stream) {
             HIP_OK(hipEventRecord(g.scratch_ev, g.stream));

@@ -288,6 +288,9 @@ void stream_fill_common(StreamArgs& a, const void* q, const void* k_pages, const
     a.pair_cost = 0;  // (set by the caller once the workgroup shape is known: stream_pair_cost)
     a.new_k = a.new_v = nullptr;
     a.new_ids = a.new_slots = nullptr;
+    a.split_frag = nullptr;
+    a.split_exp = nullptr;
+    a.split_rows = 0;
 }
 
 }  // namespace

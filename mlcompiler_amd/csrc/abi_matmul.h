@@ -77,7 +77,13 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
                             !(reinterpret_cast<uintptr_t>(out) & 15u) && q4_fast_shape(rows, cols, row_stride) &&
                             g.gemm.active && g.gemm.silu && !g.rows.active && !g.kv.active && g.gemm.silu_out == in &&
                             g.gemm.batch == batch && g.gemm.ffn_inner == cols;
-    if (!feeds && !feeds_silu && !settle()) return 0;
+    // ... or the output of the held-back decode attention?  Then the attention kernel splits it.
+    const bool feeds_attn = !feeds && !feeds_silu && batch <= 64 && g.opt_fuse_rows && g.opt_q4_int_operand &&
+                            !g.opt_q4_force_generic && !(reinterpret_cast<uintptr_t>(out) & 15u) &&
+                            q4_fast_shape(rows, cols, row_stride) && g.dec.active && g.dec.o == in &&
+                            g.dec.batch == batch && g.dec.cols == cols;
+    const bool block_scales = feeds_silu || feeds_attn;
+    if (!feeds && !block_scales && !settle()) return 0;
     Ctx::Q4Weight* w = q4_weight(weight_name, static_cast<const uint8_t*>(weights), weight_bytes, rows, cols, row_stride);
     if (!w) return 0;
 
@@ -108,15 +114,22 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
         const size_t bn = std::min<size_t>(64, batch - bo);
         const size_t bpad = (bn + 31) / 32 * 32;
         // (the held-back projection still reads "q4_x_fragments": its products go to a buffer of their own)
-        _Float16* frag = static_cast<_Float16*>(cached_buffer(feeds_silu ? "q4_x_fragments_silu" : "q4_x_fragments", bpad * cols * 4));
+        _Float16* frag = static_cast<_Float16*>(cached_buffer(
+            feeds_silu ? "q4_x_fragments_silu" : feeds_attn ? "q4_x_fragments_attention" : "q4_x_fragments", bpad * cols * 4));
         float* inv = static_cast<float*>(cached_buffer("q4_x_inv_scale", 64 * 4));
-        int8_t* blk_exp = feeds_silu ? static_cast<int8_t*>(cached_buffer("q4_x_block_exponents", bpad * nblocks)) : nullptr;
-        if (!frag || !inv || (feeds_silu && !blk_exp)) return fail("q4 matmul: scratch allocation failed");
+        int8_t* blk_exp = !block_scales ? nullptr : static_cast<int8_t*>(cached_buffer(
+            feeds_silu ? "q4_x_block_exponents_silu" : "q4_x_block_exponents_attention", bpad * nblocks));
+        if (!frag || !inv || (block_scales && !blk_exp)) return fail("q4 matmul: scratch allocation failed");
         const float* xin = static_cast<const float*>(in) + bo * cols;
         float* o = static_cast<float*>(out) + bo * rows;
         if (feeds_silu) {
             g.gemm.a.split_frag = frag;
             g.gemm.a.split_blk_exp = blk_exp;
+            if (!settle()) return 0;
+        } else if (feeds_attn) {
+            g.dec.a.split_frag = frag;
+            g.dec.a.split_exp = blk_exp;
+            g.dec.a.split_rows = (uint32_t)bpad;
             if (!settle()) return 0;
         } else if (feeds) {  // the chain that produces the input also splits it (batch <= 64: one round)
             g.rows.p.frag = frag;
@@ -146,7 +159,7 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
             Ctx::GemmPending& m = g.gemm;
             m.active = true;
             m.silu = false;
-            m.block_scales = feeds_silu;
+            m.block_scales = block_scales;
             m.a = a;
             m.grid_x = (unsigned)wgs;
             m.nbt = bpad == 32 ? 1 : 2;
@@ -157,7 +170,7 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
             return finish(sync);
         }
         const dim3 grid((unsigned)wgs, (unsigned)ksplit);
-        if (feeds_silu)
+        if (block_scales)
             launch_q4_mfma_block_scales(bpad == 32 ? 1 : 2, row_tiles, grid, a);
         else
             launch_q4_mfma(bpad == 32 ? 1 : 2, row_tiles, grid, a);

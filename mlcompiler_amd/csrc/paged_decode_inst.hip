@@ -13,35 +13,42 @@
 namespace mlc_hip {
 
 namespace {
-template <int NW, bool SMALL, int NBUF>
+template <int NW, bool SMALL, int NBUF, bool SPLIT>
 void launch_stream_pv(int pvm, const StreamArgs& a, unsigned n_wg, size_t dyn_lds, hipStream_t stream) {
     const dim3 grid(n_wg), block(64 * NW);
     if constexpr (NW == 4 && MLC_HPW * NW <= 16) {
         if (pvm == 2) {
-            hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, 2, SMALL, NBUF>), grid, block, dyn_lds, stream, a);
+            hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, 2, SMALL, NBUF, SPLIT>), grid, block, dyn_lds, stream, a);
             return;
         }
         if (pvm == 3) {
-            hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, 3, SMALL, NBUF>), grid, block, dyn_lds, stream, a);
+            hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, 3, SMALL, NBUF, SPLIT>), grid, block, dyn_lds, stream, a);
             return;
         }
     }
     if (pvm == 1 || pvm == 2)
-        hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, 1, SMALL, NBUF>), grid, block, dyn_lds, stream, a);
+        hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, 1, SMALL, NBUF, SPLIT>), grid, block, dyn_lds, stream, a);
     else
-        hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, 0, SMALL, NBUF>), grid, block, dyn_lds, stream, a);
+        hipLaunchKernelGGL((paged_decode_stream_kernel<MLC_D, MLC_HPW, NW, 0, SMALL, NBUF, SPLIT>), grid, block, dyn_lds, stream, a);
 }
 template <int NW>
 bool launch_stream(int nbuf, int pvm, const StreamArgs& a, unsigned n_wg, size_t dyn_lds, hipStream_t stream) {
     // at most 64 requests: the variant that keeps the per-request figures in registers; larger
     // batches keep them in dynamic LDS, next to two or three stages
+    // (the form that also splits its output for the matmul behind it: built for the default of
+    // small batches only, two stages)
+    if (a.split_frag) {
+        if (a.batch > 64 || nbuf != 2) return false;
+        launch_stream_pv<NW, true, 2, true>(pvm, a, n_wg, 0, stream);
+        return true;
+    }
     if (a.batch <= 64) {
-        if (nbuf == 2) launch_stream_pv<NW, true, 2>(pvm, a, n_wg, 0, stream);
-        else if (nbuf == 3) launch_stream_pv<NW, true, 3>(pvm, a, n_wg, 0, stream);
-        else launch_stream_pv<NW, true, 4>(pvm, a, n_wg, 0, stream);
+        if (nbuf == 2) launch_stream_pv<NW, true, 2, false>(pvm, a, n_wg, 0, stream);
+        else if (nbuf == 3) launch_stream_pv<NW, true, 3, false>(pvm, a, n_wg, 0, stream);
+        else launch_stream_pv<NW, true, 4, false>(pvm, a, n_wg, 0, stream);
     } else {
-        if (nbuf == 2) launch_stream_pv<NW, false, 2>(pvm, a, n_wg, dyn_lds, stream);
-        else launch_stream_pv<NW, false, 3>(pvm, a, n_wg, dyn_lds, stream);
+        if (nbuf == 2) launch_stream_pv<NW, false, 2, false>(pvm, a, n_wg, dyn_lds, stream);
+        else launch_stream_pv<NW, false, 3, false>(pvm, a, n_wg, dyn_lds, stream);
     }
     return true;
 }

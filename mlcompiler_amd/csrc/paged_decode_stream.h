@@ -72,6 +72,14 @@ struct StreamArgs {
     const uint4* new_v;
     const uint32_t* new_ids;
     const uint32_t* new_slots;
+    // The split of the output for the Q4_0 matmul that reads it (null: none): whoever writes a row
+    // of o also writes it as hi + lo fp16 fragments in that matmul's B-operand layout
+    // (q4_matmul_kernels.h), scaled by one power of two per (request, block of 32 columns), and the
+    // exponents where the matmul's block-scale form looks for them.  Requests batch .. split_rows-1
+    // are the padding of the last tile of 32 requests and are written as zeros.
+    _Float16* split_frag;
+    int8_t* split_exp;
+    uint32_t split_rows;
     // seq_lens | q_positions | page_table_offsets (at a stride of 64 words for up to 64 requests,
     // of meta_stride words above) and, where it fits as well, the flat page table behind them: a
     // call whose tables travel here copies nothing to the device
@@ -183,7 +191,9 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t x) {
 // weights as in mode 1; mode 3: the weight as the sum of two fp16 numbers, two MFMAs per V block,
 // fp32-grade like mode 0), V^T through the transposing LDS read; the waves' results are combined
 // through LDS where a pair of (request, KV head) ends.
-template <int D, int HPW, int NW, int PVM, bool SMALL, int NBUF>
+// SPLIT: the launch also writes its output as the split-fp16 activations of the Q4_0 matmul that
+// reads it (StreamArgs::split_frag).
+template <int D, int HPW, int NW, int PVM, bool SMALL, int NBUF, bool SPLIT = false>
 __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const StreamArgs a) {
     constexpr bool PV16 = PVM == 1;
     constexpr bool MF = PVM == 2 || PVM == 3;
@@ -339,6 +349,22 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         if (req_lim(rr) == 0) {
             float* orow = a.o + (size_t)rr * a.num_heads * D;
             for (uint32_t i = threadIdx.x; i < a.num_heads * D; i += 64 * NW) orow[i] = 0.f;
+        }
+    }
+    if constexpr (SPLIT) {  // ... and so are their fragments, and those of the padding requests
+        const uint32_t cols = a.num_heads * D;
+        for (uint32_t rr = blockIdx.x; rr < a.split_rows; rr += gridDim.x) {
+            if (rr < B && req_lim(rr) != 0) continue;
+            const uint32_t t32 = rr / 32, n32 = rr % 32;
+            for (uint32_t k8 = threadIdx.x; k8 < cols / 8; k8 += 64 * NW) {
+                const size_t base = ((size_t)t32 * (cols / 16) + k8 / 2) * 2;
+                const uint32_t fl = (k8 % 2) * 32 + n32;
+                const uint4 z = make_uint4(0u, 0u, 0u, 0u);
+                *reinterpret_cast<uint4*>(a.split_frag + ((base + 0) * 64 + fl) * 8) = z;
+                *reinterpret_cast<uint4*>(a.split_frag + ((base + 1) * 64 + fl) * 8) = z;
+            }
+            for (uint32_t blk = threadIdx.x; blk < cols / 32; blk += 64 * NW)
+                a.split_exp[((size_t)t32 * (cols / 32) + blk) * 32 + ((n32 % 8) / 4) * 16 + (n32 / 8) * 4 + n32 % 4] = 0;
         }
     }
 
@@ -997,11 +1023,68 @@ __global__ __launch_bounds__(64 * NW) void paged_decode_stream_kernel(const Stre
         return po;
     };
     auto store_direct = [&](float* orow, const float (&o_un)[OPL], const float (&l_all)[HPW]) {
+        float val[OPL];
 #pragma unroll
         for (int k = 0; k < OPL; ++k) {
             const float l = l_all[k / HPK];
             const float inv = l > 0.f ? 1.0f / l : 0.f;
-            orow[(k / HPK) * D + dim0 + (k % HPK)] = o_un[k] * inv;
+            val[k] = o_un[k] * inv;
+            orow[(k / HPK) * D + dim0 + (k % HPK)] = val[k];
+        }
+        if constexpr (SPLIT) {
+            // A lane holds dims c*8 + r_l*HPK + kk of a head: a block of 32 columns is four values
+            // of c, every r_l.  Its largest magnitude: over lane bits 0, 1 (c % 4) and the bits of r_l.
+            // (the request and the head come from the row's address: nothing more to carry through
+            // the stream for them)
+            const uint32_t cols = a.num_heads * D;
+            const uint32_t row_head = (uint32_t)__builtin_amdgcn_readfirstlane((int)((orow - a.o) / D));
+            const uint32_t req = (uint32_t)__builtin_amdgcn_readfirstlane((int)(row_head / a.num_heads));
+            const uint32_t head0 = row_head - req * a.num_heads;
+            const uint32_t t32 = req / 32, n32 = req % 32;
+#pragma unroll
+            for (int h = 0; h < HPW; ++h) {
+                float amax = 0.f;
+#pragma unroll
+                for (int kk = 0; kk < HPK; ++kk) amax = fmaxf(amax, fabsf(val[h * HPK + kk]));
+                amax = fmaxf(amax, dpp_f<kDppQuadXor1>(amax));
+                amax = fmaxf(amax, dpp_f<kDppQuadXor2>(amax));
+                if constexpr (CPR == 8) amax = fmaxf(amax, dpp_f<kDppRowRor8>(amax));
+                {
+                    const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(amax), __float_as_uint(amax), false, false);
+                    amax = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+                }
+                {
+                    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(amax), __float_as_uint(amax), false, false);
+                    amax = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+                }
+                int e = 0;
+                if (amax > 0.f && amax < INFINITY) (void)frexpf(amax, &e);   // q4_split_activations_kernel's scale
+                int se = 14 - e;
+                se = se > 100 ? 100 : (se < -100 ? -100 : se);
+                const uint32_t col = (head0 + (uint32_t)h) * D + (uint32_t)dim0;   // this lane's first column
+                const size_t base = ((size_t)t32 * (cols / 16) + col / 16) * 2;
+                const uint32_t fl = ((col % 16) / 8) * 32 + n32;
+                _Float16* f_hi = a.split_frag + ((base + 0) * 64 + fl) * 8 + col % 8;
+                _Float16* f_lo = a.split_frag + ((base + 1) * 64 + fl) * 8 + col % 8;
+                _Float16 hi[HPK], lo[HPK];
+#pragma unroll
+                for (int kk = 0; kk < HPK; ++kk) {
+                    const float tv = __builtin_ldexpf(val[h * HPK + kk], se);
+                    hi[kk] = (_Float16)tv;
+                    lo[kk] = (_Float16)(tv - (float)hi[kk]);
+                }
+                if constexpr (HPK == 2) {   // (dim0 is even: the two are one aligned word)
+                    typedef _Float16 sd_half2 __attribute__((ext_vector_type(2)));
+                    *reinterpret_cast<sd_half2*>(f_hi) = sd_half2{hi[0], hi[1]};
+                    *reinterpret_cast<sd_half2*>(f_lo) = sd_half2{lo[0], lo[1]};
+                } else {
+                    f_hi[0] = hi[0];
+                    f_lo[0] = lo[0];
+                }
+                if (c % 4 == 0 && r_l == 0)
+                    a.split_exp[((size_t)t32 * (cols / 32) + col / 32) * 32 + ((n32 % 8) / 4) * 16 + (n32 / 8) * 4 + n32 % 4] =
+                        (int8_t)(-se);
+            }
         }
     };
     // A wave's partial: PW tagged words per lane, word k of lane i at [k][i].  Words 0 .. OPL-1

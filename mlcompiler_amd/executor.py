@@ -304,6 +304,10 @@ class HipExecutor:
         """... of which also wrote the activation fragments of the matmul that reads the products."""
         return int(self._lib.mlc_hip_fused_matmul_silu_split_launches())
 
+    def fusedDecodeSplitLaunches(self) -> int:
+        """Decode attention launches so far that also wrote the next Q4_0 matmul's activation fragments."""
+        return int(self._lib.mlc_hip_fused_decode_split_launches())
+
     def rowProgramLaunches(self) -> int:
         """Fused row-operator launches so far (option "fuse_row_ops")."""
         return int(self._lib.mlc_hip_row_program_launches())
