@@ -355,6 +355,10 @@ long mlc_hip_fused_matmul_silu_split_launches(void);
 /* Number of decode attention launches so far that also wrote their output as the activation
  * fragments of the Q4_0 matmul that reads it (for tests). */
 long mlc_hip_fused_decode_split_launches(void);
+/* Number of Q4_0 matmuls so far that went out with the residual add behind them, the sums of
+ * squares of the RMSNorm behind that and the split-fp16 input of the Q4_0 matmul that reads the
+ * norm as epilogue (that matmul finishes the norm; for tests). */
+long mlc_hip_fused_matmul_norm_launches(void);
 /* Number of decode attention launches so far that carried the step's KV write (a pair of
  * batched K / V scatters of every request's newest position encoded just before it). */
 long mlc_hip_kv_writes_in_decode_launches(void);

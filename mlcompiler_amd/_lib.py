@@ -66,6 +66,7 @@ SIGNATURES = {
     "mlc_hip_fused_matmul_silu_launches": (C.c_long, []),
     "mlc_hip_fused_matmul_silu_split_launches": (C.c_long, []),
     "mlc_hip_fused_decode_split_launches": (C.c_long, []),
+    "mlc_hip_fused_matmul_norm_launches": (C.c_long, []),
     "mlc_hip_kv_writes_in_decode_launches": (C.c_long, []),
     "mlc_hip_set_option": (C.c_int, [C.c_char_p, C.c_long]),
 }

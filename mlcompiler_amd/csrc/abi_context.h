@@ -204,6 +204,7 @@ struct Ctx {
     long decode_split_fused = 0;     // decode launches that also wrote the next matmul's activation fragments (for tests)
     long gemm_rope_fused = 0;        // matmuls launched with the RoPE epilogue (for tests)
     long gemm_silu_fused = 0;        // ... with the gate/up split + SiLU * up as epilogue
+    long gemm_rms_fused = 0;         // ... with the residual add, the RMSNorm's sums and the next matmul's fragments as epilogue
     long gemm_silu_split_fused = 0;  // ... of which also wrote the next matmul's activation fragments
     long kv_fused = 0;               // KV writes that went out fused with a neighbour (for tests)
     long kv_in_decode = 0;           // ... of which inside the attention launch
@@ -421,22 +422,28 @@ void launch_q4_mfma(int nbt, int rt, dim3 grid, const Q4Args& a) {
 }
 
 // The same with activations that were split with one scale per (request, block): a.blk_exp.
-// Integer-operand arithmetic only.
+// Integer-operand arithmetic only.  Two row tiles per workgroup run with 8 waves (the 128 registers
+// a wave of 16 has do not hold the exponents as well), and not with two batch tiles (256 do not
+// either): q4_block_scales_fit() is what callers ask first.
+bool q4_block_scales_fit(size_t bpad, int row_tiles) { return !(bpad > 32 && row_tiles == 2); }
 void launch_q4_mfma_block_scales(int nbt, int rt, dim3 grid, const Q4Args& a) {
 #define MLC_Q4(NBT, RT, WAVES) \
     hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<NBT, RT, WAVES, true, true>), grid, dim3(WAVES * 64), 0, g.stream, a)
     if (nbt == 1) {
-        if (rt == 1) { MLC_Q4(1, 1, 16); } else { MLC_Q4(1, 2, 16); }
+        if (rt == 1) { MLC_Q4(1, 1, 16); } else { MLC_Q4(1, 2, 8); }
     } else {
-        if (rt == 1) { MLC_Q4(2, 1, 8); } else { MLC_Q4(2, 2, 8); }
+        MLC_Q4(2, 1, 8);
     }
 #undef MLC_Q4
 }
 
 // The gate/up projection with the gate/up split + SiLU * up (and, when a.split_frag is set, the
 // split of the products for the matmul that reads them) as epilogue: two row tiles per workgroup.
-void launch_q4_mfma_silu(int nbt, dim3 grid, const Q4Args& a) {
-    if (nbt == 1)
+// (with block-wise activation scales: one batch tile, 8 waves, see launch_q4_mfma_block_scales)
+void launch_q4_mfma_silu(int nbt, bool block_scales, dim3 grid, const Q4Args& a) {
+    if (nbt == 1 && block_scales)
+        hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<1, 2, 8, true, true, true>), grid, dim3(8 * 64), 0, g.stream, a);
+    else if (nbt == 1)
         hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<1, 2, 16, true, false, true>), grid, dim3(16 * 64), 0, g.stream, a);
     else
         hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<2, 2, 8, true, false, true>), grid, dim3(8 * 64), 0, g.stream, a);
@@ -459,7 +466,7 @@ int settle_gemm(const RopeArgs* rope = nullptr) {
         m.silu = false;
         ++g.gemm_silu_fused;
         if (a.split_frag) ++g.gemm_silu_split_fused;
-        launch_q4_mfma_silu(m.nbt, grid, a);
+        launch_q4_mfma_silu(m.nbt, m.block_scales, grid, a);
         HIP_OK(hipGetLastError());
         return 1;
     }

@@ -71,18 +71,33 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
     // replace a buffer the chain still refers to)
     const bool feeds = batch <= 64 && !g.opt_q4_force_generic && !(reinterpret_cast<uintptr_t>(out) & 15u) &&
                        q4_fast_shape(rows, cols, row_stride) && row_len_ok(cols) && rows_continue(in, batch, cols);
+    // ... and is that chain  held-back matmul -> + residual -> RMSNorm?  Then the held-back matmul's
+    // epilogue adds, leaves the sums of squares and writes (sum * gamma) as this matmul's fragments,
+    // block-wise scaled, and this matmul finishes the norm: no launch in between.
+    // (block-wise scaled activations: not every shape of workgroup is built for them)
+    const bool scales_fit = q4_block_scales_fit((batch + 31) / 32 * 32, rows / 32 > 256 ? 2 : 1);
+    bool feeds_rms = false;
+    if (feeds && scales_fit && g.gemm.active && g.opt_q4_int_operand) {
+        const Ctx::GemmPending& m = g.gemm;
+        const RowProgram& p = g.rows.p;
+        const size_t tiles = rows / 32, row_tiles = tiles > 256 ? 2 : 1;
+        feeds_rms = !m.silu && m.rt == 1 && m.a.rope_on == 0 && !g.kv.active && p.src == m.out && p.n_slices == 1 &&
+                    !p.src_store && !p.silu && p.addend && p.rms && !p.frag && g.rows.batch == batch &&
+                    g.rows.len == cols && m.batch == batch && m.rows == cols && cols / 32 <= (batch <= 32 ? 128u : 64u) &&
+                    batch * cols <= 2 * (tiles / row_tiles) * 512;   // (every workgroup of the reader has at least 512 threads)
+    }
     // ... or is the input the SiLU * up product that the held-back gate/up projection's epilogue
     // will write?  Then that epilogue also splits it, per (request, block of 32 columns).
-    const bool feeds_silu = !feeds && batch <= 64 && g.opt_fuse_rows && g.opt_q4_int_operand && !g.opt_q4_force_generic &&
+    const bool feeds_silu = !feeds && scales_fit && batch <= 64 && g.opt_fuse_rows && g.opt_q4_int_operand && !g.opt_q4_force_generic &&
                             !(reinterpret_cast<uintptr_t>(out) & 15u) && q4_fast_shape(rows, cols, row_stride) &&
                             g.gemm.active && g.gemm.silu && !g.rows.active && !g.kv.active && g.gemm.silu_out == in &&
                             g.gemm.batch == batch && g.gemm.ffn_inner == cols;
     // ... or the output of the held-back decode attention?  Then the attention kernel splits it.
-    const bool feeds_attn = !feeds && !feeds_silu && batch <= 64 && g.opt_fuse_rows && g.opt_q4_int_operand &&
+    const bool feeds_attn = !feeds && !feeds_silu && scales_fit && batch <= 64 && g.opt_fuse_rows && g.opt_q4_int_operand &&
                             !g.opt_q4_force_generic && !(reinterpret_cast<uintptr_t>(out) & 15u) &&
                             q4_fast_shape(rows, cols, row_stride) && g.dec.active && g.dec.o == in &&
                             g.dec.batch == batch && g.dec.cols == cols;
-    const bool block_scales = feeds_silu || feeds_attn;
+    const bool block_scales = feeds_silu || feeds_attn || feeds_rms;
     if (!feeds && !block_scales && !settle()) return 0;
     Ctx::Q4Weight* w = q4_weight(weight_name, static_cast<const uint8_t*>(weights), weight_bytes, rows, cols, row_stride);
     if (!w) return 0;
@@ -115,10 +130,15 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
         const size_t bpad = (bn + 31) / 32 * 32;
         // (the held-back projection still reads "q4_x_fragments": its products go to a buffer of their own)
         _Float16* frag = static_cast<_Float16*>(cached_buffer(
-            feeds_silu ? "q4_x_fragments_silu" : feeds_attn ? "q4_x_fragments_attention" : "q4_x_fragments", bpad * cols * 4));
+            feeds_silu ? "q4_x_fragments_silu" : feeds_attn ? "q4_x_fragments_attention" : feeds_rms ? "q4_x_fragments_norm" : "q4_x_fragments",
+            bpad * cols * 4));
         float* inv = static_cast<float*>(cached_buffer("q4_x_inv_scale", 64 * 4));
         int8_t* blk_exp = !block_scales ? nullptr : static_cast<int8_t*>(cached_buffer(
-            feeds_silu ? "q4_x_block_exponents_silu" : "q4_x_block_exponents_attention", bpad * nblocks));
+            feeds_silu ? "q4_x_block_exponents_silu" : feeds_attn ? "q4_x_block_exponents_attention" : "q4_x_block_exponents_norm",
+            bpad * nblocks));
+        float* ssq = feeds_rms ? static_cast<float*>(cached_buffer("q4_norm_partial_sums", nblocks * 64 * 4)) : nullptr;
+        if (feeds_rms && !ssq) return fail("q4 matmul: scratch allocation failed");
+        Q4Args norm{};   // (what this matmul needs to finish the norm)
         if (!frag || !inv || (block_scales && !blk_exp)) return fail("q4 matmul: scratch allocation failed");
         const float* xin = static_cast<const float*>(in) + bo * cols;
         float* o = static_cast<float*>(out) + bo * rows;
@@ -130,6 +150,27 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
             g.dec.a.split_frag = frag;
             g.dec.a.split_exp = blk_exp;
             g.dec.a.split_rows = (uint32_t)bpad;
+            if (!settle()) return 0;
+        } else if (feeds_rms) {
+            Ctx::GemmPending& m = g.gemm;
+            const RowProgram& p = g.rows.p;
+            m.a.add_resid = p.addend;
+            m.a.add_out = p.add_out;
+            m.a.gamma = p.rms_weight;
+            m.a.n_gamma = p.n_weight;
+            m.a.ssq_out = ssq;
+            m.a.split_frag = frag;
+            m.a.split_blk_exp = blk_exp;
+            norm.ssq_in = ssq;
+            norm.ssq_tiles = (uint32_t)nblocks;   // one partial per 32 columns of the norm's row
+            norm.rms_len = (uint32_t)cols;
+            norm.rms_eps = p.epsilon;
+            norm.rms_src = p.add_out;
+            norm.rms_out = p.rms_out;
+            norm.gamma = p.rms_weight;
+            norm.n_gamma = p.n_weight;
+            g.rows.active = false;   // the two matmuls do the chain's work
+            ++g.gemm_rms_fused;
             if (!settle()) return 0;
         } else if (feeds) {  // the chain that produces the input also splits it (batch <= 64: one round)
             g.rows.p.frag = frag;
@@ -146,6 +187,8 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
         Q4Args a{};
         a.qs = static_cast<const uint2*>(w->qs);
         a.blk_exp = blk_exp;
+        a.ssq_in = norm.ssq_in; a.ssq_tiles = norm.ssq_tiles; a.rms_len = norm.rms_len; a.rms_eps = norm.rms_eps;
+        a.rms_src = norm.rms_src; a.rms_out = norm.rms_out; a.gamma = norm.gamma; a.n_gamma = norm.n_gamma;
         a.d = static_cast<const _Float16*>(w->d);
         a.xfrag = frag;
         a.inv_scale = inv;

@@ -37,6 +37,7 @@ long mlc_hip_fused_matmul_rope_launches(void) { return g.gemm_rope_fused; }
 long mlc_hip_fused_matmul_silu_launches(void) { return g.gemm_silu_fused; }
 long mlc_hip_fused_matmul_silu_split_launches(void) { return g.gemm_silu_split_fused; }
 long mlc_hip_fused_decode_split_launches(void) { return g.decode_split_fused; }
+long mlc_hip_fused_matmul_norm_launches(void) { return g.gemm_rms_fused; }
 long mlc_hip_kv_writes_in_decode_launches(void) { return g.kv_in_decode; }
 long mlc_hip_row_program_launches(void) { return g.row_launches; }
 long mlc_hip_decode_table_uploads(void) { return g.table_uploads; }

@@ -63,11 +63,23 @@ int mlc_hip_add_batched(const void* a, const void* b, void* out, size_t total_el
     Ctx::RowPending& r = g.rows;
     const bool joins = fusable && r.active && (r.cur == a || r.cur == b) && !r.p.addend && !r.p.rms && !r.p.frag &&
                        (r.batch ? r.batch * r.len == total_elements && row_len_ok(r.len) : r.n_flat == total_elements);
-    if (!joins && !settle()) return 0;
+    // A residual add on top of the held-back matmul's output (the out-projection): the matmul stays
+    // held back while the chain add -> RMSNorm builds up behind it; if a Q4_0 matmul then reads the
+    // norm, the two matmuls do the chain's work (mlc_hip_matmul_q4_0_batched), and if anything
+    // else comes the matmul and the chain are launched one after the other, as always.
+    const Ctx::GemmPending& m = g.gemm;
+    const bool on_gemm = fusable && !sync && !joins && !r.active && !g.kv.active && !g.dec.active && m.active && !m.silu &&
+                         m.rt == 1 && g.opt_q4_int_operand && (m.out == a || m.out == b) &&
+                         m.batch * m.rows == total_elements && row_len_ok(m.rows);
+    if (!joins && !on_gemm && !settle()) return 0;
     if (fusable) {
         const void* other = a;
         if (joins) {
             other = r.cur == a ? b : a;
+        } else if (on_gemm) {
+            rows_begin(m.out, 0, 0);
+            r.n_flat = total_elements;
+            other = m.out == a ? b : a;
         } else {
             rows_begin(a, 0, 0);
             r.n_flat = total_elements;
@@ -112,7 +124,7 @@ int mlc_hip_gate_up_split_silu_mul(const void* gate_up, void* gate, void* up, vo
         // (workgroup j takes row tile j of the gate half and row tile j of the up half).
         Ctx::GemmPending& m = g.gemm;
         if (g.opt_fuse_rows && g.opt_q4_int_operand && !sync && m.active && !m.silu && !g.rows.active && !g.kv.active &&
-            m.rt == 2 && m.out == gate_up && m.batch == batch && m.rows == ffn_gate_up_rows &&
+            m.rt == 2 && !(m.block_scales && m.nbt != 1) && m.out == gate_up && m.batch == batch && m.rows == ffn_gate_up_rows &&
             ffn_gate_up_rows == 2 * ffn_inner && ffn_inner % 32 == 0 && aligned16(gate) && aligned16(up) && aligned16(out)) {
             m.silu = true;
             m.silu_out = out;

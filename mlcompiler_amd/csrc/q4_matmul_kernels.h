@@ -24,6 +24,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "paged_decode_kernels.h"
 #include "paged_rope_kernels.h"
 
 namespace mlc_hip {
@@ -166,7 +167,68 @@ struct Q4Args {
     float* silu_out;
     _Float16* split_frag;
     int8_t* split_blk_exp;
+    // One row tile per workgroup, ksplit == 1, no RoPE epilogue, add_resid set: the epilogue also
+    // does the residual add that follows the matmul (add_out = out + add_resid, [batch][rows]), leaves
+    // every request's sum of squares over the workgroup's 32 columns in ssq_out[tile][64] (the
+    // RMSNorm that follows is finished by the matmul that reads it, see ssq_in) and writes
+    // add_out * gamma as the split-fp16 fragments of that matmul (split_frag / split_blk_exp,
+    // K = rows).  gamma[c] for c < n_gamma, 1 beyond.
+    const float* add_resid;
+    float* add_out;
+    const float* gamma;
+    uint32_t n_gamma;
+    float* ssq_out;
+    // ssq_in set (BS kernels): the activations are h * gamma of an RMSNorm whose per-request factor
+    // 1 / sqrt(mean(h^2) + eps) is still missing: it is computed here from the ssq_tiles partial
+    // sums of squares per request (ssq_in[tile][64], summed in tile order) and multiplied into the
+    // result, and the workgroups also write the RMSNorm's own output rms_out = h * factor * gamma
+    // ([batch][rms_len], h = rms_src), one or two elements per thread of the grid.
+    const float* ssq_in;
+    uint32_t ssq_tiles, rms_len;
+    float rms_eps;
+    const float* rms_src;
+    float* rms_out;
 };
+
+// Maximum / sum over the 32 lanes of a half wave, every lane gets the result.
+__device__ __forceinline__ float q4_half_wave_max(float v) {
+    v = fmaxf(v, dpp_f<kDppQuadXor1>(v));
+    v = fmaxf(v, dpp_f<kDppQuadXor2>(v));
+    v = fmaxf(v, dpp_f<kDppHalfMirror>(v));
+    v = fmaxf(v, dpp_f<kDppRowRor8>(v));
+    const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+}
+__device__ __forceinline__ float q4_half_wave_sum(float v) {
+    v += dpp_f<kDppQuadXor1>(v);
+    v += dpp_f<kDppQuadXor2>(v);
+    v += dpp_f<kDppHalfMirror>(v);
+    v += dpp_f<kDppRowRor8>(v);
+    const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+}
+
+// One value per lane, the 32 lanes of a half wave holding columns col0 .. col0+31 (one Q4_0 block)
+// of request b: writes them as hi + lo fp16 fragments of a matmul with K = k_cols, scaled by the
+// block's own power of two, and the exponent (q4_split_activations_kernel's scale, per block).
+__device__ __forceinline__ void q4_emit_block(float v, uint32_t b, uint32_t col, uint32_t k_cols, _Float16* frag,
+                                              int8_t* blk_exp) {
+    const float amax = q4_half_wave_max(fabsf(v));
+    int e = 0;
+    if (amax > 0.f && amax < INFINITY) (void)frexpf(amax, &e);
+    int se = 14 - e;
+    se = se > 100 ? 100 : (se < -100 ? -100 : se);
+    const float tv = __builtin_ldexpf(v, se);
+    const _Float16 hi = (_Float16)tv;
+    const _Float16 lo = (_Float16)(tv - (float)hi);
+    const uint32_t t = b / 32, c = b % 32;
+    const size_t base = ((size_t)t * (k_cols / 16) + col / 16) * 2;
+    const uint32_t fl = ((col % 16) / 8) * 32 + c;
+    frag[((base + 0) * 64 + fl) * 8 + col % 8] = hi;
+    frag[((base + 1) * 64 + fl) * 8 + col % 8] = lo;
+    if (col % 32 == 0)
+        blk_exp[((size_t)t * (k_cols / 32) + col / 32) * 32 + ((c % 8) / 4) * 16 + (c / 8) * 4 + c % 4] = (int8_t)(-se);
+}
 
 // The split + RoPE + cast (+ paged write) of one element of a request's fused qkv row, by the
 // thread that just produced it; the partner of its (even, odd) pair sits in the neighbouring
@@ -263,6 +325,11 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
     constexpr int PF = WAVES >= 16 ? 2 : 4;  // blocks in flight per wave
     constexpr int PITCH = 65;                // floats per accumulator register in LDS (bank spread)
     __shared__ float red[WAVES * RT * NBT * 16 * PITCH];
+    __shared__ float rms_scale[BS ? 32 * NBT : 1];   // BS with ssq_in: every request's RMSNorm factor
+    constexpr int SSQ_P = WAVES * 64 / (32 * NBT);   // threads per request that share the sum over the partials
+    constexpr int SSQ_NL = 128 / SSQ_P < 8 ? 128 / SSQ_P : 8;   // partials per thread, at most: up to 128 tiles (rows of
+                                                                // 4096), 64 with two batch tiles (the host checks)
+    __shared__ float ssq_lds[BS ? SSQ_P * 32 * NBT : 1];
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const uint32_t lane = threadIdx.x % 64;
     const uint32_t l32 = lane % 32;
@@ -292,6 +359,22 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
 #pragma unroll
         for (uint32_t pass = 0; pass < PASSES; ++pass)
             rope_pre[pass] = q4_rope_prefetch(a.rope, pass * COLS_PER_PASS + bsub, tile0 * 32 + row);
+    }
+
+    // (the fused residual add: the residual and gamma of this thread's outputs, fetched ahead like the
+    // RoPE operands)
+    constexpr bool ADD_AHEAD = IOP && RT == 1 && PASSES <= 2;
+    float resid_pre[ADD_AHEAD ? PASSES : 1] = {};
+    float gamma_pre = 1.0f;
+    if constexpr (ADD_AHEAD) {
+        if (a.add_resid) {
+#pragma unroll
+            for (uint32_t pass = 0; pass < PASSES; ++pass) {
+                const uint32_t b = pass * COLS_PER_PASS + bsub;
+                if (b < a.batch) resid_pre[pass] = a.add_resid[(size_t)b * a.rows + tile0 * 32 + row];
+            }
+            if (tile0 * 32 + row < a.n_gamma) gamma_pre = a.gamma[tile0 * 32 + row];
+        }
     }
 
     struct Block {
@@ -335,7 +418,7 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
             for (int r = 0; r < RT; ++r) {
                 // (SILU: one row tile's products after the other, or the scheduler keeps three
                 // sets of 16 in flight and the loop no longer fits the 128 registers a wave has)
-                if constexpr (SILU) { if (r) __builtin_amdgcn_sched_barrier(0); }
+                if constexpr (SILU && WAVES == 16) { if (r) __builtin_amdgcn_sched_barrier(0); }
                 const float d = k.real ? (float)k.d[r] : 0.0f;
                 q4_half8 w[2];
 #pragma unroll
@@ -412,6 +495,30 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
         load(b0 + wave + i * WAVES, k[i]);
         asm volatile("" ::: "memory");
     }
+    // The RMSNorm that the producer of the activations left unfinished (ssq_in): the requests'
+    // factors, for the epilogue, and this thread's elements of the norm's own output, fetched now
+    // and written at the end.
+    float rms_h[BS ? 2 : 1] = {};
+    float ssq_part[BS ? SSQ_NL : 1] = {};
+    if constexpr (BS) {
+        if (a.ssq_in) {
+            // thread (request b, part p) takes the partials of tiles p, p + SSQ_P, ...: all loads go out
+            // now, next to the first blocks', and are summed behind the main loop
+            const uint32_t sb = threadIdx.x % (32 * NBT), sp = threadIdx.x / (32 * NBT);
+#pragma unroll
+            for (int j = 0; j < SSQ_NL; ++j) {
+                const uint32_t tl = sp + j * SSQ_P;
+                if (tl < a.ssq_tiles && sb < a.batch) ssq_part[j] = a.ssq_in[tl * 64 + sb];
+            }
+            const uint32_t n_el = a.batch * a.rms_len, n_thr = gridDim.x * (WAVES * 64);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const uint32_t el = j * n_thr + blockIdx.x * (WAVES * 64) + threadIdx.x;
+                if (el < n_el) rms_h[j] = a.rms_src[el];
+            }
+            asm volatile("" ::: "memory");
+        }
+    }
     for (uint32_t base = b0 + wave; base < b1; base += PF * WAVES) {
 #pragma unroll
         for (int i = 0; i < PF; ++i) {
@@ -431,14 +538,43 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
 #pragma unroll
             for (int i = 0; i < 16; ++i)
                 red[(((wave * RT + r) * NBT + t) * 16 + i) * PITCH + lane] = acc[r][t][i];
+    if constexpr (BS) {
+        if (a.ssq_in) {
+            float part = 0.f;
+#pragma unroll
+            for (int j = 0; j < SSQ_NL; ++j) part += ssq_part[j];
+            ssq_lds[threadIdx.x] = part;   // [part][request]
+        }
+    }
     __syncthreads();
+    if constexpr (BS) {
+        if (a.ssq_in) {
+            if (threadIdx.x < 32 * NBT) {
+                float total = 0.f;
+#pragma unroll
+                for (int sp = 0; sp < SSQ_P; ++sp) total += ssq_lds[sp * 32 * NBT + threadIdx.x];
+                rms_scale[threadIdx.x] = 1.0f / sqrtf(total / (float)a.rms_len + a.rms_eps);
+            }
+            __syncthreads();
+            // the norm's own output: h * factor * gamma, the arithmetic of rms_norm_batched_kernel
+            const uint32_t n_el = a.batch * a.rms_len, n_thr = gridDim.x * (WAVES * 64);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const uint32_t el = j * n_thr + blockIdx.x * (WAVES * 64) + threadIdx.x;
+                if (el < n_el) {
+                    const uint32_t rb = el / a.rms_len, rc = el - rb * a.rms_len;
+                    const float gm = rc < a.n_gamma ? a.gamma[rc] : 1.0f;
+                    a.rms_out[el] = rms_h[j] * rms_scale[rb] * gm;
+                }
+            }
+        }
+    }
     if constexpr (SILU) {
         // thread -> (column rr of the workgroup's 32 ffn columns, request b); the 32 lanes of a half
         // wave hold one request's 32 columns, which are one block of the consuming matmul's K
         constexpr uint32_t B_PER_PASS = WAVES * 2, S_PASSES = 32 * NBT / B_PER_PASS;
         const uint32_t rr = threadIdx.x % 32, bs = threadIdx.x / 32;
         const uint32_t col = tile0 * 32 + rr;            // column of gate / up / silu_out
-        const uint32_t nblk_out = a.ffn_inner / 32, ksteps_out = a.ffn_inner / 16;
 #pragma unroll
         for (uint32_t pass = 0; pass < S_PASSES; ++pass) {
             const uint32_t b = pass * B_PER_PASS + bs;
@@ -453,7 +589,7 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
             }
             float prod = 0.f;
             if (live) {
-                const float inv = a.inv_scale[b];
+                const float inv = BS ? (a.ssq_in ? rms_scale[b] : 1.0f) : a.inv_scale[b];
                 const float gv = sg * inv, uv = su * inv;
                 prod = q4_silu_times(gv, uv);
                 a.out[(size_t)b * a.rows + col] = gv;
@@ -462,27 +598,8 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
                 a.up[(size_t)b * a.ffn_inner + col] = uv;
                 a.silu_out[(size_t)b * a.ffn_inner + col] = prod;
             }
-            if (a.split_frag) {   // (uniform; requests past the batch are written as zeros)
-                float amax = fabsf(prod);
-#pragma unroll
-                for (int off = 16; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
-                int e = 0;
-                if (amax > 0.f && amax < INFINITY) (void)frexpf(amax, &e);
-                int se = 14 - e;
-                se = se > 100 ? 100 : (se < -100 ? -100 : se);
-                const float tv = prod * ldexpf(1.0f, se);
-                const _Float16 hi = (_Float16)tv;
-                const _Float16 lo = (_Float16)(tv - (float)hi);
-                const uint32_t k = col;
-                const size_t base = ((size_t)t * ksteps_out + k / 16) * 2;
-                const uint32_t fl = ((k % 16) / 8) * 32 + b % 32;
-                a.split_frag[((base + 0) * 64 + fl) * 8 + k % 8] = hi;
-                a.split_frag[((base + 1) * 64 + fl) * 8 + k % 8] = lo;
-                if (rr == 0) {
-                    const uint32_t c = b % 32;
-                    a.split_blk_exp[((size_t)t * nblk_out + tile0) * 32 + ((c % 8) / 4) * 16 + (c / 8) * 4 + c % 4] = (int8_t)(-se);
-                }
-            }
+            // (uniform; requests past the batch are written as zeros)
+            if (a.split_frag) q4_emit_block(prod, b, col, a.ffn_inner, a.split_frag, a.split_blk_exp);
         }
         return;
     }
@@ -491,18 +608,37 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
 #pragma unroll
     for (uint32_t pass = 0; pass < PASSES; ++pass) {
         const uint32_t b = pass * COLS_PER_PASS + bsub;
-        if (b >= a.batch) continue;
+        const bool fused_add = IOP && RT == 1 && a.add_resid;   // (uniform; then a half wave is one request's 32 columns)
+        if (b >= a.batch && !fused_add) continue;
+        const bool live = b < a.batch;
         const uint32_t t = b / 32;
         const uint32_t in_reg = IOP ? b % 32 : rr, in_lane = IOP ? rr : b % 32;
         const uint32_t i = (in_reg / 8) * 4 + in_reg % 4, ln = ((in_reg % 8) / 4) * 32 + in_lane;
         float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) sum += red[(((w * RT + r) * NBT + t) * 16 + i) * PITCH + ln];
-        const float val = BS ? sum : sum * a.inv_scale[b];
-        out[(size_t)b * a.rows + tile0 * 32 + row] = val;
+        float val;
+        if constexpr (BS) val = a.ssq_in ? sum * rms_scale[b % (32 * NBT)] : sum;
+        else val = live ? sum * a.inv_scale[b] : 0.f;
+        const uint32_t col = tile0 * 32 + row;
+        if (live) out[(size_t)b * a.rows + col] = val;
         if (a.rope_on)  // (the lanes of a pair share b)
-            q4_rope_epilogue(a.rope, ROPE_AHEAD ? rope_pre[ROPE_AHEAD ? pass : 0] : q4_rope_prefetch(a.rope, b, tile0 * 32 + row),
-                             b, tile0 * 32 + row, val);
+            q4_rope_epilogue(a.rope, ROPE_AHEAD ? rope_pre[ROPE_AHEAD ? pass : 0] : q4_rope_prefetch(a.rope, b, col), b, col, val);
+        if constexpr (IOP && RT == 1) {
+            if (fused_add) {
+                // residual add, this request's sum of squares over the 32 columns, and h * gamma as the
+                // next matmul's fragments (requests past the batch: zeros)
+                float hv = 0.f;
+                if (live) {
+                    hv = val + (ADD_AHEAD ? resid_pre[ADD_AHEAD ? pass : 0] : a.add_resid[(size_t)b * a.rows + col]);
+                    a.add_out[(size_t)b * a.rows + col] = hv;
+                }
+                const float ssq = q4_half_wave_sum(hv * hv);
+                if (row == 0 && live) a.ssq_out[(size_t)tile0 * 64 + b] = ssq;
+                const float gm = ADD_AHEAD ? gamma_pre : (col < a.n_gamma ? a.gamma[col] : 1.0f);
+                q4_emit_block(hv * gm, b, col, a.rows, a.split_frag, a.split_blk_exp);
+            }
+        }
     }
 }
 

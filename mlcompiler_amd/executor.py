@@ -308,6 +308,11 @@ class HipExecutor:
         """Decode attention launches so far that also wrote the next Q4_0 matmul's activation fragments."""
         return int(self._lib.mlc_hip_fused_decode_split_launches())
 
+    def fusedMatmulNormLaunches(self) -> int:
+        """Q4_0 matmuls so far launched with the residual add, the RMSNorm's sums and the next matmul's
+        input as epilogue."""
+        return int(self._lib.mlc_hip_fused_matmul_norm_launches())
+
     def rowProgramLaunches(self) -> int:
         """Fused row-operator launches so far (option "fuse_row_ops")."""
         return int(self._lib.mlc_hip_row_program_launches())

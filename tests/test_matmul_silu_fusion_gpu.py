@@ -75,7 +75,9 @@ SHAPES = {
     "tinyllama": dict(B=32, hid=2048, ffn=5632, rows_out=2048, fused=True),
     "two_batch_tiles": dict(B=40, hid=256, ffn=4128, rows_out=192, fused=True),
     "ragged_batch": dict(B=5, hid=128, ffn=4160, rows_out=64, fused=True, spread=True),
-    "down_not_split_over_k": dict(B=33, hid=64, ffn=4128, rows_out=8192 + 64, fused=True, spread=True),
+    "down_not_split_over_k": dict(B=20, hid=64, ffn=4128, rows_out=8192 + 64, fused=True, spread=True),
+    # (two batch tiles and two row tiles per workgroup: no kernel for block-wise scales, the split stays a launch)
+    "down_two_tiles_each_way": dict(B=33, hid=64, ffn=4128, rows_out=8192 + 64, fused=True, split=False, spread=True),
     "few_rows": dict(B=9, hid=256, ffn=512, rows_out=256, fused=False),
 }
 
@@ -85,12 +87,13 @@ SHAPES = {
 def test_matmul_with_silu_epilogue_matches_separate_launches(exe, shape, form):
     kw = dict(SHAPES[shape])
     expect_fused = kw.pop("fused")
+    expect_split = kw.pop("split", True)
     c = Case(seed=zlib.crc32(f"{shape}.{form}".encode()) % 1000, **kw)
     print(f"[case] {shape} {form} B={c.B} hid={c.hid} ffn={c.ffn} rows_out={c.rows_out}", flush=True)
     plain, n_plain = _run(exe, c, form, fuse=0)
     fused, n_fused = _run(exe, c, form, fuse=1)
     assert n_plain == (0, 0)
-    assert n_fused == ((1, 1 if form == "down" else 0) if expect_fused else (0, 0))
+    assert n_fused == ((1, 1 if form == "down" and expect_split else 0) if expect_fused else (0, 0))
     for n in ("gate_up", "gate", "up", "prod"):
         assert np.array_equal(plain[n].view(np.uint8), fused[n].view(np.uint8)), n
     # against the oracle: the projection, the split + SiLU of the GPU's own projection (expf and the
