@@ -13,6 +13,12 @@
 //     two per request that places the row's largest magnitude at 2^13..2^14;
 //   * out = (W_hi.X_hi + W_hi.X_lo + W_lo.X_hi) / s -- three MFMAs per 16 columns; the dropped
 //     W_lo.X_lo term is below 2^-22 of the products.
+// The default arithmetic (IOP) instead takes the integers q - 8 as operand, exact in fp16, and adds
+// every block's sum (q-8).x_hi + (q-8).x_lo to the result as d * sum: nothing is dropped.  There
+// the activations may also come with one power-of-two scale per (request, block of 32 columns)
+// (BS), which a kernel that produces 32 neighbouring columns of a request can compute on its own:
+// the epilogues below (gate/up split + SiLU * up; residual add + RMSNorm) and the decode attention
+// write the next matmul's fragments that way.
 // The weights are repacked once, when they enter the library's weight cache, so that the A
 // operand of a 32-row tile is one coalesced 8-byte load per lane and block; the activations
 // are split by a small kernel into the B-operand layout, so that a fragment is one 16-byte
