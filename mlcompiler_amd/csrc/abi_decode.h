@@ -16,7 +16,7 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
     // (batched_walker.cpp:304-331): then the attention launch does it (decided below, once the
     // tables are known to be valid); anything else pending is launched now.
     bool carries_kv = g.opt_fuse_rows && g.kv.active && !g.kv.rope && g.kv.n == 2 && g.kv.wide && !g.rows.active &&
-                      !g.gemm.active && g.kv.pages[0] == k_pages && g.kv.pages[1] == v_pages && g.kv.batch == batch &&
+                      !g.gemm.active && !g.dec.active && g.kv.pages[0] == k_pages && g.kv.pages[1] == v_pages && g.kv.batch == batch &&
                       g.kv.row_elems == kv_heads * head_dim && g.kv.page_size == page_size_tokens;
     if (!carries_kv && !settle()) return 0;
     if (!sync && !g.pass_open) return fail("encode: no open forward pass");  // :7090
@@ -163,6 +163,7 @@ int mlc_hip_paged_attn_decode(const void* q, const void* k_pages, const void* v_
         if (g.opt_fuse_rows && g.opt_q4_int_operand && !g.opt_q4_force_generic && !sync && batch <= 64 &&
             nbuf == 2 && o_cols % 32 == 0 && o_cols >= 64) {
             Ctx::DecodePending& d = g.dec;
+            if (d.active && !settle_decode()) return 0;   // (never the case: whatever led here has launched it)
             d.active = true;
             d.a = a;
             d.head_dim = head_dim; d.dyn_lds = dyn_lds;

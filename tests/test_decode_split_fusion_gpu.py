@@ -17,7 +17,8 @@ pytestmark = pytest.mark.gpu
 def _run(exe, case, w, rows_out, form, fuse, options=()):
     """form: 'proj' (attention, then the matmul that reads its output), 'alone' (attention, then the
     pass ends), 'other' (attention, then a matmul that reads another buffer), 'twice' (two attention
-    calls into the same buffer, then the matmul)."""
+    calls into the same buffer, then the matmul), 'download' (attention, then its output is read back
+    while the pass is still open, then the matmul)."""
     B, cols = case.batch, case.num_heads * case.head_dim
     dev = DeviceCase(exe, case)
     other = np.random.default_rng(3).standard_normal((B, cols)).astype(np.float32)
@@ -35,6 +36,10 @@ def _run(exe, case, w, rows_out, form, fuse, options=()):
         assert exe.encodePagedFlashAttention(*args), exe.lastError()
         if form == "twice":
             assert exe.encodePagedFlashAttention(*args), exe.lastError()
+        if form == "download":
+            early = np.empty(case.q.shape, np.float32)
+            assert exe.downloadFromBuffer(dev.o_buf, early)      # no flush in between
+            assert not np.isnan(early).any()
         if form != "alone":
             assert exe.encodeMatMulQ4_0Batched(f"{case.name}.proj", w, d_other if form == "other" else dev.o_buf, B, rows_out,
                                                cols, po.q4_0_row_bytes(cols), 1, d_out), exe.lastError()
@@ -72,7 +77,7 @@ SHAPES = {
 }
 
 
-@pytest.mark.parametrize("form", ["proj", "alone", "other", "twice"])
+@pytest.mark.parametrize("form", ["proj", "alone", "other", "twice", "download"])
 @pytest.mark.parametrize("shape", list(SHAPES), ids=list(SHAPES))
 def test_attention_writes_the_next_matmuls_activations(exe, shape, form):
     kw = SHAPES[shape]
