@@ -439,10 +439,11 @@ void launch_q4_mfma_block_scales(int nbt, int rt, dim3 grid, const Q4Args& a) {
 
 // The gate/up projection with the gate/up split + SiLU * up (and, when a.split_frag is set, the
 // split of the products for the matmul that reads them) as epilogue: two row tiles per workgroup.
-// (with block-wise activation scales: one batch tile, 8 waves, see launch_q4_mfma_block_scales)
+// (with block-wise activation scales: one batch tile only, see launch_q4_mfma_block_scales; its 16
+// waves fit their 128 registers because the epilogue's kernel schedules the scaling in groups of four)
 void launch_q4_mfma_silu(int nbt, bool block_scales, dim3 grid, const Q4Args& a) {
     if (nbt == 1 && block_scales)
-        hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<1, 2, 8, true, true, true>), grid, dim3(8 * 64), 0, g.stream, a);
+        hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<1, 2, 16, true, true, true>), grid, dim3(16 * 64), 0, g.stream, a);
     else if (nbt == 1)
         hipLaunchKernelGGL((q4_0_matmul_mfma_kernel<1, 2, 16, true, false, true>), grid, dim3(16 * 64), 0, g.stream, a);
     else

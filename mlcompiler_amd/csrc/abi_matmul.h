@@ -84,7 +84,7 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
         feeds_rms = !m.silu && m.rt == 1 && m.a.rope_on == 0 && !g.kv.active && p.src == m.out && p.n_slices == 1 &&
                     !p.src_store && !p.silu && p.addend && p.rms && !p.frag && g.rows.batch == batch &&
                     g.rows.len == cols && m.batch == batch && m.rows == cols && cols / 32 <= (batch <= 32 ? 128u : 64u) &&
-                    batch * cols <= 2 * (tiles / row_tiles) * 512;   // (every workgroup of the reader has at least 512 threads)
+                    batch * cols <= (tiles / row_tiles) * 1024;   // (every workgroup of the reader writes 1024 elements of the norm)
     }
     // ... or is the input the SiLU * up product that the held-back gate/up projection's epilogue
     // will write?  Then that epilogue also splits it, per (request, block of 32 columns).

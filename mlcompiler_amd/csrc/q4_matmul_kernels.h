@@ -188,7 +188,7 @@ struct Q4Args {
     // 1 / sqrt(mean(h^2) + eps) is still missing: it is computed here from the ssq_tiles partial
     // sums of squares per request (ssq_in[tile][64], summed in tile order) and multiplied into the
     // result, and the workgroups also write the RMSNorm's own output rms_out = h * factor * gamma
-    // ([batch][rms_len], h = rms_src), one or two elements per thread of the grid.
+    // ([batch][rms_len], h = rms_src), 1024 elements per workgroup of the grid.
     const float* ssq_in;
     uint32_t ssq_tiles, rms_len;
     float rms_eps;
@@ -336,6 +336,8 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
     constexpr int SSQ_NL = 128 / SSQ_P < 8 ? 128 / SSQ_P : 8;   // partials per thread, at most: up to 128 tiles (rows of
                                                                 // 4096), 64 with two batch tiles (the host checks)
     __shared__ float ssq_lds[BS ? SSQ_P * 32 * NBT : 1];
+    constexpr int RMS_NE = WAVES >= 16 ? 1 : 2;   // elements of the norm's output per thread: 1024 per workgroup
+    __shared__ float rms_h_lds[BS ? RMS_NE * WAVES * 64 : 1];   // ... parked here through the main loop
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const uint32_t lane = threadIdx.x % 64;
     const uint32_t l32 = lane % 32;
@@ -454,6 +456,9 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
                                 const int ex = (int)(e4 << (24 - 8 * e)) >> 24;   // signed byte e
                                 acc[r][t][j * 4 + e] = fmaf(__builtin_ldexpf(d, ex), sblk[j * 4 + e], acc[r][t][j * 4 + e]);
                             }
+                            // (16 waves with two row tiles: four scaled values of d at a time, not sixteen,
+                            // or the loop does not fit the 128 registers a wave has)
+                            if constexpr (SILU && WAVES == 16) __builtin_amdgcn_sched_barrier(0);
                         }
                     } else {
 #pragma unroll
@@ -495,21 +500,15 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
     // The empty asm statements (they claim to touch memory) pin every group of loads where it
     // is written: without them the compiler moves the loads for a later block down to just
     // before their use, across the loop's back edge too, and the prefetch is gone.
-    Block k[PF];
-#pragma unroll
-    for (int i = 0; i < PF; ++i) {
-        load(b0 + wave + i * WAVES, k[i]);
-        asm volatile("" ::: "memory");
-    }
     // The RMSNorm that the producer of the activations left unfinished (ssq_in): the requests'
-    // factors, for the epilogue, and this thread's elements of the norm's own output, fetched now
-    // and written at the end.
-    float rms_h[BS ? 2 : 1] = {};
+    // sums of squares, for the factors in the epilogue, and this thread's elements of the norm's own
+    // output, which is written at the end.  Thread (request b, part p) takes the partials of tiles
+    // p, p + SSQ_P, ...; their loads go out first, so that they are back and summed up while the
+    // first blocks' are on the way, and take no registers through the main loop.
+    float rms_h[BS ? RMS_NE : 1] = {};
     float ssq_part[BS ? SSQ_NL : 1] = {};
     if constexpr (BS) {
         if (a.ssq_in) {
-            // thread (request b, part p) takes the partials of tiles p, p + SSQ_P, ...: all loads go out
-            // now, next to the first blocks', and are summed behind the main loop
             const uint32_t sb = threadIdx.x % (32 * NBT), sp = threadIdx.x / (32 * NBT);
 #pragma unroll
             for (int j = 0; j < SSQ_NL; ++j) {
@@ -518,10 +517,27 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
             }
             const uint32_t n_el = a.batch * a.rms_len, n_thr = gridDim.x * (WAVES * 64);
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
+            for (int j = 0; j < RMS_NE; ++j) {
                 const uint32_t el = j * n_thr + blockIdx.x * (WAVES * 64) + threadIdx.x;
                 if (el < n_el) rms_h[j] = a.rms_src[el];
             }
+            asm volatile("" ::: "memory");
+        }
+    }
+    Block k[PF];
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+        load(b0 + wave + i * WAVES, k[i]);
+        asm volatile("" ::: "memory");
+    }
+    if constexpr (BS) {
+        if (a.ssq_in) {
+            float part = 0.f;
+#pragma unroll
+            for (int j = 0; j < SSQ_NL; ++j) part += ssq_part[j];
+            ssq_lds[threadIdx.x] = part;   // [part][request]; read behind the barrier that follows the main loop
+#pragma unroll
+            for (int j = 0; j < RMS_NE; ++j) rms_h_lds[j * WAVES * 64 + threadIdx.x] = rms_h[j];
             asm volatile("" ::: "memory");
         }
     }
@@ -544,14 +560,6 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
 #pragma unroll
             for (int i = 0; i < 16; ++i)
                 red[(((wave * RT + r) * NBT + t) * 16 + i) * PITCH + lane] = acc[r][t][i];
-    if constexpr (BS) {
-        if (a.ssq_in) {
-            float part = 0.f;
-#pragma unroll
-            for (int j = 0; j < SSQ_NL; ++j) part += ssq_part[j];
-            ssq_lds[threadIdx.x] = part;   // [part][request]
-        }
-    }
     __syncthreads();
     if constexpr (BS) {
         if (a.ssq_in) {
@@ -565,12 +573,12 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
             // the norm's own output: h * factor * gamma, the arithmetic of rms_norm_batched_kernel
             const uint32_t n_el = a.batch * a.rms_len, n_thr = gridDim.x * (WAVES * 64);
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
+            for (int j = 0; j < RMS_NE; ++j) {
                 const uint32_t el = j * n_thr + blockIdx.x * (WAVES * 64) + threadIdx.x;
                 if (el < n_el) {
                     const uint32_t rb = el / a.rms_len, rc = el - rb * a.rms_len;
                     const float gm = rc < a.n_gamma ? a.gamma[rc] : 1.0f;
-                    a.rms_out[el] = rms_h[j] * rms_scale[rb] * gm;
+                    a.rms_out[el] = rms_h_lds[j * WAVES * 64 + threadIdx.x] * rms_scale[rb] * gm;
                 }
             }
         }
