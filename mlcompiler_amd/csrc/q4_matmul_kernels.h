@@ -385,14 +385,22 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
         }
     }
 
-    struct Block {
+    // A block's weights (3 registers per row tile, from HBM) and its activations (16 per batch tile,
+    // from the L2) are fetched separately: the weights further ahead, PFW blocks, where the registers
+    // allow it.  A wave of the TinyLlama shapes has four blocks in all, so all of its weights are on
+    // the way from the start instead of in two rounds of a memory latency each.
+    constexpr int PFW = (IOP && WAVES >= 16 && (RT == 1 || (SILU && !BS))) ? 4 : PF;
+    static_assert(PFW % PF == 0, "a block's activations sit in slot (block number) % PF");
+    struct BlockW {
         uint2 q[RT];
         _Float16 d[RT];
-        q4_half8 x[NBT][2][2];  // [batch tile][k step][hi, lo]
-        uint4 ex[BS ? NBT : 1];   // BS: scale exponents of the 16 batch columns in this lane's registers, a byte each
         bool real;               // false: a repeat past the end of the slice, multiplied with scale 0
     };
-    auto load = [&](uint32_t blk_raw, Block& k) __attribute__((always_inline)) {
+    struct BlockX {
+        q4_half8 x[NBT][2][2];  // [batch tile][k step][hi, lo]
+        uint4 ex[BS ? NBT : 1];   // BS: scale exponents of the 16 batch columns in this lane's registers, a byte each
+    };
+    auto load_w = [&](uint32_t blk_raw, BlockW& k) __attribute__((always_inline)) {
         // Past the end of the slice: a repeat of its last block, multiplied with the scale set to
         // zero, so that the multiply needs no branch (a branch lets the compiler sink these loads
         // into it, next to their use, which undoes the prefetch).
@@ -405,6 +413,9 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
             k.q[r] = q4_stream_u2(a.qs + tb * 64 + lane);
             k.d[r] = __builtin_nontemporal_load(a.d + tb * 32 + l32);
         }
+    };
+    auto load_x = [&](uint32_t blk_raw, BlockX& k) __attribute__((always_inline)) {
+        const uint32_t blk = min(blk_raw, b1 - 1u);
 #pragma unroll
         for (int t = 0; t < NBT; ++t)
 #pragma unroll
@@ -420,7 +431,7 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
                 k.ex[t] = *reinterpret_cast<const uint4*>(a.blk_exp + ((size_t)t * a.nblocks + blk) * 32 + (lane / 32) * 16);
         }
     };
-    auto multiply = [&](const Block& k) __attribute__((always_inline)) {
+    auto multiply = [&](const BlockW& k, const BlockX& kx) __attribute__((always_inline)) {
         if constexpr (IOP) {
 #pragma unroll
             for (int r = 0; r < RT; ++r) {
@@ -444,13 +455,13 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
                     for (int i = 0; i < 16; ++i) sblk[i] = 0.f;
 #pragma unroll
                     for (int ks = 0; ks < 2; ++ks) {
-                        sblk = __builtin_amdgcn_mfma_f32_32x32x16_f16(k.x[t][ks][0], w[ks], sblk, 0, 0, 0);
-                        sblk = __builtin_amdgcn_mfma_f32_32x32x16_f16(k.x[t][ks][1], w[ks], sblk, 0, 0, 0);
+                        sblk = __builtin_amdgcn_mfma_f32_32x32x16_f16(kx.x[t][ks][0], w[ks], sblk, 0, 0, 0);
+                        sblk = __builtin_amdgcn_mfma_f32_32x32x16_f16(kx.x[t][ks][1], w[ks], sblk, 0, 0, 0);
                     }
                     if constexpr (BS) {
 #pragma unroll
                         for (int j = 0; j < 4; ++j) {
-                            const uint32_t e4 = j == 0 ? k.ex[t].x : j == 1 ? k.ex[t].y : j == 2 ? k.ex[t].z : k.ex[t].w;
+                            const uint32_t e4 = j == 0 ? kx.ex[t].x : j == 1 ? kx.ex[t].y : j == 2 ? kx.ex[t].z : kx.ex[t].w;
 #pragma unroll
                             for (int e = 0; e < 4; ++e) {
                                 const int ex = (int)(e4 << (24 - 8 * e)) >> 24;   // signed byte e
@@ -489,9 +500,9 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
                 }
 #pragma unroll
                 for (int t = 0; t < NBT; ++t) {
-                    acc[r][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi, k.x[t][ks][0], acc[r][t], 0, 0, 0);
-                    acc[r][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi, k.x[t][ks][1], acc[r][t], 0, 0, 0);
-                    acc[r][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wlo, k.x[t][ks][0], acc[r][t], 0, 0, 0);
+                    acc[r][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi, kx.x[t][ks][0], acc[r][t], 0, 0, 0);
+                    acc[r][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi, kx.x[t][ks][1], acc[r][t], 0, 0, 0);
+                    acc[r][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wlo, kx.x[t][ks][0], acc[r][t], 0, 0, 0);
                 }
             }
         }
@@ -524,10 +535,16 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
             asm volatile("" ::: "memory");
         }
     }
-    Block k[PF];
+    BlockW k[PFW];
+    BlockX kx[PF];
+#pragma unroll
+    for (int i = 0; i < PFW; ++i) {
+        load_w(b0 + wave + i * WAVES, k[i]);
+        asm volatile("" ::: "memory");
+    }
 #pragma unroll
     for (int i = 0; i < PF; ++i) {
-        load(b0 + wave + i * WAVES, k[i]);
+        load_x(b0 + wave + i * WAVES, kx[i]);
         asm volatile("" ::: "memory");
     }
     if constexpr (BS) {
@@ -541,11 +558,12 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
             asm volatile("" ::: "memory");
         }
     }
-    for (uint32_t base = b0 + wave; base < b1; base += PF * WAVES) {
+    for (uint32_t base = b0 + wave; base < b1; base += PFW * WAVES) {
 #pragma unroll
-        for (int i = 0; i < PF; ++i) {
-            multiply(k[i]);
-            load(base + (i + PF) * WAVES, k[i]);
+        for (int i = 0; i < PFW; ++i) {
+            multiply(k[i], kx[i % PF]);
+            load_w(base + (i + PFW) * WAVES, k[i]);
+            load_x(base + (i + PF) * WAVES, kx[i % PF]);
             asm volatile("" ::: "memory");
         }
     }
