@@ -177,7 +177,7 @@ struct Ctx {
     struct GemmPending {
         bool active = false;
         Q4Args a{};
-        unsigned grid_x = 0;
+        unsigned grid_x = 0, grid_z = 1;
         int nbt = 1, rt = 1;
         const void* out = nullptr;
         size_t batch = 0, rows = 0;
@@ -462,7 +462,7 @@ int settle_gemm(const RopeArgs* rope = nullptr) {
         a.rope = *rope;
         ++g.gemm_rope_fused;
     }
-    const dim3 grid(m.grid_x, 1);
+    const dim3 grid(m.grid_x, 1, m.grid_z);
     if (m.silu) {
         m.silu = false;
         ++g.gemm_silu_fused;

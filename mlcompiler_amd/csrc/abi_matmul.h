@@ -197,6 +197,10 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
         a.blocks_per_slice = (uint32_t)per_slice; a.ksplit = (uint32_t)ksplit;
         a.rope_on = 0;
         a.rope = RopeArgs{};
+        // one batch tile of more than 16 requests on a grid that fills at most half of the CUs: two
+        // workgroups per (row tile, K slice), each with half of the tile's requests
+        const unsigned bsplit = (bpad == 32 && bn > 16 && wgs * ksplit <= (size_t)g.n_cu / 2) ? 2u : 1u;
+        a.bsplit = bsplit;
         if (g.opt_fuse_rows && !sync && ksplit == 1 && batch <= 64) {
             // held back for one call: a split + RoPE + cast of this output becomes the epilogue
             Ctx::GemmPending& m = g.gemm;
@@ -205,6 +209,7 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
             m.block_scales = block_scales;
             m.a = a;
             m.grid_x = (unsigned)wgs;
+            m.grid_z = bsplit;
             m.nbt = bpad == 32 ? 1 : 2;
             m.rt = row_tiles;
             m.out = out;
@@ -212,7 +217,7 @@ int mlc_hip_matmul_q4_0_batched(const char* weight_name, const void* weights, si
             m.rows = rows;
             return finish(sync);
         }
-        const dim3 grid((unsigned)wgs, (unsigned)ksplit);
+        const dim3 grid((unsigned)wgs, (unsigned)ksplit, bsplit);
         if (block_scales)
             launch_q4_mfma_block_scales(bpad == 32 ? 1 : 2, row_tiles, grid, a);
         else

@@ -124,7 +124,7 @@ int mlc_hip_gate_up_split_silu_mul(const void* gate_up, void* gate, void* up, vo
         // (workgroup j takes row tile j of the gate half and row tile j of the up half).
         Ctx::GemmPending& m = g.gemm;
         if (g.opt_fuse_rows && g.opt_q4_int_operand && !sync && m.active && !m.silu && !g.rows.active && !g.kv.active &&
-            m.rt == 2 && !(m.block_scales && m.nbt != 1) && m.out == gate_up && m.batch == batch && m.rows == ffn_gate_up_rows &&
+            m.rt == 2 && m.grid_z == 1 && !(m.block_scales && m.nbt != 1) && m.out == gate_up && m.batch == batch && m.rows == ffn_gate_up_rows &&
             ffn_gate_up_rows == 2 * ffn_inner && ffn_inner % 32 == 0 && aligned16(gate) && aligned16(up) && aligned16(out)) {
             m.silu = true;
             m.silu_out = out;

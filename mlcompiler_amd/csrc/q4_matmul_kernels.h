@@ -149,6 +149,14 @@ struct Q4Args {
     const float* inv_scale;     // [batch]
     float* out;                 // [batch][rows], or the slice buffer [ksplit][batch][rows]
     uint32_t batch, rows, nblocks, blocks_per_slice, ksplit;
+    // 2 (one batch tile, kernels without the SiLU epilogue): the grid's z dimension halves the
+    // batch; workgroup z takes requests 16 z .. 16 z + 15 of the tile and fetches only their
+    // activation fragments (the other 16 lanes of a half wave repeat those addresses and their
+    // results are dropped).  The fragments are the largest stream of a workgroup that has all of
+    // K, 4 bytes per request and column through one CU's memory path; this halves it where the
+    // grid would otherwise leave half of the CUs idle anyway (quarters of the batch on four
+    // workgroups were measured as well and gain nothing more).  0 or 1: the whole tile.
+    uint32_t bsplit;
     // When rope_on is set (ksplit == 1, out is a fused qkv row of rope.qkv_rows = rows floats per
     // request): the epilogue also does what qkv_split_rope_cast_kernel would do with that row.
     uint32_t rope_on;
@@ -344,6 +352,8 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
     const uint32_t tile0 = SILU ? blockIdx.x : blockIdx.x * RT;
     const uint32_t tile_step = SILU ? a.tile_stride : 1u;   // row tile r of the workgroup: tile0 + r * tile_step
     const uint32_t slice = blockIdx.y;
+    const uint32_t bz = blockIdx.z;   // (batch half, with bsplit == 2)
+    const uint32_t lane_x = (a.bsplit < 2 || (lane % 32) / 16 == bz) ? lane : (lane ^ 16u);
     const uint32_t b0 = slice * a.blocks_per_slice;
     const uint32_t b1 = min(b0 + a.blocks_per_slice, a.nblocks);
     const uint32_t ksteps = a.nblocks * 2;
@@ -423,7 +433,7 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
 #pragma unroll
                 for (int p = 0; p < 2; ++p)
                     k.x[t][ks][p] = *reinterpret_cast<const q4_half8*>(
-                        a.xfrag + ((((size_t)t * ksteps + blk * 2 + ks) * 2 + p) * 64 + lane) * 8);
+                        a.xfrag + ((((size_t)t * ksteps + blk * 2 + ks) * 2 + p) * 64 + lane_x) * 8);
         if constexpr (BS) {
             // register i of the accumulator is batch column (i/4)*8 + (lane/32)*4 + i%4
 #pragma unroll
@@ -642,6 +652,7 @@ __global__ __launch_bounds__(WAVES * 64) void q4_0_matmul_mfma_kernel(const Q4Ar
         const uint32_t b = pass * COLS_PER_PASS + bsub;
         const bool fused_add = IOP && RT == 1 && a.add_resid;   // (uniform; then a half wave is one request's 32 columns)
         if (b >= a.batch && !fused_add) continue;
+        if (a.bsplit == 2 && (b % 32) / 16 != bz) continue;   // the other half's workgroup has these requests
         const bool live = b < a.batch;
         const uint32_t t = b / 32;
         const uint32_t in_reg = IOP ? b % 32 : rr, in_lane = IOP ? rr : b % 32;

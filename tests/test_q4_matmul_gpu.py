@@ -73,6 +73,9 @@ MFMA_SHAPES = [  # rows, cols, batch: TinyLlama qkv / out-proj / gate_up / down,
     (2560, 2048, 32), (2048, 2048, 64), (11264, 2048, 64), (2048, 5632, 64),
     (64, 64, 1), (128, 96, 33), (256, 2048, 7), (192, 160, 100),
     (6144, 4096, 5), (4096, 14336, 3), (28672, 4096, 2),    # Llama-3-8B qkv / down / gate_up
+    # one batch tile of more than 16 requests on a small grid: two workgroups per row tile, half of the
+    # requests each (with K split over workgroups as well; the odd batches leave one half ragged)
+    (512, 4096, 20), (1024, 512, 17), (3200, 256, 31), (4096, 2048, 32),
 ]
 
 
