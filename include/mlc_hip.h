@@ -394,7 +394,12 @@ long mlc_hip_decode_table_uploads(void);
  *                           call has sync = 1; every output buffer is still written.  The
  *                           same holds for the KV write: split + RoPE + cast and the two
  *                           batched scatters of its fp16 rows (or two batched scatters with
- *                           the same page ids) become one launch.
+ *                           the same page ids) become one launch.  A Q4_0 matmul and a decode
+ *                           attention call may be held back for a call or two as well, and
+ *                           take on the work of the operators encoded right behind them
+ *                           (split + RoPE + cast + KV write; gate/up split + SiLU * up; residual
+ *                           add + RMSNorm; the fp16 split of the matmul that reads their output):
+ *                           see the mlc_hip_fused_* counters above.
  *                           0 = each operator is launched when it is encoded
  *   "decode_pair_cost"      0..64: the tile-balanced decode kernel gives every workgroup the same
  *                           number of units, a KV tile counting one and the end of a (request,

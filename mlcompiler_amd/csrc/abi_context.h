@@ -173,7 +173,9 @@ struct Ctx {
     // When that call is the gate/up split + SiLU * up of the matmul's output (the gate/up
     // projection), the epilogue does that instead and the matmul is held back for one call more:
     // a Q4_0 matmul that reads the products (the down-projection) lets the epilogue also write
-    // its activation fragments.
+    // its activation fragments.  And while a residual add and an RMSNorm of the matmul's output
+    // build their chain (RowPending) the matmul stays held back, too: a Q4_0 matmul that reads the
+    // norm takes the chain's work over together with this one (mlc_hip_matmul_q4_0_batched).
     struct GemmPending {
         bool active = false;
         Q4Args a{};

@@ -194,7 +194,7 @@ struct Q4Args {
     float* ssq_out;
     // ssq_in set (BS kernels): the activations are h * gamma of an RMSNorm whose per-request factor
     // 1 / sqrt(mean(h^2) + eps) is still missing: it is computed here from the ssq_tiles partial
-    // sums of squares per request (ssq_in[tile][64], summed in tile order) and multiplied into the
+    // sums of squares per request (ssq_in[tile][64], summed in a fixed order) and multiplied into the
     // result, and the workgroups also write the RMSNorm's own output rms_out = h * factor * gamma
     // ([batch][rms_len], h = rms_src), 1024 elements per workgroup of the grid.
     const float* ssq_in;
