@@ -1,4 +1,5 @@
-"""Random sequences of the row-local operators (add, RMSNorm, gate/up SiLU, Q4_0 matmul) and of
+"""Random sequences of the row-local operators (add, RMSNorm, gate/up SiLU, Q4_0 matmul), of the
+paged decode attention (whose launch may be held back for the matmul behind it) and of
 the KV write (split + RoPE + cast, with the batched scatters or fused with them) with
 shared and in-place buffers, encoded in one pass twice: with the fused chains (the default) and
 with every operator launched on its own.  Deferring and fusing must never change what a
@@ -16,13 +17,27 @@ B, L = 5, 256
 # a [B][2L] buffer read as a fused qkv row: 4 query heads and 2 KV heads of 64
 H, HKV, D, P, CAP = 4, 2, 64, 8, 12
 KV_ROWS = HKV * D
+# the attention op: an [B][L] buffer as q of 4 heads over one KV head, pools of its own with 64-token pages
+A_HKV, A_P = 1, 64
 
 
 def _program(rng, n_ops):
     """ops over buffers: 'n' = [B][L] (indices 0..5), 'w' = [B][2L] (indices 0..1)"""
     ops = []
     for _ in range(n_ops):
-        kind = rng.choice(["add", "add", "rms", "rms", "mm_n", "mm_w", "mm_w", "silu", "peek", "rope", "ropec"])
+        kind = rng.choice(["add", "add", "rms", "rms", "mm_n", "mm_n", "mm_w", "mm_w", "silu", "peek", "rope", "ropec",
+                           "attn", "attn", "layer_like", "layer_like"])
+        if kind == "layer_like":
+            # the order of a decoder layer's middle, buffers drawn at random (they may alias where the
+            # operators allow it): attention -> matmul -> + residual -> norm -> matmul, any prefix of it cut off
+            q, o, proj, res, h, xn = (int(v) for v in rng.permutation(6))
+            if rng.random() < 0.3:
+                h = res                                          # the sum written over the residual
+            seq = [("attn", q, o), ("mm_n", o, proj), ("add", proj, res, h) if rng.random() < 0.5 else ("add", res, proj, h),
+                   ("rms", h, xn, int(rng.integers(0, 2))), ("mm_w", xn, int(rng.integers(0, 2)))]
+            first = int(rng.integers(0, 2))                      # with or without the attention in front
+            ops.extend(seq[first:int(rng.integers(first + 2, len(seq) + 1))])
+            continue
         if kind == "add":
             a, b, c = (int(v) for v in rng.integers(0, 6, 3))
             ops.append(("add", a, b, c))                       # c may alias a or b
@@ -35,6 +50,9 @@ def _program(rng, n_ops):
             ops.append(("mm_n", a, c))
         elif kind == "mm_w":
             ops.append(("mm_w", int(rng.integers(0, 6)), int(rng.integers(0, 2))))
+        elif kind == "attn":
+            a = int(rng.integers(0, 6))
+            ops.append(("attn", a, int(rng.choice([i for i in range(6) if i != a]))))
         elif kind == "silu":
             g, u, m = (int(v) for v in rng.choice(6, 3, replace=False))
             ops.append(("silu", int(rng.integers(0, 2)), g, u, m))
@@ -73,6 +91,10 @@ def _run(exe, ops, init_n, init_w, weights, gammas, fuse, ksplit, kv):
                                                    w[op[2]]), exe.lastError()
             elif op[0] == "silu":
                 assert exe.encodeGateUpSplitSiluMul(w[op[1]], n[op[2]], n[op[3]], n[op[4]], B, L, 2 * L)
+            elif op[0] == "attn":
+                at = kv["attn"]
+                assert exe.encodePagedFlashAttention(n[op[1]], kvb["a_k"], kvb["a_v"], n[op[2]], at["flat"], at["off"],
+                                                     at["lens"], at["pos"], B, H, A_HKV, D, A_P, True), exe.lastError()
             elif op[0] == "rope":
                 assert exe.encodeQkvSplitRopeScatter(w[op[1]], n[op[2]], kvb["kp"], kvb["vp"], kvb["cos"], kvb["sin"],
                                                      kv["ids"], kv["slots"], P, B, H, HKV, D, 2 * L, L, KV_ROWS,
@@ -125,13 +147,24 @@ def test_fused_and_unfused_sequences_agree(exe, seed):
           "init": {"cos": cos, "sin": sin, "k": np.zeros((B, KV_ROWS), np.float32), "v": np.zeros((B, KV_ROWS), np.float32),
                    "k16": np.zeros((B, KV_ROWS), np.uint16), "v16": np.zeros((B, KV_ROWS), np.uint16),
                    "kp": np.zeros(CAP * P * KV_ROWS, np.uint16), "vp": np.zeros(CAP * P * KV_ROWS, np.uint16)}}
+    a_lens = rng.integers(0, 200, B).astype(np.uint32)          # (a request without tokens now and then: a row of zeros)
+    a_pages = (a_lens.astype(np.int64) + A_P - 1) // A_P
+    a_off = np.zeros(B + 1, np.uint32)
+    a_off[1:] = np.cumsum(a_pages)
+    n_pages = max(int(a_pages.sum()), 1)
+    kv["attn"] = {"lens": a_lens, "pos": np.where(a_lens > 0, a_lens - 1, 0).astype(np.uint32), "off": a_off,
+                  "flat": rng.permutation(n_pages)[:int(a_pages.sum())].astype(np.uint32)}
+    for name in ("a_k", "a_v"):
+        kv["init"][name] = rng.standard_normal(n_pages * A_P * A_HKV * D).astype(np.float16).view(np.uint16)
     before = exe.rowProgramLaunches()
     before_mm = exe.fusedMatmulRopeLaunches()
+    before_more = exe.fusedDecodeSplitLaunches(), exe.fusedMatmulNormLaunches()
     fused, fused_peeks = _run(exe, ops, init_n, init_w, weights, gammas, 1, ksplit, kv)
     n_fused = exe.rowProgramLaunches() - before
     print(f"[fuzz {seed}] fused chains {n_fused}, matmuls with the RoPE epilogue "
-          f"{exe.fusedMatmulRopeLaunches() - before_mm}", flush=True)
-    assert n_fused > 0 or not any(o[0] in ("add", "rms", "silu") for o in ops)
+          f"{exe.fusedMatmulRopeLaunches() - before_mm}, attention launches that split their output "
+          f"{exe.fusedDecodeSplitLaunches() - before_more[0]}, matmuls that took over add + norm "
+          f"{exe.fusedMatmulNormLaunches() - before_more[1]}", flush=True)
     plain, plain_peeks = _run(exe, ops, init_n, init_w, weights, gammas, 0, ksplit, kv)
     assert exe.rowProgramLaunches() - before == n_fused       # none with fusion off
     n_final = len(fused)
